@@ -1,0 +1,277 @@
+"""Host-side mirror of the reference's cache operator and cache object.
+
+``sink_cache`` keeps the positional signature of the reference operator
+(cascade/models/cascading_cache.py:962-987) and forwards to ``ckv_update`` in ``libckv.so``;
+``CascadingKVCache`` keeps the constructor, attributes and methods of the reference class
+(cascade/models/cascading_cache.py:1031-1348) without depending on ``transformers``.
+There is no CPU path: tensors must live on a HIP device and the library must be built.
+"""
+import ctypes as C
+from typing import List, Optional, Union
+
+import torch
+from torch import Tensor
+
+from . import _abi
+
+_WORKSPACES = {}
+
+
+def workspace(device: torch.device, nbytes: int) -> Tensor:
+    """A per-device scratch buffer, grown on demand and reused by stream-ordered calls."""
+    key = (device.type, device.index)
+    buf = _WORKSPACES.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = buf
+    return buf
+
+
+def _require_device(t: Tensor, what: str):
+    if t.device.type != "cuda":
+        raise _abi.CkvError(f"{what} lives on {t.device}: libckv only runs on a HIP device (no CPU fallback)")
+
+
+def sink_cache(
+    k: Tensor, v: Tensor, s: Tensor,
+    sink_k: Tensor, sink_v: Tensor, sink_mask: Tensor, sink_pos: Tensor,
+    cache_k: Tensor, cache_v: Tensor, cache_s: Tensor,
+    mask: Tensor, pos: Tensor, og_pos: Tensor,
+    do_cache: Tensor, do_cache_every_n: Tensor,
+    stored_tokens: Tensor, start_indices: Tensor, stored_sinks: Tensor,
+    num_sink, window_size, real_token_idx, max_seq_len, eager_fill,
+    BENCHMARK: bool = False,
+):
+    """Drop-in for ``sink_cache`` (cascading_cache.py:962-1028): mutates the 13 state tensors in
+    place and returns ``(k, v)``.  ``do_cache`` is accepted and ignored, as in the reference
+    kernel (cascading_cache.py:204, 281, 361)."""
+    _require_device(k, "k")
+    lib = _abi.lib()
+    if BENCHMARK:
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+    a = _abi.fill_update_args(k, v, s, sink_k, sink_v, sink_mask, sink_pos, cache_k, cache_v, cache_s, mask, pos,
+                              og_pos, do_cache_every_n, stored_tokens, start_indices, stored_sinks, num_sink,
+                              window_size, real_token_idx, max_seq_len, eager_fill)
+    need = lib.ckv_update_workspace_bytes(a.N, a.H, a.K, a.max_seq_len, a.cascades)
+    ws = workspace(k.device, need)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    with torch.cuda.device(k.device):
+        stream = torch.cuda.current_stream(k.device).cuda_stream
+        _abi.check(lib.ckv_update(C.byref(a), C.c_void_p(stream)), "ckv_update")
+    if BENCHMARK:
+        ev1.record()
+        torch.cuda.synchronize()
+        print(ev0.elapsed_time(ev1))
+    return k, v
+
+
+def acceptance_periods(cascade_func: str, cascades: int) -> List[int]:
+    """The nine named acceptance schedules of cascading_cache.py:1201-1244."""
+    c = cascades
+    if cascade_func == "pow2":
+        return [2 ** i for i in range(c)]
+    if cascade_func == "pow2-1":
+        return [1] * (c - 1) + [2 ** (c - 1)] if c > 0 else []
+    if cascade_func in ("pow2-1-4", "pow2-2-4", "pow2-3-4"):
+        ones = {"pow2-1-4": 3, "pow2-2-4": 2, "pow2-3-4": 1}[cascade_func] * (c // 4)
+        return [1] * ones + [2 ** i for i in range(ones, c)]
+    if cascade_func == "1-then-2":
+        return [1] + [2] * (c - 1)
+    if cascade_func == "pow3":
+        return [3 ** i for i in range(c)]
+    if cascade_func == "pow4":
+        return [4 ** i for i in range(c)]
+    if cascade_func == "iplus1":
+        return [i + 1 for i in range(c)]
+    raise ValueError(f"unknown cascade func: {cascade_func}")
+
+
+class CascadingKVCache:
+    """Per-layer sink + cascade state with the interface of the reference class
+    (cascading_cache.py:1031-1348).  Tensors have the reference's shapes and dtypes
+    (cascading_cache.py:1196-1276) so code that reads them keeps working."""
+
+    def __init__(
+        self,
+        window_length: Union[int, List[int]] = 8,
+        num_sink_tokens: int = 4,
+        max_batch_size: int = 1,
+        heads: int = 16,
+        dim: int = 128,
+        max_seq_len: Union[int, List[int]] = 32,
+        device: torch.device = "cpu",
+        dtype: torch.dtype = torch.float16,
+        cascade_func: str = "pow2",
+        head_reduction: str = "mean",
+        layers: int = 32,
+        eager_fill: bool = True,
+        verbose: bool = True,
+    ) -> None:
+        if isinstance(max_seq_len, int) != isinstance(window_length, int):
+            raise ValueError(
+                f"max_seq_len must be same type as window length: {type(max_seq_len)=} {type(window_length)=}")
+        if isinstance(max_seq_len, int):
+            max_seq_len = [max_seq_len for _ in range(layers)]
+        if isinstance(window_length, int):
+            window_length = [window_length for _ in range(layers)]
+
+        self.verbose = verbose
+        self.max_seq_len = max_seq_len
+        self.max_batch_size = max_batch_size
+        self.heads = heads
+        self.dim = dim
+        self.device = device
+        self.dtype = dtype
+        self.window_length = window_length
+        self.num_sink_tokens = num_sink_tokens
+        self.cascade_func = cascade_func
+        self.head_reduction = head_reduction
+        self.layers = layers
+        self.eager_fill = eager_fill
+        self.bh = self.max_batch_size * self.heads
+
+        if not all((self.max_seq_len[l] % self.window_length[l]) == 0 for l in range(layers)):
+            raise ValueError(
+                f"window length must evenly divide max seq len: {self.window_length=} {self.max_seq_len=}")
+        self.cascades = [self.max_seq_len[l] // self.window_length[l] for l in range(layers)]
+        self._seen_tokens = 0
+        self.init_cache(self.device)
+
+    def __repr__(self):
+        return f"{self.max_seq_len=}, {self.cascades=} {self.max_batch_size=}, {self.layers=} {self.heads=}"
+
+    def __getitem__(self, layer_idx: int):
+        return self.get_vals(layer_idx)
+
+    def __iter__(self):
+        for layer_idx in range(len(self)):
+            yield self.get_vals(layer_idx)
+
+    def __len__(self):
+        return self.layers
+
+    # the HF cache methods the reference leaves unimplemented (cascading_cache.py:1126-1162)
+    def to_legacy_cache(self):
+        raise NotImplementedError()
+
+    @classmethod
+    def from_legacy_cache(cls, past_key_values=None):
+        raise NotImplementedError()
+
+    def crop(self, max_length: int):
+        raise NotImplementedError()
+
+    def batch_split(self, full_batch_size: int, split_size: int):
+        raise NotImplementedError()
+
+    @classmethod
+    def from_batch_splits(cls, splits):
+        raise NotImplementedError()
+
+    def batch_repeat_interleave(self, repeats: int):
+        raise NotImplementedError()
+
+    def batch_select_indices(self, indices: torch.Tensor):
+        raise NotImplementedError()
+
+    def reorder_cache(self, beam_idx: torch.LongTensor):
+        raise NotImplementedError()
+
+    @property
+    def seen_tokens(self):
+        raise NotImplementedError()
+
+    def get_seq_length(self, layer_idx: Optional[int] = 0, cascade_idx: Optional[int] = -1) -> int:
+        stored_sinks = self.stored_sinks[layer_idx][0, 0].item()
+        stored_tokens = self.stored_tokens[layer_idx][0, 0].sum().item()
+        return stored_sinks + stored_tokens
+
+    def get_max_length(self) -> Optional[int]:
+        return self.max_seq_len[0]
+
+    def reset(self, verbose=True):
+        if verbose:
+            print(f"RESET HIP CACHE {self.cascade_func=}")
+        self._seen_tokens = 0
+        self._seen_host = [0 for _ in range(self.layers)]
+        self.seen_tokens_by_layer.zero_()
+        for group in (self.stored_tokens, self.stored_sinks, self.start_indices, self.pos, self.sink_pos,
+                      self.key_cache, self.value_cache, self.score_cache, self.sink_keys, self.sink_values,
+                      self.og_pos):
+            for t in group:
+                t.zero_()
+        for group in (self.do_cache, self.mask, self.sink_mask):
+            for t in group:
+                t.fill_(True)
+
+    def init_cache(self, device):
+        L, B, H, D = self.layers, self.max_batch_size, self.heads, self.dim
+        nsink, dev, dtp = self.num_sink_tokens, device, self.dtype
+        if self.verbose:
+            print(f"INIT CLEAN HIP CACHE {self.cascade_func=}")
+        self._seen_tokens = 0
+        # host mirror of seen_tokens_by_layer: lets callers branch without a device sync
+        self._seen_host = [0 for _ in range(L)]
+        self.seen_tokens_by_layer = torch.zeros(L, dtype=torch.long, device=dev)
+        self.do_cache = [torch.ones(self.cascades[l], device=dev, dtype=torch.bool) for l in range(L)]
+        self.do_cache_every_n = [
+            torch.tensor(acceptance_periods(self.cascade_func, self.cascades[l]), device=dev, dtype=torch.long)
+            for l in range(L)]
+        self.beta = 0.9999999  # cascading_cache.py:1247
+
+        self.stored_tokens = [torch.zeros(B, H, self.cascades[l], device=dev, dtype=torch.long) for l in range(L)]
+        self.stored_sinks = [torch.zeros(B, H, device=dev, dtype=torch.long) for _ in range(L)]
+        self.start_indices = [torch.zeros(B, H, self.cascades[l], device=dev, dtype=torch.long) for l in range(L)]
+        self.pos = [torch.zeros(B, H, self.max_seq_len[l], device=dev, dtype=torch.long) for l in range(L)]
+        self.og_pos = [torch.zeros(B, H, self.max_seq_len[l], device=dev, dtype=torch.long) for l in range(L)]
+        self.sink_pos = [torch.zeros(B, H, nsink, device=dev, dtype=torch.long) for _ in range(L)]
+        self.key_cache = [torch.zeros(B, H, self.max_seq_len[l], D, device=dev, dtype=dtp) for l in range(L)]
+        self.value_cache = [torch.zeros(B, H, self.max_seq_len[l], D, device=dev, dtype=dtp) for l in range(L)]
+        self.score_cache = [torch.zeros(B, H, self.max_seq_len[l], device=dev, dtype=dtp) for l in range(L)]
+        self.sink_keys = [torch.zeros(B, H, nsink, D, device=dev, dtype=dtp) for _ in range(L)]
+        self.sink_values = [torch.zeros(B, H, nsink, D, device=dev, dtype=dtp) for _ in range(L)]
+        self.mask = [torch.ones(B, H, self.max_seq_len[l], device=dev, dtype=torch.bool) for l in range(L)]
+        self.sink_mask = [torch.ones(B, H, nsink, device=dev, dtype=torch.bool) for _ in range(L)]
+
+    def pos_shift(self, layer_idx: int) -> int:
+        """The sink shift of get_vals (cascading_cache.py:1282-1283), from the host counter."""
+        return self.num_sink_tokens if self._seen_host[layer_idx] > self.num_sink_tokens else 0
+
+    def get_vals(self, layer_idx: int):
+        pos_shift = self.pos_shift(layer_idx)
+        return (
+            self.sink_keys[layer_idx],
+            self.sink_values[layer_idx],
+            self.sink_pos[layer_idx][:1, 0],
+            self.sink_mask[layer_idx],
+            self.key_cache[layer_idx],
+            self.value_cache[layer_idx],
+            self.pos[layer_idx][:1, 0] + pos_shift,
+            self.mask[layer_idx],
+            self.og_pos[layer_idx],
+        )
+
+    def update(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None):
+        """cascading_cache.py:1297-1348."""
+        if score_states is None:
+            score_states = torch.zeros(self.max_batch_size, self.heads, key_states.size(2),
+                                       device=key_states.device, dtype=key_states.dtype)
+        if layer_idx == 0:
+            self._seen_tokens += key_states.shape[-2]
+
+        sink_cache(
+            key_states, value_states, score_states,
+            self.sink_keys[layer_idx], self.sink_values[layer_idx],
+            self.sink_mask[layer_idx], self.sink_pos[layer_idx],
+            self.key_cache[layer_idx], self.value_cache[layer_idx], self.score_cache[layer_idx],
+            self.mask[layer_idx], self.pos[layer_idx], self.og_pos[layer_idx],
+            self.do_cache[layer_idx], self.do_cache_every_n[layer_idx],
+            self.stored_tokens[layer_idx], self.start_indices[layer_idx], self.stored_sinks[layer_idx],
+            self.num_sink_tokens, self.window_length[layer_idx],
+            self.seen_tokens_by_layer[layer_idx], self.max_seq_len[layer_idx], self.eager_fill,
+        )
+        # after the kernel, as in the reference (cascading_cache.py:1343-1346)
+        self.seen_tokens_by_layer[layer_idx] += key_states.shape[-2]
+        self._seen_host[layer_idx] += key_states.shape[-2]
+        return self.get_vals(layer_idx)

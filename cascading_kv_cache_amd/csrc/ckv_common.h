@@ -1,0 +1,67 @@
+// Shared device/host helpers for libckv (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/ckv.h"
+
+#define CKV_WAVE 64
+
+#define CKV_HIP_TRY(expr)                          \
+    do {                                           \
+        hipError_t err__ = (expr);                 \
+        if (err__ != hipSuccess) {                 \
+            (void)hipGetLastError();               \
+            return CKV_ERR_LAUNCH;                 \
+        }                                          \
+    } while (0)
+
+namespace ckv {
+
+__host__ __device__ inline int64_t elem_bytes(int dtype) { return dtype == CKV_F32 ? 4 : 2; }
+
+// exact widening of one stored score to fp32
+__device__ inline float load_as_float(const void* base, int64_t idx, int dtype) {
+    if (dtype == CKV_F32) return reinterpret_cast<const float*>(base)[idx];
+    const uint16_t h = reinterpret_cast<const uint16_t*>(base)[idx];
+    if (dtype == CKV_BF16) return __uint_as_float(static_cast<uint32_t>(h) << 16);
+    return __half2float(__ushort_as_half(h));
+}
+
+__device__ inline float bf16_bits_to_float(uint16_t h) { return __uint_as_float(static_cast<uint32_t>(h) << 16); }
+
+// round-to-nearest-even fp32 -> bf16 bits (NaN kept quiet)
+__device__ inline uint16_t float_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return static_cast<uint16_t>(u >> 16);
+}
+
+template <typename T>
+struct Elem;
+template <>
+struct Elem<float> {
+    static constexpr int code = CKV_F32;
+    __device__ static float to_float(float v) { return v; }
+    __device__ static float from_float(float v) { return v; }
+};
+template <>
+struct Elem<__hip_bfloat16> {
+    static constexpr int code = CKV_BF16;
+    __device__ static float to_float(__hip_bfloat16 v) { return __bfloat162float(v); }
+    __device__ static __hip_bfloat16 from_float(float v) { return __float2bfloat16(v); }
+};
+template <>
+struct Elem<__half> {
+    static constexpr int code = CKV_F16;
+    __device__ static float to_float(__half v) { return __half2float(v); }
+    __device__ static __half from_float(float v) { return __float2half(v); }
+};
+
+inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace ckv

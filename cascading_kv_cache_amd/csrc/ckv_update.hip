@@ -1,0 +1,556 @@
+// ckv_update: the cascading cache update as a plan + apply pair of gfx950 kernels.
+//
+// Replaces the serial per-token Triton program of the reference
+// (cascade/models/cascading_cache.py:145-299 token loop, 302-774 body) with
+//
+//   plan   one workgroup per (batch, kv-head).  Walks the cascades in order; at every cascade
+//          the arrivals of the whole call are classified (insert / challenger), numbered with a
+//          ballot prefix sum, the challengers of each group are reduced to the group's winner
+//          ("later wins iff score >=", cascading_cache.py:699), and the tokens the cascade evicts
+//          become the arrival list of the next cascade.  Everything lives in LDS.  The result is
+//          a forest of disjoint move chains in global memory:
+//              first[t]   = slot the incoming token t finally lands in (-1: dropped)
+//              next_of[d] = slot the OLD content of slot d finally lands in (-1: dropped)
+//          plus the trackers, and the position ids in closed form (cascading_cache.py:112-142,
+//          728-774).
+//   apply  one lane group per incoming token.  Follows the chain of its token from the head,
+//          carrying a whole row (K, V, score, original index) in registers with 16-byte lanes:
+//          read the displaced row, write the carried one, move on.  Chains are vertex-disjoint
+//          and only ever move towards higher cascades, so groups never touch each other's slots.
+//
+// Why this equals the serial loop: within one cascade the n-th insert of a call always lands in
+// ring position (start + stored + n) mod W whatever the scores are; only WHICH arrival owns a
+// slot depends on scores, and that is decided inside the group of arrivals between two inserts.
+#include "ckv_common.h"
+
+namespace ckv {
+namespace {
+
+constexpr int kMaxCascades = 64;
+
+struct UpdateParams {
+    ckv_update_args a;
+    int64_t token_offset;  // first incoming token handled by this launch
+    int32_t k_sub;         // tokens handled by this launch
+    int32_t do_pos;        // run the position pass (last launch of a call only)
+    int32_t* first;        // [N*H][K]
+    int32_t* next_of;      // [N*H][S]
+};
+
+// exclusive prefix sum of one flag per thread over the whole workgroup; returns the block total
+__device__ inline int block_flag_scan(bool flag, int* wave_tot, int& exclusive) {
+    const unsigned long long bal = __ballot(flag);
+    const int lane = threadIdx.x & (CKV_WAVE - 1);
+    const int wave = threadIdx.x / CKV_WAVE;
+    const int nwaves = (blockDim.x + CKV_WAVE - 1) / CKV_WAVE;
+    const int in_wave = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_tot[wave] = __popcll(bal);
+    __syncthreads();
+    int before = 0, total = 0;
+    for (int w = 0; w < nwaves; w++) {
+        const int c = wave_tot[w];
+        if (w < wave) before += c;
+        total += c;
+    }
+    __syncthreads();  // wave_tot is reused by the next call
+    exclusive = before + in_wave;
+    return total;
+}
+
+__device__ inline void emit_move(int32_t* first, int32_t* next_of, int dst, int src) {
+    next_of[dst] = -1;
+    if (src < 0) {
+        first[-1 - src] = dst;
+    } else {
+        next_of[src] = dst;
+    }
+}
+
+__global__ void ckv_update_plan_kernel(UpdateParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const ckv_update_args& A = p.a;
+    const int tid = threadIdx.x, T = blockDim.x;
+    const int64_t bh = blockIdx.x;
+    const int64_t n = bh / A.H, h = bh % A.H;
+    const int cap = p.k_sub;
+    const int C = A.cascades;
+    const int64_t W = A.window_size, S = A.max_seq_len, NS = A.num_sink;
+
+    int32_t* a_src[2];
+    int32_t* a_trig[2];
+    float* a_score[2];
+    unsigned char* ptr = smem;
+    for (int i = 0; i < 2; i++) {
+        a_src[i] = reinterpret_cast<int32_t*>(ptr); ptr += 4 * (size_t)cap;
+        a_trig[i] = reinterpret_cast<int32_t*>(ptr); ptr += 4 * (size_t)cap;
+        a_score[i] = reinterpret_cast<float*>(ptr); ptr += 4 * (size_t)cap;
+    }
+    uint32_t* eflag = reinterpret_cast<uint32_t*>(ptr); ptr += 4 * (size_t)cap;
+    int32_t* w_src = reinterpret_cast<int32_t*>(ptr); ptr += 4 * (size_t)(cap + 1);
+    float* w_score = reinterpret_cast<float*>(ptr); ptr += 4 * (size_t)(cap + 1);
+    int32_t* st_l = reinterpret_cast<int32_t*>(ptr); ptr += 4 * kMaxCascades;
+    int32_t* sx_l = reinterpret_cast<int32_t*>(ptr); ptr += 4 * kMaxCascades;
+    int* wave_tot = reinterpret_cast<int*>(ptr);
+
+    int64_t* g_stored = A.stored_tokens + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+    int64_t* g_start = A.start_indices + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+    int64_t* g_sinks = A.stored_sinks + n * A.stored_sinks_stride[0] + h * A.stored_sinks_stride[1];
+    const int64_t cs_base = n * A.cache_s_stride[0] + h * A.cache_s_stride[1];
+    int32_t* first = p.first + bh * A.K + p.token_offset;
+    int32_t* next_of = p.next_of + bh * S;
+
+    const int64_t seen = *A.real_token_idx + p.token_offset;  // tokens before token 0 of this launch
+    const int64_t sinks0 = *g_sinks;
+    int64_t room = NS - sinks0;
+    if (room < 0) room = 0;
+    const int n_sink_new = room < cap ? (int)room : cap;
+
+    for (int i = tid; i < C; i += T) {
+        st_l[i] = (int32_t)g_stored[i * A.tracker_stride[2]];
+        sx_l[i] = (int32_t)g_start[i * A.tracker_stride[2]];
+    }
+    // level-0 arrivals: the non-sink tokens of this launch, in order (cascading_cache.py:447-462)
+    for (int t = tid; t < cap; t += T) {
+        if (t < n_sink_new) {
+            first[t] = (int32_t)(S + sinks0 + t);
+        } else {
+            first[t] = -1;
+            const int a = t - n_sink_new;
+            a_src[0][a] = -1 - t;
+            a_trig[0][a] = t;
+            a_score[0][a] = load_as_float(
+                A.s, n * A.s_stride[0] + h * A.s_stride[1] + (p.token_offset + t) * A.s_stride[2], A.dtype);
+        }
+    }
+    __syncthreads();
+    if (tid == 0 && n_sink_new > 0) *g_sinks = sinks0 + n_sink_new;
+
+    int nA = cap - n_sink_new;
+    int cur = 0;
+    for (int i = 0; i < C && nA > 0; i++) {
+        const int64_t l = (int64_t)i * W;
+        const int stored0 = st_l[i], start0 = sx_l[i];
+        const int64_t per = A.do_cache_every_n[i];
+        const int32_t* Asrc = a_src[cur];
+        const int32_t* Atrig = a_trig[cur];
+        const float* Ascore = a_score[cur];
+
+        // ---- pass 1: insert flags (accept, or the first arrival of an empty cascade:
+        //      cascading_cache.py:471-478, 606) and their running index
+        int E = 0;
+        for (int base = 0; base < nA; base += T) {
+            const int a = base + tid;
+            bool f = false;
+            if (a < nA) {
+                const int64_t gidx = seen + Atrig[a];  // 0-based global index of the triggering token
+                const bool acc = (A.eager_fill && gidx <= S + NS) || (((gidx - NS) % per) == 0);
+                f = acc || (stored0 == 0 && a == 0);
+            }
+            int ex;
+            const int tot = block_flag_scan(f, wave_tot, ex);
+            if (a < nA) eflag[a] = (uint32_t)(E + ex) | (f ? 0x80000000u : 0u);
+            E += tot;
+        }
+        __syncthreads();
+
+        // ---- pass 2: the winner of every group.  Slot 0 of w_* is the newest slot left by
+        //      earlier calls (cascading_cache.py:676-680), slot e+1 belongs to insert e.
+        const int p_lead = (int)l + (stored0 > 0 ? (start0 - 1 + stored0) % stored0 : 0);
+        if (tid == 0 && stored0 > 0) {
+            int ws = p_lead;
+            float wv = load_as_float(A.cache_s, cs_base + (int64_t)p_lead * A.cache_s_stride[2], A.dtype);
+            for (int b = 0; b < nA && !(eflag[b] & 0x80000000u); b++) {
+                if (Ascore[b] >= wv) { ws = Asrc[b]; wv = Ascore[b]; }
+            }
+            w_src[0] = ws;
+            w_score[0] = wv;
+        }
+        for (int a = tid; a < nA; a += T) {
+            const uint32_t ef = eflag[a];
+            if (!(ef & 0x80000000u)) continue;
+            int ws = Asrc[a];
+            float wv = Ascore[a];
+            for (int b = a + 1; b < nA && !(eflag[b] & 0x80000000u); b++) {
+                if (Ascore[b] >= wv) { ws = Asrc[b]; wv = Ascore[b]; }
+            }
+            const int e = (int)(ef & 0x7fffffffu);
+            w_src[e + 1] = ws;
+            w_score[e + 1] = wv;
+        }
+        __syncthreads();
+
+        // ---- pass 3: evictions feed the next cascade; surviving slots become moves
+        const int room_i = (int)W - stored0;          // inserts that still append
+        const bool has_next = (i + 1 < C);
+        int32_t* Bsrc = a_src[cur ^ 1];
+        int32_t* Btrig = a_trig[cur ^ 1];
+        float* Bscore = a_score[cur ^ 1];
+        for (int a = tid; a < nA; a += T) {
+            const uint32_t ef = eflag[a];
+            if (!(ef & 0x80000000u)) continue;
+            const int e = (int)(ef & 0x7fffffffu);
+            if (e >= room_i && has_next) {  // full: the oldest entry leaves (cascading_cache.py:542-604)
+                const int mv = e - room_i;  // index of the evicted entry in [old ring | inserts]
+                int ns;
+                float nv;
+                if (mv < stored0 - 1) {     // an old ring entry nobody touched in this call
+                    ns = (int)l + (int)((start0 + (int64_t)mv) % W);
+                    nv = load_as_float(A.cache_s, cs_base + (int64_t)ns * A.cache_s_stride[2], A.dtype);
+                } else {
+                    ns = w_src[mv - stored0 + 1];
+                    nv = w_score[mv - stored0 + 1];
+                }
+                Bsrc[mv] = ns;
+                Bscore[mv] = nv;
+                Btrig[mv] = Atrig[a];
+            }
+            if (e >= E - (int)W) {  // not evicted again before the call ends
+                const int phys = (int)l + (int)(((int64_t)start0 + stored0 + e) % W);
+                emit_move(first, next_of, phys, w_src[e + 1]);
+            }
+        }
+        if (tid == 0 && stored0 > 0 && E <= (int)W - 1 && w_src[0] != p_lead) {
+            emit_move(first, next_of, p_lead, w_src[0]);
+        }
+        const int n_ev = (stored0 + E > (int)W) ? stored0 + E - (int)W : 0;
+        __syncthreads();
+        if (tid == 0) {
+            const int st_new = stored0 + E < (int)W ? stored0 + E : (int)W;
+            const int sx_new = (int)(((int64_t)start0 + n_ev) % W);
+            st_l[i] = st_new;
+            sx_l[i] = sx_new;
+            g_stored[i * A.tracker_stride[2]] = st_new;
+            g_start[i * A.tracker_stride[2]] = sx_new;
+        }
+        nA = has_next ? n_ev : 0;
+        cur ^= 1;
+    }
+    __syncthreads();
+
+    // ---- position pass (cascading_cache.py:728-774, 129-142): only when the last token of the
+    //      call went to the cascades
+    if (p.do_pos && cap > n_sink_new) {
+        int64_t ub = 0;
+        for (int i = 0; i < C; i++) ub += st_l[i];
+        int64_t* pos = A.pos + n * A.pos_stride[0] + h * A.pos_stride[1];
+        for (int i = 0; i < C; i++) {
+            const int64_t seg = st_l[i] < W ? st_l[i] : W;
+            if (seg <= 0) break;
+            const int64_t sx = sx_l[i];
+            for (int64_t j = tid; j < W; j += T) {
+                pos[((int64_t)i * W + j) * A.pos_stride[2]] = ((j + seg - sx) % seg) + ub - seg;
+            }
+            ub -= W;
+            if (ub <= 0) break;
+        }
+    }
+}
+
+// One 16-byte piece of a row per lane.
+struct RowPiece {
+    uint4 k, v;
+};
+
+template <int LANES>
+__global__ void ckv_update_apply_vec_kernel(UpdateParams p) {
+    const ckv_update_args& A = p.a;
+    constexpr int kGroups = 256 / LANES;
+    const int g = blockIdx.x * kGroups + threadIdx.x / LANES;
+    const int lane = threadIdx.x % LANES;
+    if (g >= p.k_sub) return;
+    const int64_t bh = blockIdx.y;
+    const int64_t n = bh / A.H, h = bh % A.H;
+    const int64_t S = A.max_seq_len;
+    const int32_t* first = p.first + bh * A.K + p.token_offset;
+    const int32_t* next_of = p.next_of + bh * S;
+    int d = first[g];
+    if (d < 0) return;  // the token entered and left the cache inside this call
+
+    const int es = (int)elem_bytes(A.dtype);
+    const int chunks = (int)(A.HID * es / 16);
+    const bool active = lane < chunks;
+    const int64_t t_in = p.token_offset + g;
+
+    const char* kin = reinterpret_cast<const char*>(A.k) +
+                      (n * A.kv_stride[0] + h * A.kv_stride[1] + t_in * A.kv_stride[2]) * es;
+    const char* vin = reinterpret_cast<const char*>(A.v) +
+                      (n * A.kv_stride[0] + h * A.kv_stride[1] + t_in * A.kv_stride[2]) * es;
+    RowPiece carry;
+    carry.k = make_uint4(0, 0, 0, 0);
+    carry.v = make_uint4(0, 0, 0, 0);
+    if (active) {
+        carry.k = reinterpret_cast<const uint4*>(kin)[lane];
+        carry.v = reinterpret_cast<const uint4*>(vin)[lane];
+    }
+
+    if (d >= S) {  // sink slot (cascading_cache.py:61-109)
+        const int64_t j = d - S;
+        const int64_t so = (n * A.sink_stride[0] + h * A.sink_stride[1] + j * A.sink_stride[2]) * es;
+        if (active) {
+            reinterpret_cast<uint4*>(reinterpret_cast<char*>(A.sink_k) + so)[lane] = carry.k;
+            reinterpret_cast<uint4*>(reinterpret_cast<char*>(A.sink_v) + so)[lane] = carry.v;
+        }
+        if (lane == 0) {
+            A.sink_pos[n * A.sink_pos_stride[0] + h * A.sink_pos_stride[1] + j * A.sink_pos_stride[2]] = j;
+            A.sink_mask[n * A.sink_mask_stride[0] + h * A.sink_mask_stride[1] + j * A.sink_mask_stride[2]] = 0;
+        }
+        return;
+    }
+
+    // scalars that travel with the row: score bits and original token index (lane 0 only)
+    uint32_t c_score = 0;
+    int64_t c_og = 0;
+    if (lane == 0) {
+        const int64_t so = n * A.s_stride[0] + h * A.s_stride[1] + t_in * A.s_stride[2];
+        c_score = es == 4 ? reinterpret_cast<const uint32_t*>(A.s)[so] : reinterpret_cast<const uint16_t*>(A.s)[so];
+        c_og = *A.real_token_idx + t_in + 1;  // cascading_cache.py:388
+    }
+    char* ck = reinterpret_cast<char*>(A.cache_k) + (n * A.cache_stride[0] + h * A.cache_stride[1]) * es;
+    char* cv = reinterpret_cast<char*>(A.cache_v) + (n * A.cache_stride[0] + h * A.cache_stride[1]) * es;
+    const int64_t row_bytes = A.cache_stride[2] * es;
+    const int64_t cs_base = n * A.cache_s_stride[0] + h * A.cache_s_stride[1];
+    int64_t* og = A.og_pos + n * A.og_pos_stride[0] + h * A.og_pos_stride[1];
+    uint8_t* mask = A.mask + n * A.mask_stride[0] + h * A.mask_stride[1];
+
+    for (int hop = 0; hop <= A.cascades; hop++) {  // a chain visits each cascade at most once
+        const int nd = next_of[d];
+        RowPiece old;
+        uint32_t o_score = 0;
+        int64_t o_og = 0;
+        uint4* kd = reinterpret_cast<uint4*>(ck + (int64_t)d * row_bytes);
+        uint4* vd = reinterpret_cast<uint4*>(cv + (int64_t)d * row_bytes);
+        const int64_t sidx = cs_base + (int64_t)d * A.cache_s_stride[2];
+        if (nd >= 0) {  // the displaced row lives on elsewhere: pick it up before overwriting
+            if (active) {
+                old.k = kd[lane];
+                old.v = vd[lane];
+            }
+            if (lane == 0) {
+                o_score = es == 4 ? reinterpret_cast<const uint32_t*>(A.cache_s)[sidx]
+                                  : reinterpret_cast<const uint16_t*>(A.cache_s)[sidx];
+                o_og = og[(int64_t)d * A.og_pos_stride[2]];
+            }
+        }
+        if (active) {
+            kd[lane] = carry.k;
+            vd[lane] = carry.v;
+        }
+        if (lane == 0) {
+            if (es == 4) {
+                reinterpret_cast<uint32_t*>(A.cache_s)[sidx] = c_score;
+            } else {
+                reinterpret_cast<uint16_t*>(A.cache_s)[sidx] = (uint16_t)c_score;
+            }
+            og[(int64_t)d * A.og_pos_stride[2]] = c_og;
+            mask[(int64_t)d * A.mask_stride[2]] = 0;
+        }
+        if (nd < 0) break;
+        carry = old;
+        c_score = o_score;
+        c_og = o_og;
+        d = nd;
+    }
+}
+
+// Layouts the vector kernel cannot address (innermost stride != 1, rows not a multiple of 16
+// bytes, unaligned bases): one wavefront per token, one element at a time.
+template <typename U>
+__global__ void ckv_update_apply_elem_kernel(UpdateParams p) {
+    const ckv_update_args& A = p.a;
+    constexpr int kPerLane = 8;
+    const int g = blockIdx.x * (256 / CKV_WAVE) + threadIdx.x / CKV_WAVE;
+    const int lane = threadIdx.x % CKV_WAVE;
+    if (g >= p.k_sub) return;
+    const int64_t bh = blockIdx.y;
+    const int64_t n = bh / A.H, h = bh % A.H;
+    const int64_t S = A.max_seq_len;
+    const int32_t* first = p.first + bh * A.K + p.token_offset;
+    const int32_t* next_of = p.next_of + bh * S;
+    int d = first[g];
+    if (d < 0) return;
+    const int64_t t_in = p.token_offset + g;
+    const U* kin = reinterpret_cast<const U*>(A.k) + n * A.kv_stride[0] + h * A.kv_stride[1] + t_in * A.kv_stride[2];
+    const U* vin = reinterpret_cast<const U*>(A.v) + n * A.kv_stride[0] + h * A.kv_stride[1] + t_in * A.kv_stride[2];
+    U ck_[kPerLane], cv_[kPerLane], ok_[kPerLane], ov_[kPerLane];
+#pragma unroll
+    for (int r = 0; r < kPerLane; r++) {
+        const int64_t e = lane + (int64_t)r * CKV_WAVE;
+        if (e < A.HID) {
+            ck_[r] = kin[e * A.kv_stride[3]];
+            cv_[r] = vin[e * A.kv_stride[3]];
+        }
+    }
+    if (d >= S) {
+        const int64_t j = d - S;
+        U* sk = reinterpret_cast<U*>(A.sink_k) + n * A.sink_stride[0] + h * A.sink_stride[1] + j * A.sink_stride[2];
+        U* sv = reinterpret_cast<U*>(A.sink_v) + n * A.sink_stride[0] + h * A.sink_stride[1] + j * A.sink_stride[2];
+#pragma unroll
+        for (int r = 0; r < kPerLane; r++) {
+            const int64_t e = lane + (int64_t)r * CKV_WAVE;
+            if (e < A.HID) {
+                sk[e * A.sink_stride[3]] = ck_[r];
+                sv[e * A.sink_stride[3]] = cv_[r];
+            }
+        }
+        if (lane == 0) {
+            A.sink_pos[n * A.sink_pos_stride[0] + h * A.sink_pos_stride[1] + j * A.sink_pos_stride[2]] = j;
+            A.sink_mask[n * A.sink_mask_stride[0] + h * A.sink_mask_stride[1] + j * A.sink_mask_stride[2]] = 0;
+        }
+        return;
+    }
+    U c_score = reinterpret_cast<const U*>(A.s)[n * A.s_stride[0] + h * A.s_stride[1] + t_in * A.s_stride[2]];
+    int64_t c_og = *A.real_token_idx + t_in + 1;
+    U* ck = reinterpret_cast<U*>(A.cache_k) + n * A.cache_stride[0] + h * A.cache_stride[1];
+    U* cv = reinterpret_cast<U*>(A.cache_v) + n * A.cache_stride[0] + h * A.cache_stride[1];
+    U* cs = reinterpret_cast<U*>(A.cache_s) + n * A.cache_s_stride[0] + h * A.cache_s_stride[1];
+    int64_t* og = A.og_pos + n * A.og_pos_stride[0] + h * A.og_pos_stride[1];
+    uint8_t* mask = A.mask + n * A.mask_stride[0] + h * A.mask_stride[1];
+    for (int hop = 0; hop <= A.cascades; hop++) {
+        const int nd = next_of[d];
+        U* kd = ck + (int64_t)d * A.cache_stride[2];
+        U* vd = cv + (int64_t)d * A.cache_stride[2];
+        U o_score = c_score;
+        int64_t o_og = 0;
+        if (nd >= 0) {
+#pragma unroll
+            for (int r = 0; r < kPerLane; r++) {
+                const int64_t e = lane + (int64_t)r * CKV_WAVE;
+                if (e < A.HID) {
+                    ok_[r] = kd[e * A.cache_stride[3]];
+                    ov_[r] = vd[e * A.cache_stride[3]];
+                }
+            }
+            o_score = cs[(int64_t)d * A.cache_s_stride[2]];
+            o_og = og[(int64_t)d * A.og_pos_stride[2]];
+        }
+#pragma unroll
+        for (int r = 0; r < kPerLane; r++) {
+            const int64_t e = lane + (int64_t)r * CKV_WAVE;
+            if (e < A.HID) {
+                kd[e * A.cache_stride[3]] = ck_[r];
+                vd[e * A.cache_stride[3]] = cv_[r];
+            }
+        }
+        if (lane == 0) {
+            cs[(int64_t)d * A.cache_s_stride[2]] = c_score;
+            og[(int64_t)d * A.og_pos_stride[2]] = c_og;
+            mask[(int64_t)d * A.mask_stride[2]] = 0;
+        }
+        if (nd < 0) break;
+#pragma unroll
+        for (int r = 0; r < kPerLane; r++) {
+            ck_[r] = ok_[r];
+            cv_[r] = ov_[r];
+        }
+        c_score = o_score;
+        c_og = o_og;
+        d = nd;
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline size_t plan_lds_bytes(int cap) {
+    return (size_t)cap * 28 + (size_t)(cap + 1) * 8 + kMaxCascades * 8 + 64 * sizeof(int) + 64;
+}
+
+}  // namespace
+}  // namespace ckv
+
+extern "C" int64_t ckv_update_workspace_bytes(int64_t N, int64_t H, int64_t K, int64_t max_seq_len,
+                                              int32_t cascades) {
+    (void)cascades;
+    if (N <= 0 || H <= 0 || K < 0 || max_seq_len <= 0) return 0;
+    return ckv::align_up(N * H * (K + max_seq_len) * (int64_t)sizeof(int32_t), 256) + 256;
+}
+
+extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
+    using namespace ckv;
+    if (!args) return CKV_ERR_NULL;
+    const ckv_update_args& A = *args;
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (A.dtype != CKV_F32 && A.dtype != CKV_F16 && A.dtype != CKV_BF16) return CKV_ERR_DTYPE;
+    if (A.N <= 0 || A.H <= 0 || A.K < 0 || A.HID <= 0 || A.num_sink < 0) return CKV_ERR_SHAPE;
+    if (A.window_size <= 0 || A.cascades <= 0 || A.cascades > kMaxCascades) return CKV_ERR_SHAPE;
+    if ((int64_t)A.cascades * A.window_size != A.max_seq_len) return CKV_ERR_SHAPE;
+    if (A.max_seq_len + A.num_sink >= (int64_t)1 << 30 || A.K >= (int64_t)1 << 30) return CKV_ERR_SHAPE;
+    if (A.N * A.H > 65535) return CKV_ERR_UNSUPPORTED;
+    if (!A.cache_k || !A.cache_v || !A.cache_s || !A.mask || !A.pos || !A.og_pos || !A.stored_tokens ||
+        !A.start_indices || !A.stored_sinks || !A.do_cache_every_n || !A.real_token_idx)
+        return CKV_ERR_NULL;
+    if (A.num_sink > 0 && (!A.sink_k || !A.sink_v || !A.sink_mask || !A.sink_pos)) return CKV_ERR_NULL;
+    if (A.K == 0) return CKV_OK;
+    if (!A.k || !A.v || !A.s) return CKV_ERR_NULL;
+    const int64_t need = ckv_update_workspace_bytes(A.N, A.H, A.K, A.max_seq_len, A.cascades);
+    if (!A.workspace || A.workspace_bytes < need) return CKV_ERR_WORKSPACE;
+
+    const int es = (int)elem_bytes(A.dtype);
+    const bool vec = A.kv_stride[3] == 1 && A.cache_stride[3] == 1 && (A.num_sink == 0 || A.sink_stride[3] == 1) &&
+                     (A.HID * es) % 16 == 0 && A.HID * es <= 16 * 64 && aligned16(A.k) && aligned16(A.v) &&
+                     aligned16(A.cache_k) && aligned16(A.cache_v) &&
+                     (A.num_sink == 0 || (aligned16(A.sink_k) && aligned16(A.sink_v))) &&
+                     (A.kv_stride[0] * es) % 16 == 0 && (A.kv_stride[1] * es) % 16 == 0 &&
+                     (A.kv_stride[2] * es) % 16 == 0 && (A.cache_stride[0] * es) % 16 == 0 &&
+                     (A.cache_stride[1] * es) % 16 == 0 && (A.cache_stride[2] * es) % 16 == 0 &&
+                     (A.sink_stride[0] * es) % 16 == 0 && (A.sink_stride[1] * es) % 16 == 0 &&
+                     (A.sink_stride[2] * es) % 16 == 0;
+    if (!vec && A.HID > 8 * CKV_WAVE) return CKV_ERR_UNSUPPORTED;
+
+    int dev = 0, lds_max = 65536;
+    CKV_HIP_TRY(hipGetDevice(&dev));
+    if (hipDeviceGetAttribute(&lds_max, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        lds_max = 65536;
+    }
+    int qmax = (int)((lds_max - 2048) / 36);
+    qmax = qmax / 64 * 64;
+    if (qmax > 8192) qmax = 8192;
+    if (qmax < 64) return CKV_ERR_UNSUPPORTED;
+
+    UpdateParams p;
+    p.a = A;
+    p.first = reinterpret_cast<int32_t*>(A.workspace);
+    p.next_of = p.first + A.N * A.H * A.K;
+
+    for (int64_t off = 0; off < A.K; off += qmax) {
+        const int ksub = (int)((A.K - off < qmax) ? (A.K - off) : qmax);
+        p.token_offset = off;
+        p.k_sub = ksub;
+        p.do_pos = (off + ksub == A.K) ? 1 : 0;
+        const int T = ksub <= 64 ? 64 : (ksub <= 256 ? 256 : 1024);
+        const size_t lds = plan_lds_bytes(ksub);
+        if (lds > 48 * 1024) {
+            CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(ckv_update_plan_kernel),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        }
+        hipLaunchKernelGGL(ckv_update_plan_kernel, dim3((unsigned)(A.N * A.H)), dim3(T), lds, stream, p);
+        CKV_HIP_TRY(hipGetLastError());
+
+        if (vec) {
+            const int chunks = (int)(A.HID * es / 16);
+            int lanes = 1;
+            while (lanes < chunks) lanes *= 2;
+            const dim3 block(256);
+            const dim3 grid((unsigned)((ksub + 256 / lanes - 1) / (256 / lanes)), (unsigned)(A.N * A.H));
+            switch (lanes) {
+                case 1: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<1>, grid, block, 0, stream, p); break;
+                case 2: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<2>, grid, block, 0, stream, p); break;
+                case 4: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<4>, grid, block, 0, stream, p); break;
+                case 8: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<8>, grid, block, 0, stream, p); break;
+                case 16: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<16>, grid, block, 0, stream, p); break;
+                case 32: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<32>, grid, block, 0, stream, p); break;
+                default: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<64>, grid, block, 0, stream, p); break;
+            }
+        } else {
+            const dim3 block(256);
+            const dim3 grid((unsigned)((ksub + 3) / 4), (unsigned)(A.N * A.H));
+            if (es == 4) {
+                hipLaunchKernelGGL(ckv_update_apply_elem_kernel<uint32_t>, grid, block, 0, stream, p);
+            } else {
+                hipLaunchKernelGGL(ckv_update_apply_elem_kernel<uint16_t>, grid, block, 0, stream, p);
+            }
+        }
+        CKV_HIP_TRY(hipGetLastError());
+    }
+    return CKV_OK;
+}
