@@ -1,0 +1,177 @@
+"""Host-side mirror of the reference's attention wrapper (cascade/models/cascade_attention.py).
+
+``cascade_attention`` is the fused operator: one ``ckv_attn`` call replaces the RoPE of the whole
+cache, ``repeat_kv``, the concatenations, ``attention``/the eager matmuls, ``calc_scores`` and the
+score-EMA assignment (cascade_attention.py:150-224 / 250-330), then ``cache.update`` scatters the
+chunk (cascade_attention.py:226-227, 334-339).  ``CascadeAttention`` keeps the method names of
+the reference mixin so model code written against it keeps working.
+"""
+import ctypes as C
+import math
+from typing import Optional
+
+import torch
+from torch import nn
+
+from . import _abi
+from .cascading_cache import CascadingKVCache, _require_device, workspace
+
+
+def default_inv_freq(head_dim: int, theta: float, device) -> torch.Tensor:
+    """The unscaled rotary frequencies, computed exactly like the HF default initialiser the
+    reference model uses (modeling_llama.py:166-177): fp32 ``1 / theta^(2i/d)``."""
+    inv = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.int64).float() / head_dim))
+    return inv.to(device)
+
+
+def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_pos: bool = False) -> torch.Tensor:
+    """Position ids of the incoming chunk (cascade_attention.py:119-150) without a host sync:
+    0.. on the first call, otherwise one past the largest id among sinks and cache slots
+    (stale and masked entries included, as in the reference)."""
+    dev = cache.key_cache[layer_idx].device
+    ar = torch.arange(q_len, device=dev, dtype=torch.long)
+    if cache._seen_host[layer_idx] == 0:
+        return ar
+    if do_og_pos:
+        key_max = cache.og_pos[layer_idx].amax()
+    else:
+        key_max = cache.pos[layer_idx][0, 0].amax() + cache.pos_shift(layer_idx)
+    if cache.num_sink_tokens > 0:
+        key_max = torch.maximum(key_max, cache.sink_pos[layer_idx][0, 0].amax())
+    return ar + (key_max + 1)
+
+
+def cascade_attention(query_states, key_states, value_states, cache: CascadingKVCache, layer_idx: int,
+                      inv_freq: torch.Tensor, head_reduction: Optional[str] = None,
+                      homogeneous_heads: bool = False, do_og_pos: bool = False, scale: Optional[float] = None,
+                      update_cache: bool = True):
+    """Attention of one chunk over [sink | cascades | chunk] plus the cache bookkeeping.
+
+    query_states ``(B, H, q, D)``, key/value_states ``(B, KVH, q, D)``, all un-rotated.
+    Returns ``out (B, H, q, D)``; mutates ``cache.score_cache[layer_idx]`` and, if
+    ``update_cache``, scatters the chunk into the cache with its new scores.
+    """
+    _require_device(query_states, "query_states")
+    lib = _abi.lib()
+    B, H, Q, D = query_states.shape
+    KVH = key_states.size(1)
+    assert key_states.shape == (B, KVH, Q, D) and value_states.shape == (B, KVH, Q, D)
+    assert _abi.same_layout(key_states, value_states)
+    dtype = query_states.dtype
+    L = layer_idx
+    NS, S = cache.num_sink_tokens, cache.max_seq_len[L]
+    reduction = head_reduction or cache.head_reduction
+    if scale is None:
+        scale = 1 / math.sqrt(D)
+
+    q_pos = chunk_positions(cache, L, Q, do_og_pos)
+    out = torch.empty((B, H, Q, D), dtype=dtype, device=query_states.device)
+    new_scores = torch.empty((B, KVH, Q), dtype=dtype, device=query_states.device)
+
+    a = _abi.AttnArgs()
+    a.q = query_states.data_ptr()
+    _abi.set_strides(a.q_stride, query_states)
+    a.k_new, a.v_new = key_states.data_ptr(), value_states.data_ptr()
+    _abi.set_strides(a.kv_new_stride, key_states)
+    a.sink_k, a.sink_v = cache.sink_keys[L].data_ptr(), cache.sink_values[L].data_ptr()
+    _abi.set_strides(a.sink_stride, cache.sink_keys[L])
+    a.cache_k, a.cache_v = cache.key_cache[L].data_ptr(), cache.value_cache[L].data_ptr()
+    _abi.set_strides(a.cache_stride, cache.key_cache[L])
+    assert cache.sink_mask[L].stride(-1) == 1 and cache.mask[L].stride(-1) == 1
+    a.sink_mask, a.mask = cache.sink_mask[L].data_ptr(), cache.mask[L].data_ptr()  # row [0, 0]
+    a.q_pos = q_pos.data_ptr()
+    assert cache.sink_pos[L].stride(-1) == 1 and cache.pos[L].stride(-1) == 1 and cache.og_pos[L].stride(-1) == 1
+    a.sink_pos = cache.sink_pos[L].data_ptr()
+    a.sink_pos_stride[0], a.sink_pos_stride[1] = 0, 0
+    if do_og_pos:  # every (batch, head) rotates its keys at their original positions (:161-164)
+        a.pos = cache.og_pos[L].data_ptr()
+        a.pos_stride[0], a.pos_stride[1] = cache.og_pos[L].stride(0), cache.og_pos[L].stride(1)
+        a.pos_shift = 0
+    else:
+        a.pos = cache.pos[L].data_ptr()
+        a.pos_stride[0], a.pos_stride[1] = 0, 0
+        a.pos_shift = cache.pos_shift(L)
+    a.cache_s = cache.score_cache[L].data_ptr()
+    _abi.set_strides(a.cache_s_stride, cache.score_cache[L])
+    a.out = out.data_ptr()
+    _abi.set_strides(a.out_stride, out)
+    a.new_scores = new_scores.data_ptr()
+    _abi.set_strides(a.new_scores_stride, new_scores)
+    a.lse = None
+    a.B, a.H, a.KVH, a.Q, a.D = B, H, KVH, Q, D
+    a.num_sink, a.S = NS, S
+    a.scale = float(scale)
+    a.rope_theta = 0.0
+    assert inv_freq.dtype == torch.float32 and inv_freq.numel() == D // 2 and inv_freq.is_contiguous()
+    a.inv_freq = inv_freq.data_ptr()
+    a.beta = float(cache.beta)
+    a.head_reduction = _abi.CKV_REDUCE[reduction]
+    a.homogeneous_heads = int(bool(homogeneous_heads))
+    a.dtype = _abi.dtype_code(dtype)
+    need = lib.ckv_attn_workspace_bytes(B, H, KVH, Q, D, NS, S, a.dtype)
+    ws = workspace(query_states.device, need)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    with torch.cuda.device(query_states.device):
+        stream = torch.cuda.current_stream(query_states.device).cuda_stream
+        _abi.check(lib.ckv_attn(C.byref(a), C.c_void_p(stream)), "ckv_attn")
+    if update_cache:
+        cache.update(key_states, value_states, L, score_states=new_scores)
+    return out, new_scores
+
+
+class CascadeAttention(nn.Module):
+    """Attention layer with the reference mixin's surface (cascade_attention.py:38-340).
+
+    A concrete layer provides ``q_proj/k_proj/v_proj/o_proj``, ``num_heads``,
+    ``num_key_value_heads``, ``head_dim``, ``layer_idx``, ``rope_theta`` and a ``config`` with
+    ``_homogeneous_heads``, ``_do_og_pos`` and ``_head_reduction`` (llama_eval.py:142-152).
+    Chunked prefill and single-token decode both run the fused HIP path; there is no eager arm.
+    """
+
+    def forward(self, hidden_states, attention_mask=None, position_ids=None, past_key_value=None,
+                output_attentions=False, use_cache=False, cache_position=None, position_embeddings=None):
+        if isinstance(past_key_value, CascadingKVCache):
+            return self.forward_cascade(
+                hidden_states=hidden_states, past_key_value=past_key_value,
+                homogeneous_heads=self.config._homogeneous_heads, do_og_pos=self.config._do_og_pos)
+        raise ValueError("unknown custom attention")
+
+    def qkv(self, x, size, kv_size):
+        q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+        q = q.view(*size).transpose(1, 2)
+        k = k.view(*kv_size).transpose(1, 2)
+        v = v.view(*kv_size).transpose(1, 2)
+        return q, k, v
+
+    def forward_cascade(self, hidden_states, attention_mask=None, position_ids=None, past_key_value=None,
+                        output_attentions=False, use_cache=False, cache_position=None, use_flash=True,
+                        homogeneous_heads=True, do_og_pos=False, use_selfextend=False, position_embeddings=None):
+        if use_selfextend:
+            raise NotImplementedError("use_selfextend is a dead arm in the reference (never enabled)")
+        bsz, q_len, _ = hidden_states.size()
+        query_states, key_states, value_states = self.qkv(
+            hidden_states, (bsz, q_len, self.num_heads, self.head_dim),
+            (bsz, q_len, self.num_key_value_heads, self.head_dim))
+        if not hasattr(self, "_inv_freq") or self._inv_freq.device != hidden_states.device:
+            self._inv_freq = default_inv_freq(self.head_dim, self.rope_theta, hidden_states.device)
+        out, _ = cascade_attention(query_states, key_states, value_states, past_key_value, self.layer_idx,
+                                   self._inv_freq, head_reduction=self.config._head_reduction,
+                                   homogeneous_heads=homogeneous_heads, do_og_pos=do_og_pos)
+        out = out.transpose(1, 2).contiguous().view(bsz, q_len, -1)
+        out = self.o_proj(out)
+        return out, None, past_key_value
+
+    def calc_scores(self, scores, homogeneous_heads, n_keys, q_len):
+        """Head reduction of per-head score sums (cascade_attention.py:231-248), for callers
+        that hold per-head scores of their own; the fused path reduces inside the kernels."""
+        kvh = self.num_key_value_heads
+        func = {"mean": torch.mean, "max": torch.amax,
+                "median": lambda x, **kw: torch.median(x, **kw).values}[self.config._head_reduction]
+        if homogeneous_heads:
+            ema_scores = func(scores[:, :, :n_keys], dim=1, keepdim=True)
+            scores = func(scores[:, :, -q_len:], dim=1, keepdim=True).repeat(1, kvh, 1)
+        else:
+            b, h, s = scores.size()
+            ema_scores = func(scores[:, :, :n_keys].view(b, kvh, h // kvh, -1), dim=2)
+            scores = func(scores[:, :, -q_len:].view(b, kvh, h // kvh, -1), dim=2)
+        return ema_scores, scores

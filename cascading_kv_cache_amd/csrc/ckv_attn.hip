@@ -1,6 +1,188 @@
-// placeholder until the attention kernels land
-#include "ckv_common.h"
-extern "C" int64_t ckv_attn_workspace_bytes(int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int32_t) { return 0; }
-extern "C" int ckv_attn(const ckv_attn_args*, void*) { return CKV_ERR_UNSUPPORTED; }
-extern "C" int64_t ckv_dense_workspace_bytes(int64_t, int64_t, int64_t, int64_t, int64_t, int32_t) { return 0; }
-extern "C" int ckv_attn_dense(const ckv_dense_args*, void*) { return CKV_ERR_UNSUPPORTED; }
+// ckv_attn / ckv_attn_dense: argument checking, workspace carving and kernel-family dispatch.
+#include "ckv_attn_internal.h"
+
+#include <math.h>
+
+namespace ckv {
+namespace {
+
+struct Carver {
+    char* base;
+    int64_t off = 0;
+    explicit Carver(void* b) : base(reinterpret_cast<char*>(b)) {}
+    void* take(int64_t bytes) {
+        void* p = base ? base + off : nullptr;
+        off += align_up(bytes, 256);
+        return p;
+    }
+};
+
+struct AttnWorkspace {
+    void *qr, *kr, *vc;
+    uint8_t* kmasked;
+    float *lse, *colsum, *w_ema, *w_new;
+    int64_t bytes;
+};
+
+AttnWorkspace carve_attn(void* base, int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t D, int64_t NS, int64_t S,
+                         int dtype) {
+    const int64_t es = elem_bytes(dtype), N = NS + S + Q;
+    Carver c(base);
+    AttnWorkspace w;
+    w.qr = c.take(B * H * Q * D * es);
+    w.kr = c.take(B * KVH * N * D * es);
+    w.vc = c.take(B * KVH * N * D * es);
+    w.kmasked = (uint8_t*)c.take(NS + S);
+    w.lse = (float*)c.take(B * H * Q * 4);
+    w.colsum = (float*)c.take(B * H * N * 4);
+    w.w_ema = (float*)c.take(Q * 4);
+    w.w_new = (float*)c.take(Q * 4);
+    w.bytes = c.off;
+    return w;
+}
+
+void contiguous_strides(int64_t* st, int64_t d1, int64_t d2, int64_t d3) {
+    st[0] = d1 * d2 * d3;
+    st[1] = d2 * d3;
+    st[2] = d3;
+    st[3] = 1;
+}
+
+}  // namespace
+}  // namespace ckv
+
+extern "C" int64_t ckv_attn_workspace_bytes(int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t D, int64_t num_sink,
+                                            int64_t S, int32_t dtype) {
+    if (B <= 0 || H <= 0 || KVH <= 0 || Q <= 0 || D <= 0 || num_sink < 0 || S < 0) return 0;
+    return ckv::carve_attn(nullptr, B, H, KVH, Q, D, num_sink, S, dtype).bytes;
+}
+
+extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
+    using namespace ckv;
+    if (!args) return CKV_ERR_NULL;
+    const ckv_attn_args& a = *args;
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (a.dtype != CKV_F32 && a.dtype != CKV_F16 && a.dtype != CKV_BF16) return CKV_ERR_DTYPE;
+    if (a.B <= 0 || a.H <= 0 || a.KVH <= 0 || a.Q <= 0 || a.D <= 0 || a.num_sink < 0 || a.S < 0) return CKV_ERR_SHAPE;
+    if (a.H % a.KVH != 0 || a.D % 2 != 0) return CKV_ERR_SHAPE;
+    if (a.head_reduction < CKV_REDUCE_MEAN || a.head_reduction > CKV_REDUCE_MEDIAN) return CKV_ERR_SHAPE;
+    if ((a.homogeneous_heads ? a.H : a.H / a.KVH) > 128) return CKV_ERR_UNSUPPORTED;
+    if (!a.q || !a.k_new || !a.v_new || !a.out || !a.q_pos) return CKV_ERR_NULL;
+    if (a.num_sink > 0 && (!a.sink_k || !a.sink_v || !a.sink_mask || !a.sink_pos)) return CKV_ERR_NULL;
+    if (a.S > 0 && (!a.cache_k || !a.cache_v || !a.mask || !a.pos)) return CKV_ERR_NULL;
+    if (!(a.beta > 0.0) || !(a.beta <= 1.0)) return CKV_ERR_SHAPE;
+    AttnWorkspace w = carve_attn(a.workspace, a.B, a.H, a.KVH, a.Q, a.D, a.num_sink, a.S, a.dtype);
+    if (!a.workspace || a.workspace_bytes < w.bytes) return CKV_ERR_WORKSPACE;
+
+    const int64_t N = a.num_sink + a.S + a.Q;
+    const bool want_scores = a.cache_s || a.new_scores;
+    int rc;
+    if (want_scores) {
+        rc = launch_weights(w.w_ema, w.w_new, a.Q, a.beta, a.dtype, stream);
+        if (rc) return rc;
+    }
+    PrepProblem pp{&a, w.qr, w.kr, w.vc, w.kmasked};
+    rc = launch_prep_generic(pp, stream);
+    if (rc) return rc;
+
+    CoreProblem cp;
+    cp.q = w.qr;
+    contiguous_strides(cp.q_stride, a.H, a.Q, a.D);
+    cp.k = w.kr;
+    cp.v = w.vc;
+    contiguous_strides(cp.kv_stride, a.KVH, N, a.D);
+    cp.kmasked = (a.num_sink + a.S) > 0 ? w.kmasked : nullptr;
+    cp.out = a.out;
+    for (int i = 0; i < 4; i++) cp.out_stride[i] = a.out_stride[i];
+    cp.lse = w.lse;
+    cp.colsum = want_scores ? w.colsum : nullptr;
+    cp.w_ema = w.w_ema;
+    cp.w_new = w.w_new;
+    cp.new_mode = 1;
+    cp.B = a.B; cp.H = a.H; cp.KVH = a.KVH; cp.Q = a.Q; cp.N = N; cp.D = a.D;
+    cp.scale = a.scale;
+    cp.dtype = a.dtype;
+    rc = launch_core_generic(cp, stream);
+    if (rc) return rc;
+    if (a.lse) {
+        CKV_HIP_TRY(hipMemcpyAsync(a.lse, w.lse, a.B * a.H * a.Q * sizeof(float), hipMemcpyDeviceToDevice, stream));
+    }
+    if (want_scores) {
+        FinishProblem fp;
+        fp.colsum = w.colsum;
+        fp.N = N;
+        fp.cache_s = a.S > 0 ? a.cache_s : nullptr;
+        fp.new_scores = a.new_scores;
+        for (int i = 0; i < 3; i++) {
+            fp.cache_s_stride[i] = a.cache_s_stride[i];
+            fp.new_scores_stride[i] = a.new_scores_stride[i];
+        }
+        fp.B = a.B; fp.H = a.H; fp.KVH = a.KVH; fp.Q = a.Q; fp.S = a.S; fp.num_sink = a.num_sink;
+        fp.beta_pow_q = (float)pow(a.beta, (double)a.Q);
+        fp.head_reduction = a.head_reduction;
+        fp.homogeneous = a.homogeneous_heads;
+        fp.dtype = a.dtype;
+        rc = launch_finish(fp, stream);
+        if (rc) return rc;
+    }
+    return CKV_OK;
+}
+
+extern "C" int64_t ckv_dense_workspace_bytes(int64_t B, int64_t H, int64_t n_ctx, int64_t n_kv, int64_t D,
+                                             int32_t dtype) {
+    (void)D;
+    (void)dtype;
+    if (B <= 0 || H <= 0 || n_ctx <= 0 || n_kv < n_ctx) return 0;
+    using ckv::align_up;
+    return align_up(B * H * n_ctx * 4, 256) + align_up(B * H * n_kv * 4, 256) + 2 * align_up(n_ctx * 4, 256);
+}
+
+extern "C" int ckv_attn_dense(const ckv_dense_args* args, void* stream_) {
+    using namespace ckv;
+    if (!args) return CKV_ERR_NULL;
+    const ckv_dense_args& a = *args;
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    if (a.dtype != CKV_F32 && a.dtype != CKV_F16 && a.dtype != CKV_BF16) return CKV_ERR_DTYPE;
+    if (a.B <= 0 || a.H <= 0 || a.n_ctx <= 0 || a.n_kv < a.n_ctx || a.D <= 0) return CKV_ERR_SHAPE;
+    if (!a.q || !a.k || !a.v || !a.out) return CKV_ERR_NULL;
+    if (a.n_kv > a.n_ctx && !a.mask) return CKV_ERR_NULL;
+    if (!(a.beta > 0.0) || !(a.beta <= 1.0)) return CKV_ERR_SHAPE;
+    const int64_t need = ckv_dense_workspace_bytes(a.B, a.H, a.n_ctx, a.n_kv, a.D, a.dtype);
+    if (!a.workspace || a.workspace_bytes < need) return CKV_ERR_WORKSPACE;
+    Carver c(a.workspace);
+    float* lse = (float*)c.take(a.B * a.H * a.n_ctx * 4);
+    float* colsum = (float*)c.take(a.B * a.H * a.n_kv * 4);
+    float* w_ema = (float*)c.take(a.n_ctx * 4);
+    float* w_new = (float*)c.take(a.n_ctx * 4);
+    int rc;
+    if (a.scores) {
+        rc = launch_weights(w_ema, w_new, a.n_ctx, a.beta, a.dtype, stream);
+        if (rc) return rc;
+    }
+    CoreProblem cp;
+    cp.q = a.q;
+    cp.k = a.k;
+    cp.v = a.v;
+    for (int i = 0; i < 4; i++) {
+        cp.q_stride[i] = a.q_stride[i];
+        cp.kv_stride[i] = a.kv_stride[i];
+        cp.out_stride[i] = a.out_stride[i];
+    }
+    cp.kmasked = a.n_kv > a.n_ctx ? a.mask : nullptr;
+    cp.out = a.out;
+    cp.lse = lse;
+    cp.colsum = a.scores ? colsum : nullptr;
+    cp.w_ema = w_ema;
+    cp.w_new = w_new;
+    cp.new_mode = 0;  // every key is weighted by the query row alone (flash_attention.py:73-77)
+    cp.B = a.B; cp.H = a.H; cp.KVH = a.H; cp.Q = a.n_ctx; cp.N = a.n_kv; cp.D = a.D;
+    cp.scale = a.scale;
+    cp.dtype = a.dtype;
+    rc = launch_core_generic(cp, stream);
+    if (rc) return rc;
+    if (a.scores) {
+        rc = launch_cast_scores(colsum, a.scores, a.scores_stride, a.B, a.H, a.n_kv, a.dtype, stream);
+        if (rc) return rc;
+    }
+    return CKV_OK;
+}

@@ -1,0 +1,405 @@
+// fp32-math attention kernels for every dtype: the parity path for float32 caches and the
+// fallback for shapes the MFMA kernels do not take.  Also the small shared stages: score-sum
+// weights, the rotate+gather prologue, and the head-reduction / EMA epilogue.
+#include "ckv_attn_internal.h"
+
+namespace ckv {
+namespace {
+
+template <typename T>
+__device__ inline float round_t(float v) {
+    return Elem<T>::to_float(Elem<T>::from_float(v));
+}
+
+// ---------------------------------------------------------------------------------------------
+// weights: w_ema[m] = (1-beta) * beta^(Q-1-m) as fp32 (cascade_attention.py:315-317);
+//          w_new[k] = (1-beta) * beta^k built in the tensor dtype (cascade_attention.py:270-276)
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void weights_kernel(float* w_ema, float* w_new, int64_t Q, double beta) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= Q) return;
+    const float omb = (float)(1.0 - beta);
+    const float b32 = (float)beta;
+    w_ema[i] = __fmul_rn(omb, powf(b32, (float)(Q - 1 - i)));
+    const float bt = round_t<T>(b32);
+    const float pw = round_t<T>(powf(bt, round_t<T>((float)i)));
+    w_new[i] = round_t<T>(__fmul_rn(omb, pw));
+}
+
+// ---------------------------------------------------------------------------------------------
+// prologue: rotate and gather.  One thread per (row, rotation pair).
+// Rotation is evaluated in the tensor dtype exactly like x*cos + rotate_half(x)*sin
+// (cascade_attention.py:31-35) with cos/sin from fp32 angles cast to the dtype
+// (modeling_llama.py:205-220).
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__device__ inline void rotate_pair(const T* src, int64_t sd, T* dst, int64_t j, int64_t half, int64_t pos,
+                                   const float* inv_freq, float theta, int64_t D) {
+    const float f = inv_freq ? inv_freq[j] : 1.0f / powf(theta, (float)(2 * j) / (float)D);
+    const float ang = __fmul_rn((float)pos, f);
+    float sn, cs;
+    sincosf(ang, &sn, &cs);
+    cs = round_t<T>(cs);
+    sn = round_t<T>(sn);
+    const float x1 = Elem<T>::to_float(src[j * sd]);
+    const float x2 = Elem<T>::to_float(src[(j + half) * sd]);
+    // out[j] = x1*cos + (-x2)*sin ; out[j+half] = x2*cos + x1*sin, each product rounded first
+    const float o1 = round_t<T>(__fadd_rn(round_t<T>(__fmul_rn(x1, cs)), round_t<T>(__fmul_rn(-x2, sn))));
+    const float o2 = round_t<T>(__fadd_rn(round_t<T>(__fmul_rn(x2, cs)), round_t<T>(__fmul_rn(x1, sn))));
+    dst[j] = Elem<T>::from_float(o1);
+    dst[j + half] = Elem<T>::from_float(o2);
+}
+
+template <typename T>
+__global__ void prep_generic_kernel(ckv_attn_args a, T* qr, T* kr, T* vc, uint8_t* kmasked) {
+    const int64_t D = a.D, half = D / 2, NS = a.num_sink, S = a.S, Q = a.Q;
+    const int64_t N = NS + S + Q;
+    const int64_t n_key_items = a.B * a.KVH * N * half;
+    const int64_t n_q_items = a.B * a.H * Q * half;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx < NS + S) kmasked[idx] = idx < NS ? a.sink_mask[idx] : a.mask[idx - NS];
+    if (idx < n_key_items) {
+        const int64_t j = idx % half;
+        const int64_t n = (idx / half) % N;
+        const int64_t kvh = (idx / (half * N)) % a.KVH;
+        const int64_t b = idx / (half * N * a.KVH);
+        const T *ks, *vs;
+        int64_t sd, pos;
+        if (n < NS) {
+            const int64_t off = b * a.sink_stride[0] + kvh * a.sink_stride[1] + n * a.sink_stride[2];
+            ks = (const T*)a.sink_k + off;
+            vs = (const T*)a.sink_v + off;
+            sd = a.sink_stride[3];
+            pos = a.sink_pos[b * a.sink_pos_stride[0] + kvh * a.sink_pos_stride[1] + n];
+        } else if (n < NS + S) {
+            const int64_t slot = n - NS;
+            const int64_t off = b * a.cache_stride[0] + kvh * a.cache_stride[1] + slot * a.cache_stride[2];
+            ks = (const T*)a.cache_k + off;
+            vs = (const T*)a.cache_v + off;
+            sd = a.cache_stride[3];
+            pos = a.pos[b * a.pos_stride[0] + kvh * a.pos_stride[1] + slot] + a.pos_shift;
+        } else {
+            const int64_t m = n - NS - S;
+            const int64_t off = b * a.kv_new_stride[0] + kvh * a.kv_new_stride[1] + m * a.kv_new_stride[2];
+            ks = (const T*)a.k_new + off;
+            vs = (const T*)a.v_new + off;
+            sd = a.kv_new_stride[3];
+            pos = a.q_pos[m];
+        }
+        T* kd = kr + ((b * a.KVH + kvh) * N + n) * D;
+        T* vd = vc + ((b * a.KVH + kvh) * N + n) * D;
+        rotate_pair<T>(ks, sd, kd, j, half, pos, a.inv_freq, a.rope_theta, D);
+        vd[j] = vs[j * sd];
+        vd[j + half] = vs[(j + half) * sd];
+    }
+    if (idx < n_q_items) {
+        const int64_t j = idx % half;
+        const int64_t m = (idx / half) % Q;
+        const int64_t h = (idx / (half * Q)) % a.H;
+        const int64_t b = idx / (half * Q * a.H);
+        const T* qs = (const T*)a.q + b * a.q_stride[0] + h * a.q_stride[1] + m * a.q_stride[2];
+        T* qd = qr + ((b * a.H + h) * Q + m) * D;
+        rotate_pair<T>(qs, a.q_stride[3], qd, j, half, a.q_pos[m], a.inv_freq, a.rope_theta, D);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward: one wavefront per query row, lanes = keys for the logits, lanes = dims for P.V
+// ---------------------------------------------------------------------------------------------
+constexpr int kMaxD = 256;
+
+template <typename T>
+__global__ void fwd_generic_kernel(CoreProblem p) {
+    __shared__ float q_lds[4][kMaxD];
+    const int wave = threadIdx.x / CKV_WAVE, lane = threadIdx.x % CKV_WAVE;
+    const int64_t rows = p.B * p.H * p.Q;
+    int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    const bool active = row < rows;
+    if (!active) row = rows - 1;
+    const int64_t m = row % p.Q;
+    const int64_t h = (row / p.Q) % p.H;
+    const int64_t b = row / (p.Q * p.H);
+    const int64_t G = p.H / p.KVH, kvh = h / G;
+    const int64_t D = p.D, N = p.N, Nc = N - p.Q;
+    const T* qrow = (const T*)p.q + b * p.q_stride[0] + h * p.q_stride[1] + m * p.q_stride[2];
+    for (int64_t d = lane; d < D; d += CKV_WAVE) q_lds[wave][d] = Elem<T>::to_float(qrow[d * p.q_stride[3]]);
+    __syncthreads();
+    if (!active) return;
+    const T* kbase = (const T*)p.k + b * p.kv_stride[0] + kvh * p.kv_stride[1];
+    const T* vbase = (const T*)p.v + b * p.kv_stride[0] + kvh * p.kv_stride[1];
+
+    float m_run = -INFINITY, l_run = 0.f;
+    float o[kMaxD / CKV_WAVE] = {0.f, 0.f, 0.f, 0.f};
+    const int64_t n_end = Nc + m + 1;  // keys past the diagonal are never visible
+    for (int64_t base = 0; base < n_end; base += CKV_WAVE) {
+        const int64_t n = base + lane;
+        bool valid = n < n_end;
+        if (valid && n < Nc && p.kmasked) valid = p.kmasked[n] == 0;
+        float s = -INFINITY;
+        if (valid) {
+            const T* kr = kbase + n * p.kv_stride[2];
+            float acc = 0.f;
+            for (int64_t d = 0; d < D; d++) acc = fmaf(q_lds[wave][d], Elem<T>::to_float(kr[d * p.kv_stride[3]]), acc);
+            s = acc * p.scale;
+        }
+        float cmax = s;
+        for (int off = 32; off > 0; off >>= 1) cmax = fmaxf(cmax, __shfl_xor(cmax, off));
+        if (cmax == -INFINITY) continue;  // nothing visible in this chunk
+        const float m_new = fmaxf(m_run, cmax);
+        const float pe = valid ? expf(s - m_new) : 0.f;
+        float csum = pe;
+        for (int off = 32; off > 0; off >>= 1) csum += __shfl_xor(csum, off);
+        const float alpha = m_run == -INFINITY ? 0.f : expf(m_run - m_new);
+        l_run = l_run * alpha + csum;
+        m_run = m_new;
+#pragma unroll
+        for (int r = 0; r < kMaxD / CKV_WAVE; r++) o[r] *= alpha;
+        const int64_t cnt = n_end - base < CKV_WAVE ? n_end - base : CKV_WAVE;
+        for (int j = 0; j < cnt; j++) {
+            const float pj = __shfl(pe, j);
+            if (pj == 0.f) continue;
+            const T* vr = vbase + (base + j) * p.kv_stride[2];
+#pragma unroll
+            for (int r = 0; r < kMaxD / CKV_WAVE; r++) {
+                const int64_t d = lane + r * CKV_WAVE;
+                if (d < D) o[r] = fmaf(pj, Elem<T>::to_float(vr[d * p.kv_stride[3]]), o[r]);
+            }
+        }
+    }
+    const float inv = 1.f / l_run;
+    T* orow = (T*)p.out + b * p.out_stride[0] + h * p.out_stride[1] + m * p.out_stride[2];
+#pragma unroll
+    for (int r = 0; r < kMaxD / CKV_WAVE; r++) {
+        const int64_t d = lane + r * CKV_WAVE;
+        if (d < D) orow[d * p.out_stride[3]] = Elem<T>::from_float(o[r] * inv);
+    }
+    if (lane == 0 && p.lse) p.lse[row] = m_run + logf(l_run);
+}
+
+// ---------------------------------------------------------------------------------------------
+// score sums: one wavefront per (b, h, 64 keys); lanes = keys, loop over the query rows
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void colsum_generic_kernel(CoreProblem p) {
+    extern __shared__ float k_lds[];  // [64][D + 1]
+    const int lane = threadIdx.x;
+    const int64_t D = p.D, N = p.N, Q = p.Q, Nc = N - Q;
+    const int64_t chunks = (N + CKV_WAVE - 1) / CKV_WAVE;
+    const int64_t c = blockIdx.x % chunks;
+    const int64_t h = (blockIdx.x / chunks) % p.H;
+    const int64_t b = blockIdx.x / (chunks * p.H);
+    const int64_t G = p.H / p.KVH, kvh = h / G;
+    const int64_t n = c * CKV_WAVE + lane;
+    const T* kbase = (const T*)p.k + b * p.kv_stride[0] + kvh * p.kv_stride[1];
+    const int64_t pitch = D + 1;
+    for (int64_t i = lane; i < CKV_WAVE * D; i += CKV_WAVE) {
+        const int64_t r = i / D, d = i % D;
+        const int64_t nn = c * CKV_WAVE + r;
+        k_lds[r * pitch + d] = nn < N ? Elem<T>::to_float(kbase[nn * p.kv_stride[2] + d * p.kv_stride[3]]) : 0.f;
+    }
+    __syncthreads();
+    bool live = n < N;
+    if (live && n < Nc && p.kmasked) live = p.kmasked[n] == 0;
+    const int64_t nrel = n - Nc;  // >= 0 for chunk keys
+    // first query row that can see any key of this chunk of keys
+    int64_t m0 = c * CKV_WAVE - Nc;
+    if (m0 < 0) m0 = 0;
+    const T* qbase = (const T*)p.q + b * p.q_stride[0] + h * p.q_stride[1];
+    const float* lse = p.lse + (b * p.H + h) * Q;
+    float acc = 0.f;
+    for (int64_t m = m0; m < Q; m++) {
+        const T* qr = qbase + m * p.q_stride[2];
+        float s = 0.f;
+        for (int64_t d = 0; d < D; d++) s = fmaf(Elem<T>::to_float(qr[d * p.q_stride[3]]), k_lds[lane * pitch + d], s);
+        const bool vis = live && (n < Nc || nrel <= m);
+        if (vis) {
+            // the eager path holds P in the tensor dtype (softmax output) before weighting it;
+            // chunk-key products are rounded to the dtype as well (cascade_attention.py:319-323)
+            const float pt = round_t<T>(expf(s * p.scale - lse[m]));
+            if (n >= Nc && p.new_mode) {
+                acc = __fadd_rn(acc, round_t<T>(__fmul_rn(pt, p.w_new[m - nrel])));
+            } else {
+                acc = fmaf(p.w_ema[m], pt, acc);
+            }
+        }
+    }
+    if (n < N) p.colsum[(b * p.H + h) * N + n] = acc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// epilogue: per-head sums -> dtype -> head reduction -> EMA / new-token scores
+// (cascade_attention.py:231-248, 319-330)
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__device__ inline float reduce_heads(const float* colsum, int64_t b, int64_t h0, int64_t nh, int64_t H, int64_t N,
+                                     int64_t n, int mode) {
+    const float* base = colsum + (b * H + h0) * N + n;
+    if (mode == CKV_REDUCE_MAX) {
+        float r = round_t<T>(base[0]);
+        for (int64_t g = 1; g < nh; g++) r = fmaxf(r, round_t<T>(base[g * N]));
+        return r;
+    }
+    if (mode == CKV_REDUCE_MEAN) {
+        float r = 0.f;
+        for (int64_t g = 0; g < nh; g++) r = __fadd_rn(r, round_t<T>(base[g * N]));
+        return round_t<T>(r / (float)nh);
+    }
+    float vals[128];  // lower median (torch.median): element (nh-1)/2 of the sorted values
+    for (int64_t g = 0; g < nh; g++) {
+        const float x = round_t<T>(base[g * N]);
+        int64_t i = g;
+        while (i > 0 && vals[i - 1] > x) {
+            vals[i] = vals[i - 1];
+            i--;
+        }
+        vals[i] = x;
+    }
+    return vals[(nh - 1) / 2];
+}
+
+template <typename T>
+__global__ void finish_kernel(FinishProblem p) {
+    const int64_t per = p.S + p.Q;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= p.B * p.KVH * per) return;
+    const int64_t i = idx % per;
+    const int64_t kvh = (idx / per) % p.KVH;
+    const int64_t b = idx / (per * p.KVH);
+    const int64_t G = p.H / p.KVH;
+    const int64_t h0 = p.homogeneous ? 0 : kvh * G;
+    const int64_t nh = p.homogeneous ? p.H : G;
+    if (i < p.S) {
+        if (!p.cache_s) return;
+        const float red = reduce_heads<T>(p.colsum, b, h0, nh, p.H, p.N, p.num_sink + i, p.head_reduction);
+        T* cs = (T*)p.cache_s + b * p.cache_s_stride[0] + kvh * p.cache_s_stride[1] + i * p.cache_s_stride[2];
+        const float decayed = round_t<T>(__fmul_rn(p.beta_pow_q, Elem<T>::to_float(*cs)));
+        *cs = Elem<T>::from_float(__fadd_rn(decayed, red));
+    } else {
+        if (!p.new_scores) return;
+        const int64_t m = i - p.S;
+        const float red = reduce_heads<T>(p.colsum, b, h0, nh, p.H, p.N, p.num_sink + p.S + m, p.head_reduction);
+        T* ns = (T*)p.new_scores + b * p.new_scores_stride[0] + kvh * p.new_scores_stride[1] +
+                m * p.new_scores_stride[2];
+        *ns = Elem<T>::from_float(red);
+    }
+}
+
+template <typename T>
+__global__ void cast_scores_kernel(const float* colsum, T* scores, int64_t s0, int64_t s1, int64_t s2, int64_t B,
+                                   int64_t H, int64_t N) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= B * H * N) return;
+    const int64_t n = idx % N, h = (idx / N) % H, b = idx / (N * H);
+    scores[b * s0 + h * s1 + n * s2] = Elem<T>::from_float(colsum[idx]);
+}
+
+template <typename T>
+int core_generic_t(const CoreProblem& p, hipStream_t stream) {
+    const int64_t rows = p.B * p.H * p.Q;
+    hipLaunchKernelGGL(fwd_generic_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
+    CKV_HIP_TRY(hipGetLastError());
+    if (p.colsum) {
+        const int64_t chunks = (p.N + CKV_WAVE - 1) / CKV_WAVE;
+        const size_t lds = (size_t)CKV_WAVE * (p.D + 1) * sizeof(float);
+        if (lds > 48 * 1024) {
+            CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(colsum_generic_kernel<T>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        }
+        hipLaunchKernelGGL(colsum_generic_kernel<T>, dim3((unsigned)(p.B * p.H * chunks)), dim3(CKV_WAVE), lds,
+                           stream, p);
+        CKV_HIP_TRY(hipGetLastError());
+    }
+    return CKV_OK;
+}
+
+}  // namespace
+
+int launch_core_generic(const CoreProblem& p, hipStream_t stream) {
+    if (p.D > kMaxD) return CKV_ERR_UNSUPPORTED;
+    switch (p.dtype) {
+        case CKV_F32: return core_generic_t<float>(p, stream);
+        case CKV_F16: return core_generic_t<__half>(p, stream);
+        case CKV_BF16: return core_generic_t<__hip_bfloat16>(p, stream);
+        default: return CKV_ERR_DTYPE;
+    }
+}
+
+int launch_cast_scores(const float* colsum, void* scores, const int64_t* stride, int64_t B, int64_t H, int64_t N,
+                       int dtype, hipStream_t stream) {
+    const dim3 grid((unsigned)((B * H * N + 255) / 256)), block(256);
+    switch (dtype) {
+        case CKV_F32:
+            hipLaunchKernelGGL(cast_scores_kernel<float>, grid, block, 0, stream, colsum, (float*)scores, stride[0],
+                               stride[1], stride[2], B, H, N);
+            break;
+        case CKV_F16:
+            hipLaunchKernelGGL(cast_scores_kernel<__half>, grid, block, 0, stream, colsum, (__half*)scores, stride[0],
+                               stride[1], stride[2], B, H, N);
+            break;
+        case CKV_BF16:
+            hipLaunchKernelGGL(cast_scores_kernel<__hip_bfloat16>, grid, block, 0, stream, colsum,
+                               (__hip_bfloat16*)scores, stride[0], stride[1], stride[2], B, H, N);
+            break;
+        default: return CKV_ERR_DTYPE;
+    }
+    CKV_HIP_TRY(hipGetLastError());
+    return CKV_OK;
+}
+
+int launch_weights(float* w_ema, float* w_new, int64_t Q, double beta, int dtype, hipStream_t stream) {
+    const dim3 grid((unsigned)((Q + 255) / 256)), block(256);
+    switch (dtype) {
+        case CKV_F32: hipLaunchKernelGGL(weights_kernel<float>, grid, block, 0, stream, w_ema, w_new, Q, beta); break;
+        case CKV_F16: hipLaunchKernelGGL(weights_kernel<__half>, grid, block, 0, stream, w_ema, w_new, Q, beta); break;
+        case CKV_BF16:
+            hipLaunchKernelGGL(weights_kernel<__hip_bfloat16>, grid, block, 0, stream, w_ema, w_new, Q, beta);
+            break;
+        default: return CKV_ERR_DTYPE;
+    }
+    CKV_HIP_TRY(hipGetLastError());
+    return CKV_OK;
+}
+
+int launch_prep_generic(const PrepProblem& p, hipStream_t stream) {
+    const ckv_attn_args& a = *p.a;
+    const int64_t half = a.D / 2;
+    const int64_t N = a.num_sink + a.S + a.Q;
+    int64_t items = a.B * a.KVH * N * half;
+    const int64_t qitems = a.B * a.H * a.Q * half;
+    if (qitems > items) items = qitems;
+    if (a.num_sink + a.S > items) items = a.num_sink + a.S;
+    const dim3 grid((unsigned)((items + 255) / 256)), block(256);
+    switch (a.dtype) {
+        case CKV_F32:
+            hipLaunchKernelGGL(prep_generic_kernel<float>, grid, block, 0, stream, a, (float*)p.qr, (float*)p.kr,
+                               (float*)p.vc, p.kmasked);
+            break;
+        case CKV_F16:
+            hipLaunchKernelGGL(prep_generic_kernel<__half>, grid, block, 0, stream, a, (__half*)p.qr, (__half*)p.kr,
+                               (__half*)p.vc, p.kmasked);
+            break;
+        case CKV_BF16:
+            hipLaunchKernelGGL(prep_generic_kernel<__hip_bfloat16>, grid, block, 0, stream, a,
+                               (__hip_bfloat16*)p.qr, (__hip_bfloat16*)p.kr, (__hip_bfloat16*)p.vc, p.kmasked);
+            break;
+        default: return CKV_ERR_DTYPE;
+    }
+    CKV_HIP_TRY(hipGetLastError());
+    return CKV_OK;
+}
+
+int launch_finish(const FinishProblem& p, hipStream_t stream) {
+    const int64_t items = p.B * p.KVH * (p.S + p.Q);
+    const dim3 grid((unsigned)((items + 255) / 256)), block(256);
+    switch (p.dtype) {
+        case CKV_F32: hipLaunchKernelGGL(finish_kernel<float>, grid, block, 0, stream, p); break;
+        case CKV_F16: hipLaunchKernelGGL(finish_kernel<__half>, grid, block, 0, stream, p); break;
+        case CKV_BF16: hipLaunchKernelGGL(finish_kernel<__hip_bfloat16>, grid, block, 0, stream, p); break;
+        default: return CKV_ERR_DTYPE;
+    }
+    CKV_HIP_TRY(hipGetLastError());
+    return CKV_OK;
+}
+
+}  // namespace ckv

@@ -1,0 +1,65 @@
+// Internal interfaces between the attention entry points and the kernel families.
+#pragma once
+
+#include "ckv_common.h"
+
+namespace ckv {
+
+// Attention over keys that are already rotated and laid out as [cached | chunk]:
+//   out[b,h,m]  = softmax_n(scale * q[b,h,m] . k[b,h/G,n] + mask) v[b,h/G,n]
+//   cached key n < n_cached is masked iff kmasked[n]; chunk key n is visible iff n-n_cached <= m
+//   colsum[b,h,n] = sum_m weight(m,n) * P[m,n]   (optional)
+//     weight = w_ema[m]                         for cached keys, and for chunk keys if !new_mode
+//     weight = w_new[m - (n - n_cached)]        for chunk keys if new_mode (m >= n - n_cached)
+struct CoreProblem {
+    const void* q;
+    int64_t q_stride[4];      // (B, H, Q, D)
+    const void* k;
+    const void* v;
+    int64_t kv_stride[4];     // (B, KVH, N, D)
+    const uint8_t* kmasked;   // (n_cached,) 1 = masked; may be null when n_cached == 0
+    void* out;
+    int64_t out_stride[4];    // (B, H, Q, D)
+    float* lse;               // (B, H, Q) natural-log normaliser of every row
+    float* colsum;            // (B, H, N) or null
+    const float* w_ema;       // (Q,)
+    const float* w_new;       // (Q,)
+    int new_mode;
+    int64_t B, H, KVH, Q, N, D;
+    float scale;
+    int dtype;
+};
+
+// fp32-math kernels for every dtype and head size (<= 256): the parity path for float32 caches
+// and the fallback for shapes the MFMA kernels do not cover.
+int launch_core_generic(const CoreProblem& p, hipStream_t stream);
+
+// weights of the score sums (cascade_attention.py:270-282, 315-317), rounded like the eager path
+int launch_weights(float* w_ema, float* w_new, int64_t Q, double beta, int dtype, hipStream_t stream);
+
+int launch_cast_scores(const float* colsum, void* scores, const int64_t* stride, int64_t B, int64_t H, int64_t N,
+                       int dtype, hipStream_t stream);
+
+struct PrepProblem {
+    const ckv_attn_args* a;
+    void* qr;        // (B, H, Q, D) rotated queries
+    void* kr;        // (B, KVH, N, D) rotated keys, [sink | cache | chunk]
+    void* vc;        // (B, KVH, N, D) values in the same order
+    uint8_t* kmasked;  // (num_sink + S,)
+};
+int launch_prep_generic(const PrepProblem& p, hipStream_t stream);
+
+struct FinishProblem {
+    const float* colsum;   // (B, H, N)
+    int64_t N;
+    void* cache_s;         // (B, KVH, S) strides below; may be null
+    int64_t cache_s_stride[3];
+    void* new_scores;      // (B, KVH, Q); may be null
+    int64_t new_scores_stride[3];
+    int64_t B, H, KVH, Q, S, num_sink;
+    float beta_pow_q;      // beta^Q rounded to fp32
+    int head_reduction, homogeneous, dtype;
+};
+int launch_finish(const FinishProblem& p, hipStream_t stream);
+
+}  // namespace ckv

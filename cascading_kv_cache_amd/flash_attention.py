@@ -1,0 +1,60 @@
+"""Drop-in for the reference operator ``attention`` (cascade/models/flash_attention.py:713).
+
+    o, scores = attention(q, k, v, causal, sm_scale, mask, beta)
+
+``q`` is ``(B, H, n_ctx, D)``; ``k``/``v`` are ``(B, H, n_kv, D)``, already rotated, expanded to the
+query heads and concatenated as ``[cached | chunk]``; ``mask`` is a 1-D bool tensor over the
+``n_kv - n_ctx`` cached keys (True = masked).  As in the reference kernel the last ``n_ctx`` keys
+are always causal, whatever ``causal`` says (flash_attention.py:55-61 never reads STAGE).
+``scores[b, h, n] = sum_m (1-beta) beta^(n_ctx-1-m) P[m, n]``: the exact value of what the
+reference kernel approximates with atomics (flash_attention.py:73-100), deterministic here.
+Forward only: the result carries no autograd graph.
+"""
+import ctypes as C
+
+import torch
+
+from . import _abi
+from .cascading_cache import _require_device, workspace
+
+
+def attention(q, k, v, causal, sm_scale, mask, beta):
+    _require_device(q, "q")
+    # the reference's shape checks (flash_attention.py:545-551)
+    HEAD_DIM_Q, HEAD_DIM_K, HEAD_DIM_V = q.shape[-1], k.shape[-1], v.shape[-1]
+    assert HEAD_DIM_Q == HEAD_DIM_K and HEAD_DIM_K == HEAD_DIM_V
+    assert HEAD_DIM_K in {16, 32, 64, 128, 256}
+    assert k.size(2) == v.size(2)
+    assert _abi.same_layout(k, v)
+    B, H, n_ctx, D = q.shape
+    n_kv = k.size(2)
+    assert n_kv >= n_ctx
+    if mask is not None:
+        assert mask.ndim == 1 and mask.numel() == n_kv - n_ctx, "mask covers exactly the cached keys"
+        mask = mask.contiguous()
+        if mask.dtype != torch.bool:
+            mask = mask != 0
+    lib = _abi.lib()
+    o = torch.empty((B, H, n_ctx, D), dtype=q.dtype, device=q.device)
+    scores = torch.empty((B, H, n_kv), dtype=q.dtype, device=q.device)
+    a = _abi.DenseArgs()
+    a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    _abi.set_strides(a.q_stride, q)
+    _abi.set_strides(a.kv_stride, k)
+    a.mask = mask.data_ptr() if mask is not None and mask.numel() > 0 else None
+    a.out = o.data_ptr()
+    _abi.set_strides(a.out_stride, o)
+    a.scores = scores.data_ptr()
+    _abi.set_strides(a.scores_stride, scores)
+    a.B, a.H, a.n_ctx, a.n_kv, a.D = B, H, n_ctx, n_kv, D
+    a.scale = float(sm_scale)
+    a.beta = float(beta)
+    a.causal = int(bool(causal))
+    a.dtype = _abi.dtype_code(q.dtype)
+    need = lib.ckv_dense_workspace_bytes(B, H, n_ctx, n_kv, D, a.dtype)
+    ws = workspace(q.device, need)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        _abi.check(lib.ckv_attn_dense(C.byref(a), C.c_void_p(stream)), "ckv_attn_dense")
+    return o, scores
