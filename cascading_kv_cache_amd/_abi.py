@@ -194,12 +194,31 @@ def lib():
         L.ckv_attn_dense.restype = C.c_int
         L.ckv_dense_workspace_bytes.argtypes = [I64, I64, I64, I64, I64, C.c_int32]
         L.ckv_dense_workspace_bytes.restype = I64
+        L.ckv_profile_enable.argtypes = [C.c_int]
+        L.ckv_profile_enable.restype = C.c_int
+        L.ckv_profile_read.argtypes = [C.POINTER(C.c_double), C.POINTER(I64)]
+        L.ckv_profile_read.restype = C.c_int
         L.ckv_strerror.argtypes = [C.c_int]
         L.ckv_strerror.restype = C.c_char_p
         L.ckv_abi_version.argtypes = []
         L.ckv_abi_version.restype = C.c_int
         _LIB = L
     return _LIB
+
+
+STAGES = ("prep", "fwd", "scores", "finish", "decode", "decode_tail", "plan", "apply")
+
+
+def profile_enable(on: bool) -> bool:
+    return bool(lib().ckv_profile_enable(int(on)))
+
+
+def profile_read():
+    """{stage: (milliseconds, launches)} accumulated since the last read (waits for the events)."""
+    ms = (C.c_double * len(STAGES))()
+    n = (I64 * len(STAGES))()
+    check(lib().ckv_profile_read(ms, n), "ckv_profile_read")
+    return {name: (ms[i], n[i]) for i, name in enumerate(STAGES)}
 
 
 def check(status: int, what: str):

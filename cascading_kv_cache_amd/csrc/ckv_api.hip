@@ -1,6 +1,58 @@
 // Entry points of libckv that are not tied to one kernel family.
 #include "ckv_common.h"
 
+#include <vector>
+
+namespace ckv {
+namespace {
+struct Span {
+    int stage;
+    hipEvent_t t0, t1;
+};
+bool g_prof_on = false;
+std::vector<Span> g_spans;
+hipEvent_t g_open[CKV_STAGE_COUNT];
+}  // namespace
+
+void prof_begin(int stage, hipStream_t stream) {
+    if (!g_prof_on) return;
+    hipEvent_t e;
+    if (hipEventCreate(&e) != hipSuccess) return;
+    (void)hipEventRecord(e, stream);
+    g_open[stage] = e;
+}
+
+void prof_end(int stage, hipStream_t stream) {
+    if (!g_prof_on || !g_open[stage]) return;
+    hipEvent_t e;
+    if (hipEventCreate(&e) != hipSuccess) return;
+    (void)hipEventRecord(e, stream);
+    g_spans.push_back(Span{stage, g_open[stage], e});
+    g_open[stage] = nullptr;
+}
+}  // namespace ckv
+
+extern "C" int ckv_profile_enable(int on) {
+    const int prev = ckv::g_prof_on ? 1 : 0;
+    ckv::g_prof_on = on != 0;
+    return prev;
+}
+
+extern "C" int ckv_profile_read(double* ms, int64_t* launches) {
+    if (!ms || !launches) return CKV_ERR_NULL;
+    for (auto& s : ckv::g_spans) {
+        float t = 0.f;
+        if (hipEventSynchronize(s.t1) == hipSuccess && hipEventElapsedTime(&t, s.t0, s.t1) == hipSuccess) {
+            ms[s.stage] += t;
+            launches[s.stage] += 1;
+        }
+        (void)hipEventDestroy(s.t0);
+        (void)hipEventDestroy(s.t1);
+    }
+    ckv::g_spans.clear();
+    return CKV_OK;
+}
+
 extern "C" const char* ckv_strerror(int status) {
     switch (status) {
         case CKV_OK: return "ok";

@@ -19,6 +19,7 @@ struct Carver {
 
 struct AttnWorkspace {
     void *qr, *kr, *vc;
+    unsigned long long* tile_vis;
     uint8_t* kmasked;
     float *lse, *colsum, *w_ema, *w_new;
     int64_t bytes;
@@ -26,12 +27,13 @@ struct AttnWorkspace {
 
 AttnWorkspace carve_attn(void* base, int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t D, int64_t NS, int64_t S,
                          int dtype) {
-    const int64_t es = elem_bytes(dtype), N = NS + S + Q;
+    const int64_t es = elem_bytes(dtype), N = NS + S + Q, n_pad = mfma_n_pad(N);
     Carver c(base);
     AttnWorkspace w;
     w.qr = c.take(B * H * Q * D * es);
-    w.kr = c.take(B * KVH * N * D * es);
-    w.vc = c.take(B * KVH * N * D * es);
+    w.kr = c.take(B * KVH * n_pad * D * es);   // padded to whole key tiles for the MFMA family
+    w.vc = c.take(B * KVH * n_pad * D * es);
+    w.tile_vis = (unsigned long long*)c.take(n_pad / 64 * 8);
     w.kmasked = (uint8_t*)c.take(NS + S);
     w.lse = (float*)c.take(B * H * Q * 4);
     w.colsum = (float*)c.take(B * H * N * 4);
@@ -81,29 +83,60 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
         rc = launch_weights(w.w_ema, w.w_new, a.Q, a.beta, a.dtype, stream);
         if (rc) return rc;
     }
-    PrepProblem pp{&a, w.qr, w.kr, w.vc, w.kmasked};
-    rc = launch_prep_generic(pp, stream);
-    if (rc) return rc;
+    const bool use_mfma = mfma_supported(a.dtype, a.D, a.H, a.KVH) && a.Q > 1;
+    if (use_mfma) {
+        MfmaProblem mp;
+        mp.seg[0] = MfmaSegment{a.sink_k, a.sink_v, {a.sink_stride[0], a.sink_stride[1], a.sink_stride[2], a.sink_stride[3]},
+                                a.sink_pos, {a.sink_pos_stride[0], a.sink_pos_stride[1]}, 0, a.sink_mask, a.num_sink};
+        mp.seg[1] = MfmaSegment{a.cache_k, a.cache_v,
+                                {a.cache_stride[0], a.cache_stride[1], a.cache_stride[2], a.cache_stride[3]},
+                                a.pos, {a.pos_stride[0], a.pos_stride[1]}, a.pos_shift, a.mask, a.S};
+        mp.seg[2] = MfmaSegment{a.k_new, a.v_new,
+                                {a.kv_new_stride[0], a.kv_new_stride[1], a.kv_new_stride[2], a.kv_new_stride[3]},
+                                a.q_pos, {0, 0}, 0, nullptr, a.Q};
+        mp.q = a.q;
+        for (int i = 0; i < 4; i++) { mp.q_stride[i] = a.q_stride[i]; mp.out_stride[i] = a.out_stride[i]; }
+        mp.q_pos = a.q_pos;
+        mp.inv_freq = a.inv_freq;
+        mp.theta = a.rope_theta;
+        mp.shared_pos = a.sink_pos_stride[0] == 0 && a.sink_pos_stride[1] == 0 && a.pos_stride[0] == 0 &&
+                        a.pos_stride[1] == 0;
+        mp.qr = w.qr; mp.kr = w.kr; mp.vt = w.vc; mp.tile_vis = w.tile_vis;
+        mp.out = a.out;
+        mp.lse = w.lse;
+        mp.colsum = want_scores ? w.colsum : nullptr;
+        mp.w_ema = w.w_ema; mp.w_new = w.w_new;
+        mp.new_mode = 1;
+        mp.B = a.B; mp.H = a.H; mp.KVH = a.KVH; mp.Q = a.Q; mp.n = N; mp.n_pad = mfma_n_pad(N);
+        mp.scale = a.scale;
+        mp.dtype = a.dtype;
+        rc = launch_mfma(mp, stream);
+        if (rc) return rc;
+    } else {
+        PrepProblem pp{&a, w.qr, w.kr, w.vc, w.kmasked};
+        rc = launch_prep_generic(pp, stream);
+        if (rc) return rc;
 
-    CoreProblem cp;
-    cp.q = w.qr;
-    contiguous_strides(cp.q_stride, a.H, a.Q, a.D);
-    cp.k = w.kr;
-    cp.v = w.vc;
-    contiguous_strides(cp.kv_stride, a.KVH, N, a.D);
-    cp.kmasked = (a.num_sink + a.S) > 0 ? w.kmasked : nullptr;
-    cp.out = a.out;
-    for (int i = 0; i < 4; i++) cp.out_stride[i] = a.out_stride[i];
-    cp.lse = w.lse;
-    cp.colsum = want_scores ? w.colsum : nullptr;
-    cp.w_ema = w.w_ema;
-    cp.w_new = w.w_new;
-    cp.new_mode = 1;
-    cp.B = a.B; cp.H = a.H; cp.KVH = a.KVH; cp.Q = a.Q; cp.N = N; cp.D = a.D;
-    cp.scale = a.scale;
-    cp.dtype = a.dtype;
-    rc = launch_core_generic(cp, stream);
-    if (rc) return rc;
+        CoreProblem cp;
+        cp.q = w.qr;
+        contiguous_strides(cp.q_stride, a.H, a.Q, a.D);
+        cp.k = w.kr;
+        cp.v = w.vc;
+        contiguous_strides(cp.kv_stride, a.KVH, N, a.D);
+        cp.kmasked = (a.num_sink + a.S) > 0 ? w.kmasked : nullptr;
+        cp.out = a.out;
+        for (int i = 0; i < 4; i++) cp.out_stride[i] = a.out_stride[i];
+        cp.lse = w.lse;
+        cp.colsum = want_scores ? w.colsum : nullptr;
+        cp.w_ema = w.w_ema;
+        cp.w_new = w.w_new;
+        cp.new_mode = 1;
+        cp.B = a.B; cp.H = a.H; cp.KVH = a.KVH; cp.Q = a.Q; cp.N = N; cp.D = a.D;
+        cp.scale = a.scale;
+        cp.dtype = a.dtype;
+        rc = launch_core_generic(cp, stream);
+        if (rc) return rc;
+    }
     if (a.lse) {
         CKV_HIP_TRY(hipMemcpyAsync(a.lse, w.lse, a.B * a.H * a.Q * sizeof(float), hipMemcpyDeviceToDevice, stream));
     }

@@ -297,7 +297,10 @@ __global__ void cast_scores_kernel(const float* colsum, T* scores, int64_t s0, i
 template <typename T>
 int core_generic_t(const CoreProblem& p, hipStream_t stream) {
     const int64_t rows = p.B * p.H * p.Q;
-    hipLaunchKernelGGL(fwd_generic_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
+    {
+        StageScope sc(CKV_STAGE_FWD, stream);
+        hipLaunchKernelGGL(fwd_generic_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
+    }
     CKV_HIP_TRY(hipGetLastError());
     if (p.colsum) {
         const int64_t chunks = (p.N + CKV_WAVE - 1) / CKV_WAVE;
@@ -306,8 +309,11 @@ int core_generic_t(const CoreProblem& p, hipStream_t stream) {
             CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(colsum_generic_kernel<T>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         }
-        hipLaunchKernelGGL(colsum_generic_kernel<T>, dim3((unsigned)(p.B * p.H * chunks)), dim3(CKV_WAVE), lds,
-                           stream, p);
+        {
+            StageScope sc(CKV_STAGE_SCORES, stream);
+            hipLaunchKernelGGL(colsum_generic_kernel<T>, dim3((unsigned)(p.B * p.H * chunks)), dim3(CKV_WAVE), lds,
+                               stream, p);
+        }
         CKV_HIP_TRY(hipGetLastError());
     }
     return CKV_OK;
@@ -362,6 +368,7 @@ int launch_weights(float* w_ema, float* w_new, int64_t Q, double beta, int dtype
 }
 
 int launch_prep_generic(const PrepProblem& p, hipStream_t stream) {
+    StageScope sc(CKV_STAGE_PREP, stream);
     const ckv_attn_args& a = *p.a;
     const int64_t half = a.D / 2;
     const int64_t N = a.num_sink + a.S + a.Q;
@@ -390,6 +397,7 @@ int launch_prep_generic(const PrepProblem& p, hipStream_t stream) {
 }
 
 int launch_finish(const FinishProblem& p, hipStream_t stream) {
+    StageScope sc(CKV_STAGE_FINISH, stream);
     const int64_t items = p.B * p.KVH * (p.S + p.Q);
     const dim3 grid((unsigned)((items + 255) / 256)), block(256);
     switch (p.dtype) {

@@ -62,4 +62,42 @@ struct FinishProblem {
 };
 int launch_finish(const FinishProblem& p, hipStream_t stream);
 
+// ---- bf16/fp16 MFMA family (head_dim 128) ----
+struct MfmaSegment {
+    const void* k;
+    const void* v;
+    int64_t stride[4];     // (B, KVH, len, D)
+    const int64_t* pos;    // null: keys are already rotated
+    int64_t pos_stride[2];
+    int64_t pos_shift;
+    const uint8_t* masked; // null: all visible
+    int64_t len;
+};
+
+struct MfmaProblem {
+    MfmaSegment seg[3];    // keys in order; the LAST Q keys overall are the causal chunk
+    const void* q;
+    int64_t q_stride[4];
+    const int64_t* q_pos;  // null: queries are already rotated
+    const float* inv_freq;
+    float theta;
+    int shared_pos;
+    void *qr, *kr, *vt;
+    unsigned long long* tile_vis;
+    void* out;
+    int64_t out_stride[4];
+    float* lse;
+    float* colsum;         // (B, H, n) or null
+    const float* w_ema;
+    const float* w_new;
+    int new_mode;
+    int64_t B, H, KVH, Q, n, n_pad;
+    float scale;
+    int dtype;
+};
+
+bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH);
+int64_t mfma_n_pad(int64_t n);
+int launch_mfma(const MfmaProblem& p, hipStream_t stream);
+
 }  // namespace ckv

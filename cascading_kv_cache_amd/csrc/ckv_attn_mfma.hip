@@ -1,0 +1,687 @@
+// bf16 / fp16 MFMA attention for head_dim 128 on gfx950 (CDNA4, wave64, v_mfma_f32_32x32x16).
+//
+// Stages (all stream-ordered):
+//   stage_keys   rotate K on the way into a padded row-major buffer Kr, transpose V into 64-key
+//                tiles Vt[tile][d][key'] (key' = the order the PV MFMA consumes), build one 64-bit
+//                visibility word per key tile.  cos/sin are computed once per key and reused for
+//                every (batch, kv-head) that shares the position row.
+//   stage_q      rotate Q.
+//   fwd          flash forward.  One workgroup = one kv head x 256 (head, position) rows, so the G
+//                query heads of a group share every K/V tile staged in LDS.  S^T = K Q^T keeps a
+//                query in one lane pair: the row max / sum need a single cross-half exchange and
+//                exp(S^T) is already laid out as the B operand of O^T += V^T P^T.
+//   colsum       exact score sums.  One workgroup = one kv head x 256 keys held in registers;
+//                the queries stream through LDS, P = exp(S - lse) with the final normaliser, and
+//                the weighted column sums stay inside a lane (S = Q K^T orientation).
+#include "ckv_attn_internal.h"
+
+namespace ckv {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kD = 128;    // head dim
+constexpr int kBN = 64;    // keys per tile
+constexpr int kKP = kD + 8;   // LDS pitch of a K / Q row (elements): 16-byte reads stay conflict-free
+constexpr int kVP = kBN + 8;  // LDS pitch of a V^T row
+constexpr int kRows = 256;    // (head, position) rows per forward workgroup
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<__hip_bfloat16> {
+    __device__ static f32x16 mma(uint4 a, uint4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                       0, 0, 0);
+    }
+    __device__ static uint32_t pack2(float lo, float hi) {
+        f32x2 f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+    }
+    __device__ static float round1(float v) {
+        f32x2 f = {v, 0.f};
+        const uint32_t u = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+        return __uint_as_float(u << 16);
+    }
+};
+template <>
+struct Mma<__half> {
+    __device__ static f32x16 mma(uint4 a, uint4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                      0, 0);
+    }
+    __device__ static uint32_t pack2(float lo, float hi) {
+        f32x2 f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+    }
+    __device__ static float round1(float v) { return (float)(_Float16)v; }
+};
+
+// position of key `k` (0..63) of a tile inside a V^T row: the PV contraction step s covers keys
+// 16s..16s+15; lane half h supplies keys 16s + 8a + 4h + e (a = 0,1; e = 0..3) as elements 4a+e
+__host__ __device__ inline int vt_slot(int k) {
+    const int s = k >> 4, a = (k >> 3) & 1, h = (k >> 2) & 1, e = k & 3;
+    return 16 * s + 8 * h + 4 * a + e;
+}
+
+// ---------------------------------------------------------------------------------------------
+// staging
+// ---------------------------------------------------------------------------------------------
+struct KeySegment {
+    const void* k;
+    const void* v;
+    int64_t stride[4];       // (B, KVH, len, D)
+    const int64_t* pos;      // position ids, or null when keys are already rotated
+    int64_t pos_stride[2];
+    int64_t pos_shift;
+    const uint8_t* masked;   // 1 = masked, or null (all visible)
+    int64_t len;
+};
+
+struct StageParams {
+    KeySegment seg[3];
+    const float* inv_freq;
+    float theta;
+    int shared_pos;          // every (b, kvh) uses position row [0, 0]
+    void* kr;                // (B*KVH, n_pad, D)
+    void* vt;                // (B*KVH, n_pad/64, D, 64)
+    unsigned long long* tile_vis;  // (n_pad/64,)
+    int64_t B, KVH, n, n_pad;
+};
+
+__device__ inline int find_segment(const StageParams& p, int64_t n, int64_t& local) {
+    if (n < p.seg[0].len) { local = n; return 0; }
+    n -= p.seg[0].len;
+    if (n < p.seg[1].len) { local = n; return 1; }
+    local = n - p.seg[1].len;
+    return 2;
+}
+
+// grid (n_pad/64, splits); 256 threads: thread = (key = tid/4, quarter = tid%4) owns rotation pairs
+// j = 16*quarter .. 16*quarter+15, i.e. elements [16q,16q+16) and [64+16q, 64+16q+16) of its row.
+template <typename T>
+__global__ void __launch_bounds__(256) stage_keys_kernel(StageParams p) {
+    __shared__ T v_lds[kBN][kD + 2];
+    const int tid = threadIdx.x;
+    const int key = tid >> 2, quarter = tid & 3;
+    const int64_t tile = blockIdx.x;
+    const int64_t n = tile * kBN + key;
+    int64_t local = 0;
+    const int sidx = n < p.n ? find_segment(p, n, local) : -1;
+
+    if (blockIdx.y == 0 && tid < kBN) {  // visibility word of this tile
+        const int64_t nn = tile * kBN + tid;
+        bool vis = nn < p.n;
+        if (vis) {
+            int64_t loc;
+            const int si = find_segment(p, nn, loc);
+            if (p.seg[si].masked) vis = p.seg[si].masked[loc] == 0;
+        }
+        const unsigned long long bal = __ballot(vis);
+        if (tid == 0) p.tile_vis[tile] = bal;
+    }
+
+    float cs[16], sn[16];
+    const bool rotate = sidx >= 0 && p.seg[sidx].pos != nullptr;
+    if (rotate && p.shared_pos) {
+        const int64_t pos = p.seg[sidx].pos[local] + p.seg[sidx].pos_shift;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int j = 16 * quarter + i;
+            const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
+            sincosf(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
+        }
+    }
+    const int64_t nbh = p.B * p.KVH;
+    for (int64_t bh = blockIdx.y; bh < nbh; bh += gridDim.y) {
+        const int64_t b = bh / p.KVH, kvh = bh % p.KVH;
+        uint4 lo[2], hi[2], vlo[2], vhi[2];
+        lo[0] = lo[1] = hi[0] = hi[1] = vlo[0] = vlo[1] = vhi[0] = vhi[1] = make_uint4(0, 0, 0, 0);
+        if (sidx >= 0) {
+            const KeySegment& sg = p.seg[sidx];
+            const int64_t off = b * sg.stride[0] + kvh * sg.stride[1] + local * sg.stride[2];
+            const T* kp = (const T*)sg.k + off;
+            const T* vp = (const T*)sg.v + off;
+            if (sg.stride[3] == 1 && ((reinterpret_cast<uintptr_t>(kp) | reinterpret_cast<uintptr_t>(vp)) & 15) == 0) {
+                lo[0] = *reinterpret_cast<const uint4*>(kp + 16 * quarter);
+                lo[1] = *reinterpret_cast<const uint4*>(kp + 16 * quarter + 8);
+                hi[0] = *reinterpret_cast<const uint4*>(kp + 64 + 16 * quarter);
+                hi[1] = *reinterpret_cast<const uint4*>(kp + 64 + 16 * quarter + 8);
+                vlo[0] = *reinterpret_cast<const uint4*>(vp + 16 * quarter);
+                vlo[1] = *reinterpret_cast<const uint4*>(vp + 16 * quarter + 8);
+                vhi[0] = *reinterpret_cast<const uint4*>(vp + 64 + 16 * quarter);
+                vhi[1] = *reinterpret_cast<const uint4*>(vp + 64 + 16 * quarter + 8);
+            } else {
+                T* l0 = reinterpret_cast<T*>(lo);
+                T* h0 = reinterpret_cast<T*>(hi);
+                T* vl = reinterpret_cast<T*>(vlo);
+                T* vh = reinterpret_cast<T*>(vhi);
+                for (int i = 0; i < 16; i++) {
+                    l0[i] = kp[(16 * quarter + i) * sg.stride[3]];
+                    h0[i] = kp[(64 + 16 * quarter + i) * sg.stride[3]];
+                    vl[i] = vp[(16 * quarter + i) * sg.stride[3]];
+                    vh[i] = vp[(64 + 16 * quarter + i) * sg.stride[3]];
+                }
+            }
+            if (rotate) {
+                if (!p.shared_pos) {
+                    const int64_t pos = sg.pos[b * sg.pos_stride[0] + kvh * sg.pos_stride[1] + local] + sg.pos_shift;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int j = 16 * quarter + i;
+                        const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
+                        sincosf(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
+                    }
+                }
+                T* l0 = reinterpret_cast<T*>(lo);
+                T* h0 = reinterpret_cast<T*>(hi);
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const float x1 = Elem<T>::to_float(l0[i]), x2 = Elem<T>::to_float(h0[i]);
+                    l0[i] = Elem<T>::from_float(x1 * cs[i] - x2 * sn[i]);
+                    h0[i] = Elem<T>::from_float(x2 * cs[i] + x1 * sn[i]);
+                }
+            }
+        }
+        T* krow = (T*)p.kr + (bh * p.n_pad + n) * kD;
+        *reinterpret_cast<uint4*>(krow + 16 * quarter) = lo[0];
+        *reinterpret_cast<uint4*>(krow + 16 * quarter + 8) = lo[1];
+        *reinterpret_cast<uint4*>(krow + 64 + 16 * quarter) = hi[0];
+        *reinterpret_cast<uint4*>(krow + 64 + 16 * quarter + 8) = hi[1];
+
+        // V: through LDS into the transposed tile
+        __syncthreads();
+        {
+            const T* vl = reinterpret_cast<const T*>(vlo);
+            const T* vh = reinterpret_cast<const T*>(vhi);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                v_lds[key][16 * quarter + i] = vl[i];
+                v_lds[key][64 + 16 * quarter + i] = vh[i];
+            }
+        }
+        __syncthreads();
+        T* vt = (T*)p.vt + (bh * (p.n_pad / kBN) + tile) * (int64_t)(kD * kBN);
+        // thread -> (d = tid/2, half of the 64 slots): 32 slots = 4 x 16 bytes
+        {
+            const int d = tid >> 1, sh = (tid & 1) * 32;
+            T tmp[32];
+#pragma unroll
+            for (int sl = 0; sl < 32; sl++) {
+                const int slot = sh + sl;
+                // inverse of vt_slot: slot = 16s + 8h + 4a + e  ->  key = 16s + 8a + 4h + e
+                const int s = slot >> 4, h = (slot >> 3) & 1, a = (slot >> 2) & 1, e = slot & 3;
+                tmp[sl] = v_lds[16 * s + 8 * a + 4 * h + e][d];
+            }
+            uint4* dst = reinterpret_cast<uint4*>(vt + d * kBN + sh);
+            const uint4* src = reinterpret_cast<const uint4*>(tmp);
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[i] = src[i];
+        }
+    }
+}
+
+struct StageQParams {
+    const void* q;
+    int64_t stride[4];
+    const int64_t* q_pos;    // null: copy only
+    const float* inv_freq;
+    float theta;
+    void* qr;                // (B*H, Q, D) contiguous
+    int64_t rows;            // B*H*Q
+    int64_t H, Q;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) stage_q_kernel(StageQParams p) {
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t row = idx >> 2;
+    const int quarter = idx & 3;
+    if (row >= p.rows) return;
+    const int64_t m = row % p.Q, h = (row / p.Q) % p.H, b = row / (p.Q * p.H);
+    const T* src = (const T*)p.q + b * p.stride[0] + h * p.stride[1] + m * p.stride[2];
+    T lo[16], hi[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        lo[i] = src[(16 * quarter + i) * p.stride[3]];
+        hi[i] = src[(64 + 16 * quarter + i) * p.stride[3]];
+    }
+    if (p.q_pos) {
+        const int64_t pos = p.q_pos[m];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int j = 16 * quarter + i;
+            const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
+            float sn, cs;
+            sincosf(__fmul_rn((float)pos, f), &sn, &cs);
+            const float x1 = Elem<T>::to_float(lo[i]), x2 = Elem<T>::to_float(hi[i]);
+            lo[i] = Elem<T>::from_float(x1 * cs - x2 * sn);
+            hi[i] = Elem<T>::from_float(x2 * cs + x1 * sn);
+        }
+    }
+    T* dst = (T*)p.qr + row * kD;
+    *reinterpret_cast<uint4*>(dst + 16 * quarter) = reinterpret_cast<uint4*>(lo)[0];
+    *reinterpret_cast<uint4*>(dst + 16 * quarter + 8) = reinterpret_cast<uint4*>(lo)[1];
+    *reinterpret_cast<uint4*>(dst + 64 + 16 * quarter) = reinterpret_cast<uint4*>(hi)[0];
+    *reinterpret_cast<uint4*>(dst + 64 + 16 * quarter + 8) = reinterpret_cast<uint4*>(hi)[1];
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------------------------
+struct FwdParams {
+    const void* qr;   // (B*H, Q, D)
+    const void* kr;   // (B*KVH, n_pad, D)
+    const void* vt;   // (B*KVH, n_pad/64, D, 64)
+    const unsigned long long* tile_vis;
+    void* out;
+    int64_t out_stride[4];
+    float* lse;       // (B*H, Q)
+    int64_t B, H, KVH, Q, N, Nc, n_pad;
+    int G, QT;        // heads per kv head, positions per workgroup (G * QT <= 256)
+    float scale_log2; // softmax scale * log2(e)
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) fwd_mfma_kernel(FwdParams p) {
+    __shared__ __align__(16) T k_lds[kBN * kKP];
+    __shared__ __align__(16) T v_lds[kD * kVP];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int col = lane & 31, half = lane >> 5;
+    const int64_t bkv = blockIdx.y;
+    const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
+    const int64_t m0 = (int64_t)blockIdx.x * p.QT;
+
+    // the two query rows (one per 32-row subtile) this lane owns as MFMA column `col`
+    int64_t row_m[2], row_h[2];
+    bool row_ok[2];
+    uint4 qreg[2][8];
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const int r = wave * 64 + c * 32 + col;
+        const int g = r / p.QT, mloc = r % p.QT;
+        row_m[c] = m0 + mloc;
+        row_h[c] = kvh * p.G + g;
+        row_ok[c] = g < p.G && row_m[c] < p.Q;
+        const T* qrow = (const T*)p.qr + ((b * p.H + row_h[c]) * p.Q + row_m[c]) * kD;
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++) {
+            qreg[c][kk] = row_ok[c] ? *reinterpret_cast<const uint4*>(qrow + 16 * kk + 8 * half) : make_uint4(0, 0, 0, 0);
+        }
+    }
+
+    f32x16 oacc[4][2];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) oacc[dt][c][v] = 0.f;
+    float m_run[2] = {-INFINITY, -INFINITY};
+    float l_run[2] = {0.f, 0.f};  // partial over this lane's keys; halves are added at the end
+
+    int64_t m_hi = m0 + p.QT - 1;
+    if (m_hi > p.Q - 1) m_hi = p.Q - 1;
+    const int64_t n_tiles = (p.Nc + m_hi) / kBN + 1;
+    const T* kbase = (const T*)p.kr + bkv * p.n_pad * kD;
+    const T* vbase = (const T*)p.vt + bkv * p.n_pad * kD;
+
+    for (int64_t t = 0; t < n_tiles; t++) {
+        const unsigned long long vis = p.tile_vis[t];
+        if (vis == 0ull) continue;  // uniform: every key of the tile is masked
+        __syncthreads();            // previous tile fully consumed
+        {   // 64 x 128 K rows and 128 x 64 V^T rows, 16 bytes per thread per pass
+            const T* kt = kbase + t * (int64_t)(kBN * kD);
+            const T* vtile = vbase + t * (int64_t)(kBN * kD);
+#pragma unroll
+            for (int it = 0; it < 4; it++) {
+                const int chunk = it * 256 + tid;       // 0..1023
+                const int kr_ = chunk >> 4, kc = chunk & 15;  // K: 16 chunks per row
+                *reinterpret_cast<uint4*>(&k_lds[kr_ * kKP + kc * 8]) =
+                    *reinterpret_cast<const uint4*>(kt + kr_ * kD + kc * 8);
+                const int vr = chunk >> 3, vc = chunk & 7;    // V^T: 8 chunks per row
+                *reinterpret_cast<uint4*>(&v_lds[vr * kVP + vc * 8]) =
+                    *reinterpret_cast<const uint4*>(vtile + vr * kBN + vc * 8);
+            }
+        }
+        __syncthreads();
+
+        // S^T tile: sacc[ks][c][v] = logit of key 32ks + 8(v/4) + 4half + v%4 for query column col
+        f32x16 sacc[2][2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) sacc[ks][c][v] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                const uint4 a = *reinterpret_cast<const uint4*>(&k_lds[(32 * ks + col) * kKP + 16 * kk + 8 * half]);
+                sacc[ks][0] = Mma<T>::mma(a, qreg[0][kk], sacc[ks][0]);
+                sacc[ks][1] = Mma<T>::mma(a, qreg[1][kk], sacc[ks][1]);
+            }
+        }
+
+        // masking is needed only on tiles with hidden keys or tiles that reach past the diagonal
+        const int64_t key0 = t * kBN;
+        const bool need_mask = (vis != ~0ull) || (key0 + kBN - 1 - p.Nc > m0);
+        uint32_t pk[2][4][4];  // P^T as MFMA B operands: [query subtile][step][4 x 2 elements]
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    float s = sacc[ks][c][v] * p.scale_log2;
+                    if (need_mask) {
+                        const int kidx = 32 * ks + 8 * (v >> 2) + 4 * half + (v & 3);
+                        const int64_t n = key0 + kidx;
+                        const bool ok = ((vis >> kidx) & 1ull) && (n < p.Nc || n - p.Nc <= row_m[c]);
+                        s = ok ? s : -INFINITY;
+                    }
+                    sacc[ks][c][v] = s;
+                    mx = fmaxf(mx, s);
+                }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run[c], mx);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run[c] - m_use);
+            m_run[c] = m_new;
+            float rs = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+                for (int v = 0; v < 16; v += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(sacc[ks][c][v] - m_use);
+                    const float p1 = __builtin_amdgcn_exp2f(sacc[ks][c][v + 1] - m_use);
+                    rs += p0 + p1;
+                    // step = 2ks + v/8, element = v%8
+                    pk[c][2 * ks + (v >> 3)][(v & 7) >> 1] = Mma<T>::pack2(p0, p1);
+                }
+            }
+            l_run[c] = l_run[c] * alpha + rs;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) oacc[dt][c][v] *= alpha;
+        }
+
+        // O^T += V^T P^T
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const uint4 a = *reinterpret_cast<const uint4*>(&v_lds[(32 * dt + col) * kVP + 16 * s + 8 * half]);
+                const uint4 b0 = make_uint4(pk[0][s][0], pk[0][s][1], pk[0][s][2], pk[0][s][3]);
+                const uint4 b1 = make_uint4(pk[1][s][0], pk[1][s][1], pk[1][s][2], pk[1][s][3]);
+                oacc[dt][0] = Mma<T>::mma(a, b0, oacc[dt][0]);
+                oacc[dt][1] = Mma<T>::mma(a, b1, oacc[dt][1]);
+            }
+        }
+    }
+
+    // epilogue: lane owns d = 32dt + 8(v/4) + 4half + v%4 of its query row
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const float l_tot = l_run[c] + __shfl_xor(l_run[c], 32);
+        if (!row_ok[c]) continue;
+        const float inv = 1.f / l_tot;
+        T* orow = (T*)p.out + b * p.out_stride[0] + row_h[c] * p.out_stride[1] + row_m[c] * p.out_stride[2];
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+#pragma unroll
+            for (int v4 = 0; v4 < 4; v4++) {
+                const int d = 32 * dt + 8 * v4 + 4 * half;
+                if (p.out_stride[3] == 1) {
+                    uint2 w;
+                    w.x = Mma<T>::pack2(oacc[dt][c][4 * v4] * inv, oacc[dt][c][4 * v4 + 1] * inv);
+                    w.y = Mma<T>::pack2(oacc[dt][c][4 * v4 + 2] * inv, oacc[dt][c][4 * v4 + 3] * inv);
+                    *reinterpret_cast<uint2*>(orow + d) = w;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        orow[(d + e) * p.out_stride[3]] = Elem<T>::from_float(oacc[dt][c][4 * v4 + e] * inv);
+                }
+            }
+        }
+        if (half == 0) {
+            p.lse[(b * p.H + row_h[c]) * p.Q + row_m[c]] = (m_run[c] + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// score sums
+// ---------------------------------------------------------------------------------------------
+struct ColsumParams {
+    const void* qr;
+    const void* kr;
+    const unsigned long long* tile_vis;
+    const float* lse;     // natural log
+    const float* w_ema;
+    const float* w_new;
+    float* colsum;        // (B*H, N)
+    int64_t B, H, KVH, Q, N, Nc, n_pad;
+    int G;
+    int new_mode;
+    float scale_log2;
+};
+
+constexpr int kQT2 = 64;  // query rows per LDS tile of the column pass
+
+template <typename T>
+__global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
+    __shared__ __align__(16) T q_lds[kQT2 * kKP];
+    __shared__ float lse_lds[kQT2];
+    __shared__ float w_lds[kQT2];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int col = lane & 31, half = lane >> 5;
+    const int64_t bkv = blockIdx.y;
+    const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
+    const int64_t key_blk = (int64_t)blockIdx.x * 256;   // first key of the workgroup
+    const int64_t key_w = key_blk + wave * 64;            // first key of this wave
+
+    // K as the B operand: lane (col, half) holds key key_w + 32ks + col, elements 16kk + 8half ..
+    uint4 kreg[2][8];
+    const T* kbase = (const T*)p.kr + bkv * p.n_pad * kD;
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        const int64_t n = key_w + 32 * ks + col;
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++) {
+            kreg[ks][kk] = n < p.n_pad ? *reinterpret_cast<const uint4*>(kbase + n * kD + 16 * kk + 8 * half)
+                                       : make_uint4(0, 0, 0, 0);
+        }
+    }
+    bool live[2];
+    int64_t nrel[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        const int64_t n = key_w + 32 * ks + col;
+        live[ks] = n < p.N && ((p.tile_vis[n / kBN] >> (n % kBN)) & 1ull);
+        nrel[ks] = n - p.Nc;
+    }
+    // first query row that can see any key of the workgroup
+    int64_t m_first = key_blk - p.Nc;
+    if (m_first < 0) m_first = 0;
+    m_first = m_first / kQT2 * kQT2;
+    const bool chunk_keys = key_blk + 255 >= p.Nc;  // some key of the workgroup belongs to the chunk
+    const float kLog2e = 1.4426950408889634f;
+
+    for (int g = 0; g < p.G; g++) {
+        const int64_t h = kvh * p.G + g;
+        const T* qbase = (const T*)p.qr + (b * p.H + h) * p.Q * kD;
+        const float* lse = p.lse + (b * p.H + h) * p.Q;
+        float acc[2] = {0.f, 0.f};
+        for (int64_t mt = m_first; mt < p.Q; mt += kQT2) {
+            __syncthreads();
+#pragma unroll
+            for (int it = 0; it < 4; it++) {
+                const int chunk = it * 256 + tid;
+                const int r = chunk >> 4, cc = chunk & 15;
+                const int64_t m = mt + r;
+                *reinterpret_cast<uint4*>(&q_lds[r * kKP + cc * 8]) =
+                    m < p.Q ? *reinterpret_cast<const uint4*>(qbase + m * kD + cc * 8) : make_uint4(0, 0, 0, 0);
+            }
+            if (tid < kQT2) {
+                const int64_t m = mt + tid;
+                lse_lds[tid] = m < p.Q ? lse[m] * kLog2e : INFINITY;  // +inf -> P = 0 for padding rows
+                w_lds[tid] = m < p.Q ? p.w_ema[m] : 0.f;
+            }
+            __syncthreads();
+            f32x16 sacc[2][2];  // [c = query subtile][ks]
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) sacc[c][ks][v] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 8; kk++) {
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    const uint4 a = *reinterpret_cast<const uint4*>(&q_lds[(32 * c + col) * kKP + 16 * kk + 8 * half]);
+                    sacc[c][0] = Mma<T>::mma(a, kreg[0][kk], sacc[c][0]);
+                    sacc[c][1] = Mma<T>::mma(a, kreg[1][kk], sacc[c][1]);
+                }
+            }
+            // element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4, key column of this lane
+            const bool diag = chunk_keys && (mt < key_blk + 256 - p.Nc);  // tile may cross the diagonal
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int r = 32 * c + 8 * (v >> 2) + 4 * half + (v & 3);
+                    const float l2 = lse_lds[r];
+#pragma unroll
+                    for (int ks = 0; ks < 2; ks++) {
+                        float pe = __builtin_amdgcn_exp2f(sacc[c][ks][v] * p.scale_log2 - l2);
+                        pe = Mma<T>::round1(pe);
+                        if (chunk_keys && nrel[ks] >= 0) {
+                            const int64_t m = mt + r;
+                            if (diag && m < nrel[ks]) pe = 0.f;
+                            if (p.new_mode) {
+                                const int64_t k = m - nrel[ks];
+                                const float w = (k >= 0 && m < p.Q) ? p.w_new[k] : 0.f;
+                                acc[ks] += Mma<T>::round1(pe * w);
+                            } else {
+                                acc[ks] = fmaf(w_lds[r], pe, acc[ks]);
+                            }
+                        } else {
+                            acc[ks] = fmaf(w_lds[r], pe, acc[ks]);
+                        }
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+            const float tot = acc[ks] + __shfl_xor(acc[ks], 32);
+            const int64_t n = key_w + 32 * ks + col;
+            if (half == 0 && n < p.N) p.colsum[(b * p.H + h) * p.N + n] = live[ks] ? tot : 0.f;
+        }
+    }
+}
+
+template <typename T>
+int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
+    const int64_t n = mp.n, n_pad = mp.n_pad;
+    {
+        StageScope sc(CKV_STAGE_PREP, stream);
+        StageParams sp;
+        for (int i = 0; i < 3; i++) {
+            sp.seg[i].k = mp.seg[i].k;
+            sp.seg[i].v = mp.seg[i].v;
+            for (int j = 0; j < 4; j++) sp.seg[i].stride[j] = mp.seg[i].stride[j];
+            sp.seg[i].pos = mp.seg[i].pos;
+            sp.seg[i].pos_stride[0] = mp.seg[i].pos_stride[0];
+            sp.seg[i].pos_stride[1] = mp.seg[i].pos_stride[1];
+            sp.seg[i].pos_shift = mp.seg[i].pos_shift;
+            sp.seg[i].masked = mp.seg[i].masked;
+            sp.seg[i].len = mp.seg[i].len;
+        }
+        sp.inv_freq = mp.inv_freq;
+        sp.theta = mp.theta;
+        sp.shared_pos = mp.shared_pos;
+        sp.kr = mp.kr;
+        sp.vt = mp.vt;
+        sp.tile_vis = mp.tile_vis;
+        sp.B = mp.B; sp.KVH = mp.KVH; sp.n = n; sp.n_pad = n_pad;
+        const int64_t nbh = mp.B * mp.KVH;
+        int64_t splits = mp.shared_pos ? (nbh < 4 ? nbh : 4) : nbh;
+        if (splits > 65535) splits = 65535;
+        hipLaunchKernelGGL(stage_keys_kernel<T>, dim3((unsigned)(n_pad / kBN), (unsigned)splits), dim3(256), 0, stream,
+                           sp);
+        CKV_HIP_TRY(hipGetLastError());
+        StageQParams sq;
+        sq.q = mp.q;
+        for (int j = 0; j < 4; j++) sq.stride[j] = mp.q_stride[j];
+        sq.q_pos = mp.q_pos;
+        sq.inv_freq = mp.inv_freq;
+        sq.theta = mp.theta;
+        sq.qr = mp.qr;
+        sq.rows = mp.B * mp.H * mp.Q;
+        sq.H = mp.H; sq.Q = mp.Q;
+        hipLaunchKernelGGL(stage_q_kernel<T>, dim3((unsigned)((sq.rows * 4 + 255) / 256)), dim3(256), 0, stream, sq);
+        CKV_HIP_TRY(hipGetLastError());
+    }
+    const int G = (int)(mp.H / mp.KVH);
+    const float scale_log2 = mp.scale * 1.4426950408889634f;
+    {
+        StageScope sc(CKV_STAGE_FWD, stream);
+        FwdParams fp;
+        fp.qr = mp.qr; fp.kr = mp.kr; fp.vt = mp.vt; fp.tile_vis = mp.tile_vis;
+        fp.out = mp.out;
+        for (int j = 0; j < 4; j++) fp.out_stride[j] = mp.out_stride[j];
+        fp.lse = mp.lse;
+        fp.B = mp.B; fp.H = mp.H; fp.KVH = mp.KVH; fp.Q = mp.Q; fp.N = n; fp.Nc = n - mp.Q; fp.n_pad = n_pad;
+        fp.G = G;
+        fp.QT = kRows / G;
+        fp.scale_log2 = scale_log2;
+        const dim3 grid((unsigned)((mp.Q + fp.QT - 1) / fp.QT), (unsigned)(mp.B * mp.KVH));
+        hipLaunchKernelGGL(fwd_mfma_kernel<T>, grid, dim3(256), 0, stream, fp);
+        CKV_HIP_TRY(hipGetLastError());
+    }
+    if (mp.colsum) {
+        StageScope sc(CKV_STAGE_SCORES, stream);
+        ColsumParams cp;
+        cp.qr = mp.qr; cp.kr = mp.kr; cp.tile_vis = mp.tile_vis; cp.lse = mp.lse;
+        cp.w_ema = mp.w_ema; cp.w_new = mp.w_new; cp.colsum = mp.colsum;
+        cp.B = mp.B; cp.H = mp.H; cp.KVH = mp.KVH; cp.Q = mp.Q; cp.N = n; cp.Nc = n - mp.Q; cp.n_pad = n_pad;
+        cp.G = G;
+        cp.new_mode = mp.new_mode;
+        cp.scale_log2 = scale_log2;
+        const dim3 grid((unsigned)((n + 255) / 256), (unsigned)(mp.B * mp.KVH));
+        hipLaunchKernelGGL(colsum_mfma_kernel<T>, grid, dim3(256), 0, stream, cp);
+        CKV_HIP_TRY(hipGetLastError());
+    }
+    return CKV_OK;
+}
+
+}  // namespace
+
+bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH) {
+    if (dtype != CKV_BF16 && dtype != CKV_F16) return false;
+    if (D != kD) return false;
+    const int64_t G = H / KVH;
+    return G >= 1 && G <= kRows / 32;  // at least 32 positions per workgroup
+}
+
+int64_t mfma_n_pad(int64_t n) { return align_up(n, 256); }
+
+int launch_mfma(const MfmaProblem& mp, hipStream_t stream) {
+    if (mp.dtype == CKV_BF16) return run_mfma<__hip_bfloat16>(mp, stream);
+    if (mp.dtype == CKV_F16) return run_mfma<__half>(mp, stream);
+    return CKV_ERR_DTYPE;
+}
+
+}  // namespace ckv

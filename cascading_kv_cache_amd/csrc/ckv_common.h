@@ -62,6 +62,16 @@ struct Elem<__half> {
     __device__ static __half from_float(float v) { return __float2half(v); }
 };
 
+// stage timing hooks (ckv_profile_enable / ckv_profile_read); no-ops while disabled
+void prof_begin(int stage, hipStream_t stream);
+void prof_end(int stage, hipStream_t stream);
+struct StageScope {
+    int stage;
+    hipStream_t stream;
+    StageScope(int s, hipStream_t st) : stage(s), stream(st) { prof_begin(s, st); }
+    ~StageScope() { prof_end(stage, stream); }
+};
+
 inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace ckv

@@ -523,8 +523,12 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
             CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(ckv_update_plan_kernel),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         }
-        hipLaunchKernelGGL(ckv_update_plan_kernel, dim3((unsigned)(A.N * A.H)), dim3(T), lds, stream, p);
+        {
+            StageScope sc(CKV_STAGE_PLAN, stream);
+            hipLaunchKernelGGL(ckv_update_plan_kernel, dim3((unsigned)(A.N * A.H)), dim3(T), lds, stream, p);
+        }
         CKV_HIP_TRY(hipGetLastError());
+        StageScope sc_apply(CKV_STAGE_APPLY, stream);
 
         if (vec) {
             const int chunks = (int)(A.HID * es / 16);

@@ -220,6 +220,28 @@ int64_t ckv_dense_workspace_bytes(int64_t B, int64_t H, int64_t n_ctx, int64_t n
 
 int ckv_attn_dense(const ckv_dense_args* args, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Stage timing (the reference's BENCHMARK=True switch, cascading_cache.py:986-1026, extended to
+ * every kernel stage).  While enabled, each stage of ckv_attn / ckv_update is bracketed by HIP
+ * events on the caller's stream; ckv_profile_read waits for them, ADDS the elapsed milliseconds
+ * and launch counts per stage into the caller's arrays (length CKV_STAGE_COUNT) and forgets
+ * them.  Process-wide and not thread-safe: a measurement aid, off by default.
+ * ---------------------------------------------------------------------------------------- */
+typedef enum ckv_stage {
+    CKV_STAGE_PREP = 0,        /* rotate + gather prologue                      */
+    CKV_STAGE_FWD = 1,         /* prefill attention forward (QK^T, softmax, PV) */
+    CKV_STAGE_SCORES = 2,      /* prefill score sums (column pass)              */
+    CKV_STAGE_FINISH = 3,      /* head reduction + EMA epilogue                 */
+    CKV_STAGE_DECODE = 4,      /* decode attention main kernel                  */
+    CKV_STAGE_DECODE_TAIL = 5, /* decode combine + scores                       */
+    CKV_STAGE_PLAN = 6,        /* cache update: plan                            */
+    CKV_STAGE_APPLY = 7,       /* cache update: apply                           */
+    CKV_STAGE_COUNT = 8
+} ckv_stage;
+
+int ckv_profile_enable(int on);                       /* returns the previous setting */
+int ckv_profile_read(double* ms, int64_t* launches);  /* both arrays CKV_STAGE_COUNT long */
+
 /* human-readable text for a ckv_status (static storage, never NULL) */
 const char* ckv_strerror(int status);
 

@@ -117,6 +117,21 @@ def test_sixteen_bit_stream(dtype):
     print(f"{dtype}: {flips}/{compared} slots chose a different token (tie-level score differences)")
 
 
+@pytest.mark.parametrize("H,KVH,Q,W,C,NS,eager,dtype", [
+    (8, 2, 128, 256, 4, 64, True, torch.bfloat16),     # G = 4, the Llama grouping
+    (14, 2, 96, 128, 4, 64, True, torch.bfloat16),     # G = 7, the Qwen2 grouping
+    (4, 4, 200, 128, 2, 8, False, torch.bfloat16),     # G = 1, ragged chunk, sparse fill
+    (16, 2, 64, 64, 8, 64, True, torch.float16),       # G = 8
+    (8, 2, 300, 128, 4, 64, False, torch.bfloat16),    # chunk longer than a cascade window
+])
+def test_mfma_prefill_head128(H, KVH, Q, W, C, NS, eager, dtype):
+    """head_dim 128 in 16-bit takes the MFMA kernels: stream chunks while the cache fills up and
+    starts evicting, teacher-forced against the oracle."""
+    flips, compared = run_teacher_forced(2, H, KVH, 128, NS, W, C, Q, 8, dtype, seed=11, eager=eager, std=0.7,
+                                         q_last=Q - 37)
+    print(f"{flips}/{compared} slots chose a different token")
+
+
 def dense_reference(q, k, v, mask, sm_scale):
     n_ctx, n_kv = q.size(2), k.size(2)
     logits = torch.matmul(q.float(), k.float().transpose(2, 3)) * sm_scale
