@@ -287,23 +287,45 @@ struct FwdParams {
     float scale_log2; // softmax scale * log2(e)
 };
 
-template <typename T>
-__global__ void __launch_bounds__(256) fwd_mfma_kernel(FwdParams p) {
-    __shared__ __align__(16) T k_lds[kBN * kKP];
-    __shared__ __align__(16) T v_lds[kD * kVP];
+// Asynchronous global -> LDS copy of one 16-byte piece per lane (gfx950 global_load_lds_dwordx4):
+// the wavefront's 64 pieces land contiguously at `lds_wave_base` (uniform), lane i at +16*i.
+__device__ inline void async_copy16(const void* gptr, void* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gptr,
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
+constexpr int kStageBytes = 32768;   // one K tile (64 x 256 B) + one V^T tile (128 x 128 B)
+constexpr int kVisCap = 2048;        // key tiles whose visibility words are cached in LDS
+
+// LDS tiles are unpadded (the async copy writes 1 KiB per wavefront contiguously); bank conflicts
+// are avoided by XOR-swizzling the 16-byte piece index with the row:
+//   K tile   piece c of key row r   lives at r*256 + ((c ^ (r & 15)) << 4)
+//   V^T tile piece c of dim row d   lives at d*128 + ((c ^ ((d >> 1) & 7)) << 4)
+__device__ inline int k_lds_off(int r, int c) { return r * 256 + ((c ^ (r & 15)) << 4); }
+__device__ inline int v_lds_off(int d, int c) { return d * 128 + ((c ^ ((d >> 1) & 7)) << 4); }
+
+// NC = 32-row query subtiles per wavefront, NW = wavefronts per workgroup; a workgroup covers
+// 32 * NC * NW (head, position) rows of one kv head.
+template <typename T, int NC, int NW>
+__global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned long long* vis_lds = reinterpret_cast<unsigned long long*>(smem + 2 * kStageBytes);
+    constexpr int kThreads = 64 * NW;
+    constexpr int kBlocksPerWave = 16 / NW;  // 1 KiB blocks of each 16 KiB tile copied by one wavefront
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, half = lane >> 5;
     const int64_t bkv = blockIdx.y;
     const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
-    const int64_t m0 = (int64_t)blockIdx.x * p.QT;
+    const int m0 = (int)blockIdx.x * p.QT;
 
-    // the two query rows (one per 32-row subtile) this lane owns as MFMA column `col`
-    int64_t row_m[2], row_h[2];
-    bool row_ok[2];
-    uint4 qreg[2][8];
+    // the query rows (one per 32-row subtile) this lane owns as MFMA column `col`
+    int row_m[NC];
+    int64_t row_h[NC];
+    bool row_ok[NC];
+    uint4 qreg[NC][8];
 #pragma unroll
-    for (int c = 0; c < 2; c++) {
-        const int r = wave * 64 + c * 32 + col;
+    for (int c = 0; c < NC; c++) {
+        const int r = wave * (32 * NC) + c * 32 + col;
         const int g = r / p.QT, mloc = r % p.QT;
         row_m[c] = m0 + mloc;
         row_h[c] = kvh * p.G + g;
@@ -315,83 +337,112 @@ __global__ void __launch_bounds__(256) fwd_mfma_kernel(FwdParams p) {
         }
     }
 
-    f32x16 oacc[4][2];
+    f32x16 oacc[4][NC];
 #pragma unroll
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
-        for (int c = 0; c < 2; c++)
+        for (int c = 0; c < NC; c++)
 #pragma unroll
             for (int v = 0; v < 16; v++) oacc[dt][c][v] = 0.f;
-    float m_run[2] = {-INFINITY, -INFINITY};
-    float l_run[2] = {0.f, 0.f};  // partial over this lane's keys; halves are added at the end
-
-    int64_t m_hi = m0 + p.QT - 1;
-    if (m_hi > p.Q - 1) m_hi = p.Q - 1;
-    const int64_t n_tiles = (p.Nc + m_hi) / kBN + 1;
-    const T* kbase = (const T*)p.kr + bkv * p.n_pad * kD;
-    const T* vbase = (const T*)p.vt + bkv * p.n_pad * kD;
-
-    for (int64_t t = 0; t < n_tiles; t++) {
-        const unsigned long long vis = p.tile_vis[t];
-        if (vis == 0ull) continue;  // uniform: every key of the tile is masked
-        __syncthreads();            // previous tile fully consumed
-        {   // 64 x 128 K rows and 128 x 64 V^T rows, 16 bytes per thread per pass
-            const T* kt = kbase + t * (int64_t)(kBN * kD);
-            const T* vtile = vbase + t * (int64_t)(kBN * kD);
+    float m_run[NC], l_run[NC];  // l_run: partial over this lane's keys; halves are added at the end
 #pragma unroll
-            for (int it = 0; it < 4; it++) {
-                const int chunk = it * 256 + tid;       // 0..1023
-                const int kr_ = chunk >> 4, kc = chunk & 15;  // K: 16 chunks per row
-                *reinterpret_cast<uint4*>(&k_lds[kr_ * kKP + kc * 8]) =
-                    *reinterpret_cast<const uint4*>(kt + kr_ * kD + kc * 8);
-                const int vr = chunk >> 3, vc = chunk & 7;    // V^T: 8 chunks per row
-                *reinterpret_cast<uint4*>(&v_lds[vr * kVP + vc * 8]) =
-                    *reinterpret_cast<const uint4*>(vtile + vr * kBN + vc * 8);
-            }
+    for (int c = 0; c < NC; c++) {
+        m_run[c] = -INFINITY;
+        l_run[c] = 0.f;
+    }
+
+    int m_hi = m0 + p.QT - 1;
+    if (m_hi > (int)p.Q - 1) m_hi = (int)p.Q - 1;
+    const int n_tiles = (int)((p.Nc + m_hi) / kBN) + 1;
+    const char* kbase = (const char*)p.kr + bkv * p.n_pad * kD * (int64_t)sizeof(T);
+    const char* vbase = (const char*)p.vt + bkv * p.n_pad * kD * (int64_t)sizeof(T);
+
+    for (int i = tid; i < n_tiles && i < kVisCap; i += kThreads) vis_lds[i] = p.tile_vis[i];
+    __syncthreads();
+    auto vis_of = [&](int t) -> unsigned long long {
+        return t < kVisCap ? vis_lds[t] : p.tile_vis[__builtin_amdgcn_readfirstlane(t)];
+    };
+    auto next_visible = [&](int t) {
+        while (t < n_tiles && vis_of(t) == 0ull) t++;  // uniform: all keys of a tile masked
+        return t;
+    };
+    // this lane's source offsets inside a tile, fixed for the whole kernel
+    int k_src[kBlocksPerWave], v_src[kBlocksPerWave];
+#pragma unroll
+    for (int j = 0; j < kBlocksPerWave; j++) {
+        const int blk = wave * kBlocksPerWave + j;
+        const int pk_ = blk * 64 + lane;                     // piece position inside the LDS tile
+        const int kr_ = pk_ >> 4, kc = (pk_ & 15) ^ (kr_ & 15);
+        k_src[j] = kr_ * 256 + kc * 16;
+        const int vd = pk_ >> 3, vc = (pk_ & 7) ^ ((vd >> 1) & 7);
+        v_src[j] = vd * 128 + vc * 16;
+    }
+    auto issue = [&](int t, int stage) {
+        const char* kt = kbase + (int64_t)t * (kBN * kD * (int)sizeof(T));
+        const char* vtile = vbase + (int64_t)t * (kBN * kD * (int)sizeof(T));
+        unsigned char* st = smem + stage * kStageBytes;
+#pragma unroll
+        for (int j = 0; j < kBlocksPerWave; j++) {
+            const int blk = wave * kBlocksPerWave + j;
+            async_copy16(kt + k_src[j], st + blk * 1024);
+            async_copy16(vtile + v_src[j], st + 16384 + blk * 1024);
         }
-        __syncthreads();
+    };
+
+    int t = next_visible(0);
+    int stage = 0;
+    if (t < n_tiles) issue(t, 0);
+    while (t < n_tiles) {
+        const unsigned long long vis = vis_of(t);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's pieces of tile t have landed
+        __syncthreads();                     // ... everyone's have, and the other stage is free again
+        const int t_next = next_visible(t + 1);
+        if (t_next < n_tiles) issue(t_next, stage ^ 1);
+        const unsigned char* k_lds = smem + stage * kStageBytes;
+        const unsigned char* v_lds = k_lds + 16384;
 
         // S^T tile: sacc[ks][c][v] = logit of key 32ks + 8(v/4) + 4half + v%4 for query column col
-        f32x16 sacc[2][2];
+        f32x16 sacc[2][NC];
 #pragma unroll
         for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-            for (int c = 0; c < 2; c++)
+            for (int c = 0; c < NC; c++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) sacc[ks][c][v] = 0.f;
 #pragma unroll
         for (int kk = 0; kk < 8; kk++) {
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
-                const uint4 a = *reinterpret_cast<const uint4*>(&k_lds[(32 * ks + col) * kKP + 16 * kk + 8 * half]);
-                sacc[ks][0] = Mma<T>::mma(a, qreg[0][kk], sacc[ks][0]);
-                sacc[ks][1] = Mma<T>::mma(a, qreg[1][kk], sacc[ks][1]);
+                const uint4 a = *reinterpret_cast<const uint4*>(k_lds + k_lds_off(32 * ks + col, 2 * kk + half));
+#pragma unroll
+                for (int c = 0; c < NC; c++) sacc[ks][c] = Mma<T>::mma(a, qreg[c][kk], sacc[ks][c]);
             }
         }
 
         // masking is needed only on tiles with hidden keys or tiles that reach past the diagonal
-        const int64_t key0 = t * kBN;
-        const bool need_mask = (vis != ~0ull) || (key0 + kBN - 1 - p.Nc > m0);
-        uint32_t pk[2][4][4];  // P^T as MFMA B operands: [query subtile][step][4 x 2 elements]
+        const int key0 = t * kBN;
+        if ((vis != ~0ull) || (key0 + kBN - 1 - (int)p.Nc > m0)) {
 #pragma unroll
-        for (int c = 0; c < 2; c++) {
+            for (int c = 0; c < NC; c++)
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const int kidx = 32 * ks + 8 * (v >> 2) + 4 * half + (v & 3);
+                        const int nrel = key0 - (int)p.Nc + kidx;  // >= 0: key of the chunk
+                        const bool ok = ((vis >> kidx) & 1ull) && (nrel < 0 || nrel <= row_m[c]);
+                        sacc[ks][c][v] = ok ? sacc[ks][c][v] : -INFINITY;
+                    }
+        }
+        uint32_t pk[NC][4][4];  // P^T as MFMA B operands: [query subtile][step][4 x 2 elements]
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
             float mx = -INFINITY;
 #pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
+            for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    float s = sacc[ks][c][v] * p.scale_log2;
-                    if (need_mask) {
-                        const int kidx = 32 * ks + 8 * (v >> 2) + 4 * half + (v & 3);
-                        const int64_t n = key0 + kidx;
-                        const bool ok = ((vis >> kidx) & 1ull) && (n < p.Nc || n - p.Nc <= row_m[c]);
-                        s = ok ? s : -INFINITY;
-                    }
-                    sacc[ks][c][v] = s;
-                    mx = fmaxf(mx, s);
-                }
-            }
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+                for (int v = 0; v < 16; v++) mx = fmaxf(mx, sacc[ks][c][v]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32)) * p.scale_log2;  // scale > 0 commutes with max
             const float m_new = fmaxf(m_run[c], mx);
             const float m_use = m_new == -INFINITY ? 0.f : m_new;
             const float alpha = __builtin_amdgcn_exp2f(m_run[c] - m_use);
@@ -401,18 +452,22 @@ __global__ void __launch_bounds__(256) fwd_mfma_kernel(FwdParams p) {
             for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
                 for (int v = 0; v < 16; v += 2) {
-                    const float p0 = __builtin_amdgcn_exp2f(sacc[ks][c][v] - m_use);
-                    const float p1 = __builtin_amdgcn_exp2f(sacc[ks][c][v + 1] - m_use);
+                    const float p0 = __builtin_amdgcn_exp2f(fmaf(sacc[ks][c][v], p.scale_log2, -m_use));
+                    const float p1 = __builtin_amdgcn_exp2f(fmaf(sacc[ks][c][v + 1], p.scale_log2, -m_use));
                     rs += p0 + p1;
                     // step = 2ks + v/8, element = v%8
                     pk[c][2 * ks + (v >> 3)][(v & 7) >> 1] = Mma<T>::pack2(p0, p1);
                 }
             }
             l_run[c] = l_run[c] * alpha + rs;
+            // the running maximum settles after a few tiles: skip the accumulator rescale
+            // whenever no row of the wavefront moved (alpha == 1 everywhere)
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0ull) {
 #pragma unroll
-            for (int dt = 0; dt < 4; dt++)
+                for (int dt = 0; dt < 4; dt++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) oacc[dt][c][v] *= alpha;
+                    for (int v = 0; v < 16; v++) oacc[dt][c][v] *= alpha;
+            }
         }
 
         // O^T += V^T P^T
@@ -420,18 +475,21 @@ __global__ void __launch_bounds__(256) fwd_mfma_kernel(FwdParams p) {
         for (int s = 0; s < 4; s++) {
 #pragma unroll
             for (int dt = 0; dt < 4; dt++) {
-                const uint4 a = *reinterpret_cast<const uint4*>(&v_lds[(32 * dt + col) * kVP + 16 * s + 8 * half]);
-                const uint4 b0 = make_uint4(pk[0][s][0], pk[0][s][1], pk[0][s][2], pk[0][s][3]);
-                const uint4 b1 = make_uint4(pk[1][s][0], pk[1][s][1], pk[1][s][2], pk[1][s][3]);
-                oacc[dt][0] = Mma<T>::mma(a, b0, oacc[dt][0]);
-                oacc[dt][1] = Mma<T>::mma(a, b1, oacc[dt][1]);
+                const uint4 a = *reinterpret_cast<const uint4*>(v_lds + v_lds_off(32 * dt + col, 2 * s + half));
+#pragma unroll
+                for (int c = 0; c < NC; c++) {
+                    const uint4 bq = make_uint4(pk[c][s][0], pk[c][s][1], pk[c][s][2], pk[c][s][3]);
+                    oacc[dt][c] = Mma<T>::mma(a, bq, oacc[dt][c]);
+                }
             }
         }
+        t = t_next;
+        stage ^= 1;
     }
 
     // epilogue: lane owns d = 32dt + 8(v/4) + 4half + v%4 of its query row
 #pragma unroll
-    for (int c = 0; c < 2; c++) {
+    for (int c = 0; c < NC; c++) {
         const float l_tot = l_run[c] + __shfl_xor(l_run[c], 32);
         if (!row_ok[c]) continue;
         const float inv = 1.f / l_tot;
@@ -645,10 +703,15 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         fp.lse = mp.lse;
         fp.B = mp.B; fp.H = mp.H; fp.KVH = mp.KVH; fp.Q = mp.Q; fp.N = n; fp.Nc = n - mp.Q; fp.n_pad = n_pad;
         fp.G = G;
-        fp.QT = kRows / G;
+        constexpr int kNC = 1, kNW = 8;
+        constexpr int kWgRows = 32 * kNC * kNW;
+        fp.QT = kWgRows / G;
         fp.scale_log2 = scale_log2;
         const dim3 grid((unsigned)((mp.Q + fp.QT - 1) / fp.QT), (unsigned)(mp.B * mp.KVH));
-        hipLaunchKernelGGL(fwd_mfma_kernel<T>, grid, dim3(256), 0, stream, fp);
+        const int lds = 2 * kStageBytes + kVisCap * 8;
+        CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fwd_mfma_kernel<T, kNC, kNW>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        hipLaunchKernelGGL((fwd_mfma_kernel<T, kNC, kNW>), grid, dim3(64 * kNW), lds, stream, fp);
         CKV_HIP_TRY(hipGetLastError());
     }
     if (mp.colsum) {
