@@ -21,7 +21,7 @@ struct AttnWorkspace {
     void *qr, *kr, *vc;
     unsigned long long* tile_vis;
     uint8_t* kmasked;
-    float *lse, *colsum, *w_ema, *w_new;
+    float *lse, *lse2, *colsum, *w_ema, *w_new;
     int64_t bytes;
 };
 
@@ -30,14 +30,15 @@ AttnWorkspace carve_attn(void* base, int64_t B, int64_t H, int64_t KVH, int64_t 
     const int64_t es = elem_bytes(dtype), N = NS + S + Q, n_pad = mfma_n_pad(N);
     Carver c(base);
     AttnWorkspace w;
-    w.qr = c.take(B * H * Q * D * es);
+    w.qr = c.take((B * H * Q + 64) * D * es);  // 64 rows of slack for the MFMA column pass
     w.kr = c.take(B * KVH * n_pad * D * es);   // padded to whole key tiles for the MFMA family
     w.vc = c.take(B * KVH * n_pad * D * es);
     w.tile_vis = (unsigned long long*)c.take(n_pad / 64 * 8);
     w.kmasked = (uint8_t*)c.take(NS + S);
     w.lse = (float*)c.take(B * H * Q * 4);
+    w.lse2 = (float*)c.take((B * H * Q + 64) * 4);
     w.colsum = (float*)c.take(B * H * N * 4);
-    w.w_ema = (float*)c.take(Q * 4);
+    w.w_ema = (float*)c.take((Q + 64) * 4);
     w.w_new = (float*)c.take(Q * 4);
     w.bytes = c.off;
     return w;
@@ -83,7 +84,7 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
         rc = launch_weights(w.w_ema, w.w_new, a.Q, a.beta, a.dtype, stream);
         if (rc) return rc;
     }
-    const bool use_mfma = mfma_supported(a.dtype, a.D, a.H, a.KVH) && a.Q > 1;
+    const bool use_mfma = mfma_supported(a.dtype, a.D, a.H, a.KVH, a.Q) && a.Q > 1;
     if (use_mfma) {
         MfmaProblem mp;
         mp.seg[0] = MfmaSegment{a.sink_k, a.sink_v, {a.sink_stride[0], a.sink_stride[1], a.sink_stride[2], a.sink_stride[3]},
@@ -104,6 +105,7 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
         mp.qr = w.qr; mp.kr = w.kr; mp.vt = w.vc; mp.tile_vis = w.tile_vis;
         mp.out = a.out;
         mp.lse = w.lse;
+        mp.lse2 = w.lse2;
         mp.colsum = want_scores ? w.colsum : nullptr;
         mp.w_ema = w.w_ema; mp.w_new = w.w_new;
         mp.new_mode = 1;
@@ -167,7 +169,7 @@ extern "C" int64_t ckv_dense_workspace_bytes(int64_t B, int64_t H, int64_t n_ctx
     (void)dtype;
     if (B <= 0 || H <= 0 || n_ctx <= 0 || n_kv < n_ctx) return 0;
     using ckv::align_up;
-    return align_up(B * H * n_ctx * 4, 256) + align_up(B * H * n_kv * 4, 256) + 2 * align_up(n_ctx * 4, 256);
+    return align_up(B * H * n_ctx * 4, 256) + align_up(B * H * n_kv * 4, 256) + 2 * align_up((n_ctx + 64) * 4, 256);
 }
 
 extern "C" int ckv_attn_dense(const ckv_dense_args* args, void* stream_) {
@@ -185,7 +187,7 @@ extern "C" int ckv_attn_dense(const ckv_dense_args* args, void* stream_) {
     Carver c(a.workspace);
     float* lse = (float*)c.take(a.B * a.H * a.n_ctx * 4);
     float* colsum = (float*)c.take(a.B * a.H * a.n_kv * 4);
-    float* w_ema = (float*)c.take(a.n_ctx * 4);
+    float* w_ema = (float*)c.take((a.n_ctx + 64) * 4);
     float* w_new = (float*)c.take(a.n_ctx * 4);
     int rc;
     if (a.scores) {

@@ -35,6 +35,7 @@ struct CoreProblem {
 int launch_core_generic(const CoreProblem& p, hipStream_t stream);
 
 // weights of the score sums (cascade_attention.py:270-282, 315-317), rounded like the eager path
+// w_ema gets 64 trailing zeros (slack read by the MFMA column pass)
 int launch_weights(float* w_ema, float* w_new, int64_t Q, double beta, int dtype, hipStream_t stream);
 
 int launch_cast_scores(const float* colsum, void* scores, const int64_t* stride, int64_t B, int64_t H, int64_t N,
@@ -86,7 +87,8 @@ struct MfmaProblem {
     unsigned long long* tile_vis;
     void* out;
     int64_t out_stride[4];
-    float* lse;
+    float* lse;            // (B, H, Q) natural log
+    float* lse2;           // (B*H*Q + 64) scratch: log2-domain copy for the column pass
     float* colsum;         // (B, H, n) or null
     const float* w_ema;
     const float* w_new;
@@ -96,7 +98,7 @@ struct MfmaProblem {
     int dtype;
 };
 
-bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH);
+bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH, int64_t Q);
 int64_t mfma_n_pad(int64_t n);
 int launch_mfma(const MfmaProblem& p, hipStream_t stream);
 

@@ -27,8 +27,7 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kD = 128;    // head dim
 constexpr int kBN = 64;    // keys per tile
-constexpr int kKP = kD + 8;   // LDS pitch of a K / Q row (elements): 16-byte reads stay conflict-free
-constexpr int kVP = kBN + 8;  // LDS pitch of a V^T row
+
 constexpr int kRows = 256;    // (head, position) rows per forward workgroup
 
 template <typename T>
@@ -281,7 +280,8 @@ struct FwdParams {
     const unsigned long long* tile_vis;
     void* out;
     int64_t out_stride[4];
-    float* lse;       // (B*H, Q)
+    float* lse;       // (B*H, Q) natural log
+    float* lse2;      // (B*H, Q) log2 domain, consumed by the column pass
     int64_t B, H, KVH, Q, N, Nc, n_pad;
     int G, QT;        // heads per kv head, positions per workgroup (G * QT <= 256)
     float scale_log2; // softmax scale * log2(e)
@@ -512,7 +512,9 @@ __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
             }
         }
         if (half == 0) {
-            p.lse[(b * p.H + row_h[c]) * p.Q + row_m[c]] = (m_run[c] + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+            const float l2 = m_run[c] + __builtin_amdgcn_logf(l_tot);  // v_log_f32 is log2
+            p.lse[(b * p.H + row_h[c]) * p.Q + row_m[c]] = l2 * 0.6931471805599453f;
+            p.lse2[(b * p.H + row_h[c]) * p.Q + row_m[c]] = l2;
         }
     }
 }
@@ -521,12 +523,12 @@ __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
 // score sums
 // ---------------------------------------------------------------------------------------------
 struct ColsumParams {
-    const void* qr;
+    const void* qr;       // (B*H*Q + 64 rows of slack, D)
     const void* kr;
     const unsigned long long* tile_vis;
-    const float* lse;     // natural log
-    const float* w_ema;
-    const float* w_new;
+    const float* lse2;    // (B*H*Q + 64) log2-domain row normalisers
+    const float* w_ema;   // (Q + 64), zero beyond Q
+    const float* w_new;   // (Q)
     float* colsum;        // (B*H, N)
     int64_t B, H, KVH, Q, N, Nc, n_pad;
     int G;
@@ -534,23 +536,29 @@ struct ColsumParams {
     float scale_log2;
 };
 
-constexpr int kQT2 = 64;  // query rows per LDS tile of the column pass
+constexpr int kQT2 = 64;                      // query rows per LDS tile of the column pass
+constexpr int kCsStage = 16384 + 256 + 256;   // Q tile + its lse2 + its weights
 
+// One workgroup = one kv head x 256 keys (64 per wavefront, held in registers as the B operand of
+// S = Q K^T).  The (head, query-tile) sequence streams through a double-buffered LDS stage filled
+// by asynchronous copies; lane (col, half) owns key column `col` of each 32-key subtile, so the
+// weighted column sums never leave the lane.
 template <typename T>
 __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
-    __shared__ __align__(16) T q_lds[kQT2 * kKP];
-    __shared__ float lse_lds[kQT2];
-    __shared__ float w_lds[kQT2];
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* wnew_lds = reinterpret_cast<float*>(smem + 2 * kCsStage);
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, half = lane >> 5;
     const int64_t bkv = blockIdx.y;
     const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
+    const int Q = (int)p.Q;
     const int64_t key_blk = (int64_t)blockIdx.x * 256;   // first key of the workgroup
-    const int64_t key_w = key_blk + wave * 64;            // first key of this wave
+    const int64_t key_w = key_blk + wave * 64;            // first key of this wavefront
 
-    // K as the B operand: lane (col, half) holds key key_w + 32ks + col, elements 16kk + 8half ..
     uint4 kreg[2][8];
     const T* kbase = (const T*)p.kr + bkv * p.n_pad * kD;
+    bool live[2];
+    int nrel[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
         const int64_t n = key_w + 32 * ks + col;
@@ -559,94 +567,138 @@ __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
             kreg[ks][kk] = n < p.n_pad ? *reinterpret_cast<const uint4*>(kbase + n * kD + 16 * kk + 8 * half)
                                        : make_uint4(0, 0, 0, 0);
         }
-    }
-    bool live[2];
-    int64_t nrel[2];
-#pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
-        const int64_t n = key_w + 32 * ks + col;
         live[ks] = n < p.N && ((p.tile_vis[n / kBN] >> (n % kBN)) & 1ull);
-        nrel[ks] = n - p.Nc;
+        nrel[ks] = (int)(n - p.Nc);
     }
-    // first query row that can see any key of the workgroup
-    int64_t m_first = key_blk - p.Nc;
+    // first query tile that can see any key of the workgroup
+    int m_first = (int)(key_blk - p.Nc);
     if (m_first < 0) m_first = 0;
     m_first = m_first / kQT2 * kQT2;
     const bool chunk_keys = key_blk + 255 >= p.Nc;  // some key of the workgroup belongs to the chunk
-    const float kLog2e = 1.4426950408889634f;
+    const int last_nrel = (int)(key_blk + 255 - p.Nc);
+    if (chunk_keys && p.new_mode) {
+        for (int i = tid; i < Q; i += 256) wnew_lds[i] = p.w_new[i];
+    }
+    const int nmt = (Q - m_first + kQT2 - 1) / kQT2;  // query tiles per head
+    const int n_steps = nmt * p.G;
 
-    for (int g = 0; g < p.G; g++) {
-        const int64_t h = kvh * p.G + g;
-        const T* qbase = (const T*)p.qr + (b * p.H + h) * p.Q * kD;
-        const float* lse = p.lse + (b * p.H + h) * p.Q;
-        float acc[2] = {0.f, 0.f};
-        for (int64_t mt = m_first; mt < p.Q; mt += kQT2) {
-            __syncthreads();
+    // async copy assignments: the Q tile is 16 blocks of 1 KiB (4 per wavefront); wavefront 0 also
+    // brings the tile's 64 normalisers, wavefront 1 its 64 weights (16 lanes x 16 bytes each)
+    int q_src[4];
 #pragma unroll
-            for (int it = 0; it < 4; it++) {
-                const int chunk = it * 256 + tid;
-                const int r = chunk >> 4, cc = chunk & 15;
-                const int64_t m = mt + r;
-                *reinterpret_cast<uint4*>(&q_lds[r * kKP + cc * 8]) =
-                    m < p.Q ? *reinterpret_cast<const uint4*>(qbase + m * kD + cc * 8) : make_uint4(0, 0, 0, 0);
+    for (int j = 0; j < 4; j++) {
+        const int pos = (wave * 4 + j) * 64 + lane;
+        const int r = pos >> 4, c = (pos & 15) ^ (r & 15);
+        q_src[j] = r * 256 + c * 16;
+    }
+    auto issue = [&](int step, int stage) {
+        const int g = step / nmt, mt = m_first + (step % nmt) * kQT2;
+        const int64_t row0 = (b * p.H + kvh * p.G + g) * p.Q + mt;
+        const char* qt = (const char*)p.qr + row0 * (kD * (int64_t)sizeof(T));
+        unsigned char* st = smem + stage * kCsStage;
+#pragma unroll
+        for (int j = 0; j < 4; j++) async_copy16(qt + q_src[j], st + (wave * 4 + j) * 1024);
+        if (wave == 0 && lane < 16) async_copy16((const char*)(p.lse2 + row0) + lane * 16, st + 16384);
+        if (wave == 1 && lane < 16) async_copy16((const char*)(p.w_ema + mt) + lane * 16, st + 16384 + 256);
+    };
+
+    float acc[2] = {0.f, 0.f};
+    int stage = 0;
+    if (n_steps > 0) issue(0, 0);
+    for (int step = 0; step < n_steps; step++) {
+        const int g = step / nmt, mt = m_first + (step % nmt) * kQT2;
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        if (step + 1 < n_steps) issue(step + 1, stage ^ 1);
+        const unsigned char* q_lds = smem + stage * kCsStage;
+        const float* lse_lds = reinterpret_cast<const float*>(q_lds + 16384);
+        const float* w_lds = lse_lds + 64;
+
+        f32x16 sacc[2][2];  // [c = query subtile][ks]
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) sacc[c][ks][v] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++) {
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                const uint4 a = *reinterpret_cast<const uint4*>(q_lds + k_lds_off(32 * c + col, 2 * kk + half));
+                sacc[c][0] = Mma<T>::mma(a, kreg[0][kk], sacc[c][0]);
+                sacc[c][1] = Mma<T>::mma(a, kreg[1][kk], sacc[c][1]);
             }
-            if (tid < kQT2) {
-                const int64_t m = mt + tid;
-                lse_lds[tid] = m < p.Q ? lse[m] * kLog2e : INFINITY;  // +inf -> P = 0 for padding rows
-                w_lds[tid] = m < p.Q ? p.w_ema[m] : 0.f;
-            }
-            __syncthreads();
-            f32x16 sacc[2][2];  // [c = query subtile][ks]
+        }
+        // element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4, key column of this lane
+        const bool tail = mt + kQT2 > Q;                       // rows past the chunk end
+        const bool diag = chunk_keys && mt <= last_nrel;       // tile may cross the diagonal
+        if (!tail && !diag && !(chunk_keys && p.new_mode)) {
 #pragma unroll
-            for (int c = 0; c < 2; c++)
+            for (int c = 0; c < 2; c++) {
 #pragma unroll
-                for (int ks = 0; ks < 2; ks++)
+                for (int v4 = 0; v4 < 4; v4++) {
+                    const int r0 = 32 * c + 8 * v4 + 4 * half;
+                    const float4 l4 = *reinterpret_cast<const float4*>(lse_lds + r0);
+                    const float4 w4 = *reinterpret_cast<const float4*>(w_lds + r0);
+                    const float ls[4] = {l4.x, l4.y, l4.z, l4.w};
+                    const float ws[4] = {w4.x, w4.y, w4.z, w4.w};
 #pragma unroll
-                    for (int v = 0; v < 16; v++) sacc[c][ks][v] = 0.f;
+                    for (int e = 0; e < 4; e++) {
 #pragma unroll
-            for (int kk = 0; kk < 8; kk++) {
-#pragma unroll
-                for (int c = 0; c < 2; c++) {
-                    const uint4 a = *reinterpret_cast<const uint4*>(&q_lds[(32 * c + col) * kKP + 16 * kk + 8 * half]);
-                    sacc[c][0] = Mma<T>::mma(a, kreg[0][kk], sacc[c][0]);
-                    sacc[c][1] = Mma<T>::mma(a, kreg[1][kk], sacc[c][1]);
+                        for (int ks = 0; ks < 2; ks++) {
+                            const float pe = __builtin_amdgcn_exp2f(fmaf(sacc[c][ks][4 * v4 + e], p.scale_log2, -ls[e]));
+                            acc[ks] = fmaf(ws[e], pe, acc[ks]);
+                        }
+                    }
                 }
             }
-            // element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4, key column of this lane
-            const bool diag = chunk_keys && (mt < key_blk + 256 - p.Nc);  // tile may cross the diagonal
+        } else {
 #pragma unroll
             for (int c = 0; c < 2; c++) {
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
                     const int r = 32 * c + 8 * (v >> 2) + 4 * half + (v & 3);
+                    const int m = mt + r;
+                    const bool row_in = m < Q;
                     const float l2 = lse_lds[r];
+                    const float we = w_lds[r];
 #pragma unroll
                     for (int ks = 0; ks < 2; ks++) {
-                        float pe = __builtin_amdgcn_exp2f(sacc[c][ks][v] * p.scale_log2 - l2);
-                        pe = Mma<T>::round1(pe);
-                        if (chunk_keys && nrel[ks] >= 0) {
-                            const int64_t m = mt + r;
-                            if (diag && m < nrel[ks]) pe = 0.f;
-                            if (p.new_mode) {
-                                const int64_t k = m - nrel[ks];
-                                const float w = (k >= 0 && m < p.Q) ? p.w_new[k] : 0.f;
-                                acc[ks] += Mma<T>::round1(pe * w);
-                            } else {
-                                acc[ks] = fmaf(w_lds[r], pe, acc[ks]);
-                            }
+                        float pe = __builtin_amdgcn_exp2f(fmaf(sacc[c][ks][v], p.scale_log2, -l2));
+                        const bool is_chunk = nrel[ks] >= 0;
+                        const bool vis = row_in && (!is_chunk || m >= nrel[ks]);
+                        pe = vis ? pe : 0.f;
+                        if (is_chunk && p.new_mode) {
+                            // the eager path holds P and the products in the tensor dtype
+                            const float w = vis ? wnew_lds[m - nrel[ks]] : 0.f;
+                            acc[ks] += Mma<T>::round1(Mma<T>::round1(pe) * w);
                         } else {
-                            acc[ks] = fmaf(w_lds[r], pe, acc[ks]);
+                            acc[ks] = fmaf(row_in ? we : 0.f, pe, acc[ks]);
                         }
                     }
                 }
             }
         }
+        if ((step % nmt) == nmt - 1) {  // head finished: combine the two lane halves and store
+            const int64_t h = kvh * p.G + g;
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
-            const float tot = acc[ks] + __shfl_xor(acc[ks], 32);
-            const int64_t n = key_w + 32 * ks + col;
-            if (half == 0 && n < p.N) p.colsum[(b * p.H + h) * p.N + n] = live[ks] ? tot : 0.f;
+            for (int ks = 0; ks < 2; ks++) {
+                const float tot = acc[ks] + __shfl_xor(acc[ks], 32);
+                const int64_t n = key_w + 32 * ks + col;
+                if (half == 0 && n < p.N) p.colsum[(b * p.H + h) * p.N + n] = live[ks] ? tot : 0.f;
+                acc[ks] = 0.f;
+            }
         }
+        stage ^= 1;
+    }
+    if (n_steps == 0) {  // no query can see these keys (only possible for padding blocks)
+        for (int g = 0; g < p.G; g++)
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                const int64_t n = key_w + 32 * ks + col;
+                if (half == 0 && n < p.N) p.colsum[(b * p.H + kvh * p.G + g) * p.N + n] = 0.f;
+            }
     }
 }
 
@@ -701,6 +753,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         fp.out = mp.out;
         for (int j = 0; j < 4; j++) fp.out_stride[j] = mp.out_stride[j];
         fp.lse = mp.lse;
+        fp.lse2 = mp.lse2;
         fp.B = mp.B; fp.H = mp.H; fp.KVH = mp.KVH; fp.Q = mp.Q; fp.N = n; fp.Nc = n - mp.Q; fp.n_pad = n_pad;
         fp.G = G;
         constexpr int kNC = 1, kNW = 8;
@@ -717,14 +770,17 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
     if (mp.colsum) {
         StageScope sc(CKV_STAGE_SCORES, stream);
         ColsumParams cp;
-        cp.qr = mp.qr; cp.kr = mp.kr; cp.tile_vis = mp.tile_vis; cp.lse = mp.lse;
+        cp.qr = mp.qr; cp.kr = mp.kr; cp.tile_vis = mp.tile_vis; cp.lse2 = mp.lse2;
         cp.w_ema = mp.w_ema; cp.w_new = mp.w_new; cp.colsum = mp.colsum;
         cp.B = mp.B; cp.H = mp.H; cp.KVH = mp.KVH; cp.Q = mp.Q; cp.N = n; cp.Nc = n - mp.Q; cp.n_pad = n_pad;
         cp.G = G;
         cp.new_mode = mp.new_mode;
         cp.scale_log2 = scale_log2;
         const dim3 grid((unsigned)((n + 255) / 256), (unsigned)(mp.B * mp.KVH));
-        hipLaunchKernelGGL(colsum_mfma_kernel<T>, grid, dim3(256), 0, stream, cp);
+        const int lds = 2 * kCsStage + (int)mp.Q * 4;
+        CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(colsum_mfma_kernel<T>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        hipLaunchKernelGGL(colsum_mfma_kernel<T>, grid, dim3(256), lds, stream, cp);
         CKV_HIP_TRY(hipGetLastError());
     }
     return CKV_OK;
@@ -732,9 +788,10 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
 
 }  // namespace
 
-bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH) {
+bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH, int64_t Q) {
     if (dtype != CKV_BF16 && dtype != CKV_F16) return false;
     if (D != kD) return false;
+    if (Q > 24576) return false;  // the column pass keeps a Q-long weight table in LDS
     const int64_t G = H / KVH;
     return G >= 1 && G <= kRows / 32;  // at least 32 positions per workgroup
 }
