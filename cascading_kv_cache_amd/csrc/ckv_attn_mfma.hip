@@ -288,10 +288,19 @@ struct FwdParams {
 };
 
 // Asynchronous global -> LDS copy of one 16-byte piece per lane (gfx950 global_load_lds_dwordx4):
-// the wavefront's 64 pieces land contiguously at `lds_wave_base` (uniform), lane i at +16*i.
-__device__ inline void async_copy16(const void* gptr, void* lds_wave_base) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gptr,
-                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+// the wavefront's 64 pieces land contiguously at LDS byte address `lds_wave_base` (uniform, goes
+// to M0), lane i at +16*i.  Written as inline assembly on purpose: the compiler then keeps no
+// scoreboard entry for the copy, so it cannot force it to complete before unrelated LDS reads;
+// completion is awaited explicitly with s_waitcnt vmcnt(n) (copies retire in issue order).
+__device__ inline void async_copy16(const void* gptr, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(gptr)
+                 : "memory");
+}
+
+__device__ inline uint32_t lds_address(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
 
 constexpr int kStageBytes = 32768;   // one K tile (64 x 256 B) + one V^T tile (128 x 128 B)
@@ -309,7 +318,8 @@ __device__ inline int v_lds_off(int d, int c) { return d * 128 + ((c ^ ((d >> 1)
 template <typename T, int NC, int NW>
 __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    unsigned long long* vis_lds = reinterpret_cast<unsigned long long*>(smem + 2 * kStageBytes);
+    unsigned long long* vis_lds = reinterpret_cast<unsigned long long*>(smem + 3 * kStageBytes);
+    const uint32_t smem_addr = lds_address(smem);
     constexpr int kThreads = 64 * NW;
     constexpr int kBlocksPerWave = 16 / NW;  // 1 KiB blocks of each 16 KiB tile copied by one wavefront
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -380,7 +390,7 @@ __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
     auto issue = [&](int t, int stage) {
         const char* kt = kbase + (int64_t)t * (kBN * kD * (int)sizeof(T));
         const char* vtile = vbase + (int64_t)t * (kBN * kD * (int)sizeof(T));
-        unsigned char* st = smem + stage * kStageBytes;
+        const uint32_t st = smem_addr + stage * kStageBytes;
 #pragma unroll
         for (int j = 0; j < kBlocksPerWave; j++) {
             const int blk = wave * kBlocksPerWave + j;
@@ -389,15 +399,24 @@ __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
         }
     };
 
+    // three LDS stages: tiles t+1 and t+2 are in flight while tile t is being consumed
     int t = next_visible(0);
+    int t1 = t < n_tiles ? next_visible(t + 1) : n_tiles;
     int stage = 0;
     if (t < n_tiles) issue(t, 0);
+    if (t1 < n_tiles) issue(t1, 1);
     while (t < n_tiles) {
         const unsigned long long vis = vis_of(t);
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's pieces of tile t have landed
-        __syncthreads();                     // ... everyone's have, and the other stage is free again
-        const int t_next = next_visible(t + 1);
-        if (t_next < n_tiles) issue(t_next, stage ^ 1);
+        // every wavefront issues 2 * kBlocksPerWave copies per tile and they retire in order:
+        // leaving one tile's worth outstanding means tile t has landed
+        if (t1 < n_tiles) {
+            __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kBlocksPerWave));
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
+        __syncthreads();  // everyone's pieces have landed, and the stage used two tiles ago is free
+        const int t2 = t1 < n_tiles ? next_visible(t1 + 1) : n_tiles;
+        if (t2 < n_tiles) issue(t2, stage == 0 ? 2 : stage - 1);
         const unsigned char* k_lds = smem + stage * kStageBytes;
         const unsigned char* v_lds = k_lds + 16384;
 
@@ -483,8 +502,9 @@ __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
                 }
             }
         }
-        t = t_next;
-        stage ^= 1;
+        t = t1;
+        t1 = t2;
+        stage = stage == 2 ? 0 : stage + 1;
     }
 
     // epilogue: lane owns d = 32dt + 8(v/4) + 4half + v%4 of its query row
@@ -537,7 +557,7 @@ struct ColsumParams {
 };
 
 constexpr int kQT2 = 64;                      // query rows per LDS tile of the column pass
-constexpr int kCsStage = 16384 + 256 + 256;   // Q tile + its lse2 + its weights
+constexpr int kCsStage = 16384 + 256 + 256 + 512;   // Q tile + its lse2 + its weights + dummy landing zone
 
 // One workgroup = one kv head x 256 keys (64 per wavefront, held in registers as the B operand of
 // S = Q K^T).  The (head, query-tile) sequence streams through a double-buffered LDS stage filled
@@ -546,7 +566,8 @@ constexpr int kCsStage = 16384 + 256 + 256;   // Q tile + its lse2 + its weights
 template <typename T>
 __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    float* wnew_lds = reinterpret_cast<float*>(smem + 2 * kCsStage);
+    float* wnew_lds = reinterpret_cast<float*>(smem + 3 * kCsStage);
+    const uint32_t smem_addr = lds_address(smem);
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int col = lane & 31, half = lane >> 5;
     const int64_t bkv = blockIdx.y;
@@ -595,21 +616,29 @@ __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
         const int g = step / nmt, mt = m_first + (step % nmt) * kQT2;
         const int64_t row0 = (b * p.H + kvh * p.G + g) * p.Q + mt;
         const char* qt = (const char*)p.qr + row0 * (kD * (int64_t)sizeof(T));
-        unsigned char* st = smem + stage * kCsStage;
+        const uint32_t st = smem_addr + stage * kCsStage;
 #pragma unroll
         for (int j = 0; j < 4; j++) async_copy16(qt + q_src[j], st + (wave * 4 + j) * 1024);
-        if (wave == 0 && lane < 16) async_copy16((const char*)(p.lse2 + row0) + lane * 16, st + 16384);
-        if (wave == 1 && lane < 16) async_copy16((const char*)(p.w_ema + mt) + lane * 16, st + 16384 + 256);
+        // every wavefront issues exactly 5 copies per step so that one vmcnt value fits all
+        if (lane < 16) {
+            const char* src = (wave & 1) ? (const char*)(p.w_ema + mt) : (const char*)(p.lse2 + row0);
+            async_copy16(src + lane * 16, st + 16384 + wave * 256);  // waves 2, 3 land in the dummy zone
+        }
     };
 
     float acc[2] = {0.f, 0.f};
     int stage = 0;
     if (n_steps > 0) issue(0, 0);
+    if (n_steps > 1) issue(1, 1);
     for (int step = 0; step < n_steps; step++) {
         const int g = step / nmt, mt = m_first + (step % nmt) * kQT2;
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        if (step + 1 < n_steps) {
+            __builtin_amdgcn_s_waitcnt(0x0F75);  // vmcnt(5): only the next step's copies may be pending
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
         __syncthreads();
-        if (step + 1 < n_steps) issue(step + 1, stage ^ 1);
+        if (step + 2 < n_steps) issue(step + 2, stage == 0 ? 2 : stage - 1);
         const unsigned char* q_lds = smem + stage * kCsStage;
         const float* lse_lds = reinterpret_cast<const float*>(q_lds + 16384);
         const float* w_lds = lse_lds + 64;
@@ -690,7 +719,7 @@ __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
                 acc[ks] = 0.f;
             }
         }
-        stage ^= 1;
+        stage = stage == 2 ? 0 : stage + 1;
     }
     if (n_steps == 0) {  // no query can see these keys (only possible for padding blocks)
         for (int g = 0; g < p.G; g++)
@@ -761,7 +790,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         fp.QT = kWgRows / G;
         fp.scale_log2 = scale_log2;
         const dim3 grid((unsigned)((mp.Q + fp.QT - 1) / fp.QT), (unsigned)(mp.B * mp.KVH));
-        const int lds = 2 * kStageBytes + kVisCap * 8;
+        const int lds = 3 * kStageBytes + kVisCap * 8;
         CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fwd_mfma_kernel<T, kNC, kNW>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         hipLaunchKernelGGL((fwd_mfma_kernel<T, kNC, kNW>), grid, dim3(64 * kNW), lds, stream, fp);
@@ -777,7 +806,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         cp.new_mode = mp.new_mode;
         cp.scale_log2 = scale_log2;
         const dim3 grid((unsigned)((n + 255) / 256), (unsigned)(mp.B * mp.KVH));
-        const int lds = 2 * kCsStage + (int)mp.Q * 4;
+        const int lds = 3 * kCsStage + (int)mp.Q * 4;
         CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(colsum_mfma_kernel<T>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         hipLaunchKernelGGL(colsum_mfma_kernel<T>, grid, dim3(256), lds, stream, cp);
