@@ -15,6 +15,8 @@
 //                the weighted column sums stay inside a lane (S = Q K^T orientation).
 #include "ckv_attn_internal.h"
 
+#include <type_traits>
+
 namespace ckv {
 namespace {
 
@@ -287,15 +289,23 @@ struct FwdParams {
     float scale_log2; // softmax scale * log2(e)
 };
 
+__device__ inline const void* uniform_ptr(const void* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo);
+}
+
 // Asynchronous global -> LDS copy of one 16-byte piece per lane (gfx950 global_load_lds_dwordx4):
 // the wavefront's 64 pieces land contiguously at LDS byte address `lds_wave_base` (uniform, goes
-// to M0), lane i at +16*i.  Written as inline assembly on purpose: the compiler then keeps no
-// scoreboard entry for the copy, so it cannot force it to complete before unrelated LDS reads;
-// completion is awaited explicitly with s_waitcnt vmcnt(n) (copies retire in issue order).
-__device__ inline void async_copy16(const void* gptr, uint32_t lds_wave_base) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+// to M0), lane i at +16*i; the source is `sbase` (uniform, SGPR pair) + `voff` (per lane).
+// Inline assembly on purpose: the compiler keeps no scoreboard entry for the copy, so it cannot
+// force it to complete before unrelated LDS reads; completion is awaited explicitly with
+// s_waitcnt vmcnt(n) (copies retire in issue order).
+__device__ inline void async_copy16(const void* sbase, uint32_t voff, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
-                 : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(gptr)
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(voff), "s"(uniform_ptr(sbase))
                  : "memory");
 }
 
@@ -304,7 +314,6 @@ __device__ inline uint32_t lds_address(const void* p) {
 }
 
 constexpr int kStageBytes = 32768;   // one K tile (64 x 256 B) + one V^T tile (128 x 128 B)
-constexpr int kVisCap = 2048;        // key tiles whose visibility words are cached in LDS
 
 // LDS tiles are unpadded (the async copy writes 1 KiB per wavefront contiguously); bank conflicts
 // are avoided by XOR-swizzling the 16-byte piece index with the row:
@@ -314,21 +323,49 @@ __device__ inline int k_lds_off(int r, int c) { return r * 256 + ((c ^ (r & 15))
 __device__ inline int v_lds_off(int d, int c) { return d * 128 + ((c ^ ((d >> 1) & 7)) << 4); }
 
 // NC = 32-row query subtiles per wavefront, NW = wavefronts per workgroup; a workgroup covers
-// 32 * NC * NW (head, position) rows of one kv head.
+// 32 * NC * NW (head, position) rows of one kv head.  LDS: two tile stages, then the visibility
+// words of the key tiles and the compacted list of tiles that hold at least one visible key.
 template <typename T, int NC, int NW>
 __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    unsigned long long* vis_lds = reinterpret_cast<unsigned long long*>(smem + 3 * kStageBytes);
-    const uint32_t smem_addr = lds_address(smem);
     constexpr int kThreads = 64 * NW;
     constexpr int kBlocksPerWave = 16 / NW;  // 1 KiB blocks of each 16 KiB tile copied by one wavefront
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, half = lane >> 5;
     const int64_t bkv = blockIdx.y;
     const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
     const int m0 = (int)blockIdx.x * p.QT;
 
-    // the query rows (one per 32-row subtile) this lane owns as MFMA column `col`
+    int m_hi = m0 + p.QT - 1;
+    if (m_hi > (int)p.Q - 1) m_hi = (int)p.Q - 1;
+    const int n_tiles = (int)((p.Nc + m_hi) / kBN) + 1;
+    const int tiles_cap = (int)(p.n_pad / kBN);
+    unsigned long long* vis_lds = reinterpret_cast<unsigned long long*>(smem + 2 * kStageBytes);
+    int* list_lds = reinterpret_cast<int*>(smem + 2 * kStageBytes + 8 * tiles_cap);
+    const uint32_t smem_addr = lds_address(smem);
+
+    // ---- work list: tiles with at least one visible key; bit 31 marks tiles that need masking
+    for (int i = tid; i < n_tiles; i += kThreads) vis_lds[i] = p.tile_vis[i];
+    __syncthreads();
+    if (wave == 0) {
+        int cnt = 0;
+        for (int base = 0; base < n_tiles; base += 64) {
+            const int t = base + lane;
+            const unsigned long long v = t < n_tiles ? vis_lds[t] : 0ull;
+            const unsigned long long bal = __ballot(v != 0ull);
+            if (v != 0ull) {
+                const bool partial = (v != ~0ull) || (t * kBN + kBN - 1 - (int)p.Nc > m0);
+                list_lds[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = t | (partial ? (int)0x80000000 : 0);
+            }
+            cnt += __popcll(bal);
+        }
+        if (lane == 0) list_lds[tiles_cap] = cnt;
+    }
+    __syncthreads();
+    const int n_work = __builtin_amdgcn_readfirstlane(list_lds[tiles_cap]);
+
+    // ---- the query rows (one per 32-row subtile) this lane owns as MFMA column `col`
     int row_m[NC];
     int64_t row_h[NC];
     bool row_ok[NC];
@@ -361,64 +398,44 @@ __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
         l_run[c] = 0.f;
     }
 
-    int m_hi = m0 + p.QT - 1;
-    if (m_hi > (int)p.Q - 1) m_hi = (int)p.Q - 1;
-    const int n_tiles = (int)((p.Nc + m_hi) / kBN) + 1;
-    const char* kbase = (const char*)p.kr + bkv * p.n_pad * kD * (int64_t)sizeof(T);
-    const char* vbase = (const char*)p.vt + bkv * p.n_pad * kD * (int64_t)sizeof(T);
-
-    for (int i = tid; i < n_tiles && i < kVisCap; i += kThreads) vis_lds[i] = p.tile_vis[i];
-    __syncthreads();
-    auto vis_of = [&](int t) -> unsigned long long {
-        return t < kVisCap ? vis_lds[t] : p.tile_vis[__builtin_amdgcn_readfirstlane(t)];
-    };
-    auto next_visible = [&](int t) {
-        while (t < n_tiles && vis_of(t) == 0ull) t++;  // uniform: all keys of a tile masked
-        return t;
-    };
-    // this lane's source offsets inside a tile, fixed for the whole kernel
-    int k_src[kBlocksPerWave], v_src[kBlocksPerWave];
+    // ---- per-lane constants of the copy (source offsets) and of the operand reads (LDS offsets)
+    uint32_t k_src[kBlocksPerWave], v_src[kBlocksPerWave];
 #pragma unroll
     for (int j = 0; j < kBlocksPerWave; j++) {
         const int blk = wave * kBlocksPerWave + j;
-        const int pk_ = blk * 64 + lane;                     // piece position inside the LDS tile
-        const int kr_ = pk_ >> 4, kc = (pk_ & 15) ^ (kr_ & 15);
+        const int pos = blk * 64 + lane;                     // piece position inside the LDS tile
+        const int kr_ = pos >> 4, kc = (pos & 15) ^ (kr_ & 15);
         k_src[j] = kr_ * 256 + kc * 16;
-        const int vd = pk_ >> 3, vc = (pk_ & 7) ^ ((vd >> 1) & 7);
+        const int vd = pos >> 3, vc = (pos & 7) ^ ((vd >> 1) & 7);
         v_src[j] = vd * 128 + vc * 16;
     }
-    auto issue = [&](int t, int stage) {
+    int k_off[8], v_off[4];  // key row `col` (+32 rows = +8192 B), dim row `col` (+32 rows = +4096 B)
+#pragma unroll
+    for (int kk = 0; kk < 8; kk++) k_off[kk] = k_lds_off(col, 2 * kk + half);
+#pragma unroll
+    for (int s = 0; s < 4; s++) v_off[s] = v_lds_off(col, 2 * s + half);
+    const char* kbase = (const char*)uniform_ptr((const char*)p.kr + bkv * p.n_pad * kD * (int64_t)sizeof(T));
+    const char* vbase = (const char*)uniform_ptr((const char*)p.vt + bkv * p.n_pad * kD * (int64_t)sizeof(T));
+
+    auto issue = [&](int t, int stage) {  // t, stage uniform
         const char* kt = kbase + (int64_t)t * (kBN * kD * (int)sizeof(T));
         const char* vtile = vbase + (int64_t)t * (kBN * kD * (int)sizeof(T));
         const uint32_t st = smem_addr + stage * kStageBytes;
 #pragma unroll
         for (int j = 0; j < kBlocksPerWave; j++) {
             const int blk = wave * kBlocksPerWave + j;
-            async_copy16(kt + k_src[j], st + blk * 1024);
-            async_copy16(vtile + v_src[j], st + 16384 + blk * 1024);
+            async_copy16(kt, k_src[j], st + blk * 1024);
+            async_copy16(vtile, v_src[j], st + 16384 + blk * 1024);
         }
     };
+    auto work = [&](int j) { return __builtin_amdgcn_readfirstlane(list_lds[j]); };
 
-    // three LDS stages: tiles t+1 and t+2 are in flight while tile t is being consumed
-    int t = next_visible(0);
-    int t1 = t < n_tiles ? next_visible(t + 1) : n_tiles;
-    int stage = 0;
-    if (t < n_tiles) issue(t, 0);
-    if (t1 < n_tiles) issue(t1, 1);
-    while (t < n_tiles) {
-        const unsigned long long vis = vis_of(t);
-        // every wavefront issues 2 * kBlocksPerWave copies per tile and they retire in order:
-        // leaving one tile's worth outstanding means tile t has landed
-        if (t1 < n_tiles) {
-            __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kBlocksPerWave));
-        } else {
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-        }
-        __syncthreads();  // everyone's pieces have landed, and the stage used two tiles ago is free
-        const int t2 = t1 < n_tiles ? next_visible(t1 + 1) : n_tiles;
-        if (t2 < n_tiles) issue(t2, stage == 0 ? 2 : stage - 1);
-        const unsigned char* k_lds = smem + stage * kStageBytes;
+    // one key tile out of LDS stage ST (compile-time so that every LDS read is register + immediate)
+    auto tile_step = [&](auto stage_tag, int entry) {
+        constexpr int ST = decltype(stage_tag)::value;
+        const unsigned char* k_lds = smem + ST * kStageBytes;
         const unsigned char* v_lds = k_lds + 16384;
+        const int t = entry & 0x7fffffff;
 
         // S^T tile: sacc[ks][c][v] = logit of key 32ks + 8(v/4) + 4half + v%4 for query column col
         f32x16 sacc[2][NC];
@@ -432,15 +449,15 @@ __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
         for (int kk = 0; kk < 8; kk++) {
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
-                const uint4 a = *reinterpret_cast<const uint4*>(k_lds + k_lds_off(32 * ks + col, 2 * kk + half));
+                const uint4 a = *reinterpret_cast<const uint4*>(k_lds + k_off[kk] + ks * 8192);
 #pragma unroll
                 for (int c = 0; c < NC; c++) sacc[ks][c] = Mma<T>::mma(a, qreg[c][kk], sacc[ks][c]);
             }
         }
 
-        // masking is needed only on tiles with hidden keys or tiles that reach past the diagonal
-        const int key0 = t * kBN;
-        if ((vis != ~0ull) || (key0 + kBN - 1 - (int)p.Nc > m0)) {
+        if (entry < 0) {  // hidden keys in the tile, or the tile reaches past the diagonal
+            const unsigned long long vis = vis_lds[t];
+            const int key0 = t * kBN;
 #pragma unroll
             for (int c = 0; c < NC; c++)
 #pragma unroll
@@ -494,7 +511,7 @@ __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
         for (int s = 0; s < 4; s++) {
 #pragma unroll
             for (int dt = 0; dt < 4; dt++) {
-                const uint4 a = *reinterpret_cast<const uint4*>(v_lds + v_lds_off(32 * dt + col, 2 * s + half));
+                const uint4 a = *reinterpret_cast<const uint4*>(v_lds + v_off[s] + dt * 4096);
 #pragma unroll
                 for (int c = 0; c < NC; c++) {
                     const uint4 bq = make_uint4(pk[c][s][0], pk[c][s][1], pk[c][s][2], pk[c][s][3]);
@@ -502,9 +519,24 @@ __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
                 }
             }
         }
-        t = t1;
-        t1 = t2;
-        stage = stage == 2 ? 0 : stage + 1;
+    };
+
+    // ---- main loop, two tiles per trip: while stage s is consumed the copy of the next tile
+    //      fills stage s^1
+    if (n_work > 0) issue(work(0) & 0x7fffffff, 0);
+    for (int j = 0; j < n_work; j += 2) {
+        const int e0 = work(j);
+        const int e1 = j + 1 < n_work ? work(j + 1) : 0;
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's pieces of tile j landed
+        __syncthreads();                     // ... everyone's did, and stage 1 is free again
+        if (j + 1 < n_work) issue(e1 & 0x7fffffff, 1);
+        tile_step(std::integral_constant<int, 0>{}, e0);
+        if (j + 1 < n_work) {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+            if (j + 2 < n_work) issue(work(j + 2) & 0x7fffffff, 0);
+            tile_step(std::integral_constant<int, 1>{}, e1);
+        }
     }
 
     // epilogue: lane owns d = 32dt + 8(v/4) + 4half + v%4 of its query row
@@ -605,7 +637,7 @@ __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
 
     // async copy assignments: the Q tile is 16 blocks of 1 KiB (4 per wavefront); wavefront 0 also
     // brings the tile's 64 normalisers, wavefront 1 its 64 weights (16 lanes x 16 bytes each)
-    int q_src[4];
+    uint32_t q_src[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int pos = (wave * 4 + j) * 64 + lane;
@@ -615,14 +647,14 @@ __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
     auto issue = [&](int step, int stage) {
         const int g = step / nmt, mt = m_first + (step % nmt) * kQT2;
         const int64_t row0 = (b * p.H + kvh * p.G + g) * p.Q + mt;
-        const char* qt = (const char*)p.qr + row0 * (kD * (int64_t)sizeof(T));
+        const char* qt = (const char*)uniform_ptr((const char*)p.qr + row0 * (kD * (int64_t)sizeof(T)));
         const uint32_t st = smem_addr + stage * kCsStage;
 #pragma unroll
-        for (int j = 0; j < 4; j++) async_copy16(qt + q_src[j], st + (wave * 4 + j) * 1024);
+        for (int j = 0; j < 4; j++) async_copy16(qt, q_src[j], st + (wave * 4 + j) * 1024);
         // every wavefront issues exactly 5 copies per step so that one vmcnt value fits all
         if (lane < 16) {
             const char* src = (wave & 1) ? (const char*)(p.w_ema + mt) : (const char*)(p.lse2 + row0);
-            async_copy16(src + lane * 16, st + 16384 + wave * 256);  // waves 2, 3 land in the dummy zone
+            async_copy16(uniform_ptr(src), lane * 16, st + 16384 + wave * 256);  // waves 2, 3: dummy zone
         }
     };
 
@@ -790,7 +822,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         fp.QT = kWgRows / G;
         fp.scale_log2 = scale_log2;
         const dim3 grid((unsigned)((mp.Q + fp.QT - 1) / fp.QT), (unsigned)(mp.B * mp.KVH));
-        const int lds = 3 * kStageBytes + kVisCap * 8;
+        const int lds = 2 * kStageBytes + (int)(n_pad / kBN) * 12 + 16;
         CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fwd_mfma_kernel<T, kNC, kNW>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         hipLaunchKernelGGL((fwd_mfma_kernel<T, kNC, kNW>), grid, dim3(64 * kNW), lds, stream, fp);
