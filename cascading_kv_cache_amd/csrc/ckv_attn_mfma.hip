@@ -589,18 +589,19 @@ struct ColsumParams {
 };
 
 constexpr int kQT2 = 64;                      // query rows per LDS tile of the column pass
-constexpr int kCsStage = 16384 + 256 + 256 + 512;   // Q tile + its lse2 + its weights + dummy landing zone
+constexpr int kCsStage = 16384 + 256 + 256;   // Q tile + its lse2 + its weights
 
 // One workgroup = one kv head x 256 keys (64 per wavefront, held in registers as the B operand of
 // S = Q K^T).  The (head, query-tile) sequence streams through a double-buffered LDS stage filled
 // by asynchronous copies; lane (col, half) owns key column `col` of each 32-key subtile, so the
 // weighted column sums never leave the lane.
 template <typename T>
-__global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
+__global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    float* wnew_lds = reinterpret_cast<float*>(smem + 3 * kCsStage);
+    float* wnew_lds = reinterpret_cast<float*>(smem + 2 * kCsStage);
     const uint32_t smem_addr = lds_address(smem);
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, half = lane >> 5;
     const int64_t bkv = blockIdx.y;
     const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
@@ -629,7 +630,8 @@ __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
     m_first = m_first / kQT2 * kQT2;
     const bool chunk_keys = key_blk + 255 >= p.Nc;  // some key of the workgroup belongs to the chunk
     const int last_nrel = (int)(key_blk + 255 - p.Nc);
-    if (chunk_keys && p.new_mode) {
+    const bool new_chunk = chunk_keys && p.new_mode;
+    if (new_chunk) {
         for (int i = tid; i < Q; i += 256) wnew_lds[i] = p.w_new[i];
     }
     const int nmt = (Q - m_first + kQT2 - 1) / kQT2;  // query tiles per head
@@ -644,36 +646,30 @@ __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
         const int r = pos >> 4, c = (pos & 15) ^ (r & 15);
         q_src[j] = r * 256 + c * 16;
     }
+    int q_off[8];  // query row `col` of the tile (+32 rows = +8192 B)
+#pragma unroll
+    for (int kk = 0; kk < 8; kk++) q_off[kk] = k_lds_off(col, 2 * kk + half);
+    const int64_t head_row0 = (b * p.H + kvh * p.G) * p.Q;
     auto issue = [&](int step, int stage) {
         const int g = step / nmt, mt = m_first + (step % nmt) * kQT2;
-        const int64_t row0 = (b * p.H + kvh * p.G + g) * p.Q + mt;
-        const char* qt = (const char*)uniform_ptr((const char*)p.qr + row0 * (kD * (int64_t)sizeof(T)));
+        const int64_t row0 = head_row0 + (int64_t)g * p.Q + mt;
+        const char* qt = (const char*)p.qr + row0 * (kD * (int64_t)sizeof(T));
         const uint32_t st = smem_addr + stage * kCsStage;
 #pragma unroll
         for (int j = 0; j < 4; j++) async_copy16(qt, q_src[j], st + (wave * 4 + j) * 1024);
-        // every wavefront issues exactly 5 copies per step so that one vmcnt value fits all
-        if (lane < 16) {
-            const char* src = (wave & 1) ? (const char*)(p.w_ema + mt) : (const char*)(p.lse2 + row0);
-            async_copy16(uniform_ptr(src), lane * 16, st + 16384 + wave * 256);  // waves 2, 3: dummy zone
+        if (wave < 2 && lane < 16) {
+            const char* src = wave ? (const char*)(p.w_ema + mt) : (const char*)(p.lse2 + row0);
+            async_copy16(src, lane * 16, st + 16384 + wave * 256);
         }
     };
 
     float acc[2] = {0.f, 0.f};
-    int stage = 0;
-    if (n_steps > 0) issue(0, 0);
-    if (n_steps > 1) issue(1, 1);
-    for (int step = 0; step < n_steps; step++) {
-        const int g = step / nmt, mt = m_first + (step % nmt) * kQT2;
-        if (step + 1 < n_steps) {
-            __builtin_amdgcn_s_waitcnt(0x0F75);  // vmcnt(5): only the next step's copies may be pending
-        } else {
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-        }
-        __syncthreads();
-        if (step + 2 < n_steps) issue(step + 2, stage == 0 ? 2 : stage - 1);
-        const unsigned char* q_lds = smem + stage * kCsStage;
+    auto tile_step = [&](auto stage_tag, int step) {
+        constexpr int ST = decltype(stage_tag)::value;
+        const unsigned char* q_lds = smem + ST * kCsStage;
         const float* lse_lds = reinterpret_cast<const float*>(q_lds + 16384);
         const float* w_lds = lse_lds + 64;
+        const int g = step / nmt, mt = m_first + (step % nmt) * kQT2;
 
         f32x16 sacc[2][2];  // [c = query subtile][ks]
 #pragma unroll
@@ -686,7 +682,7 @@ __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
         for (int kk = 0; kk < 8; kk++) {
 #pragma unroll
             for (int c = 0; c < 2; c++) {
-                const uint4 a = *reinterpret_cast<const uint4*>(q_lds + k_lds_off(32 * c + col, 2 * kk + half));
+                const uint4 a = *reinterpret_cast<const uint4*>(q_lds + q_off[kk] + c * 8192);
                 sacc[c][0] = Mma<T>::mma(a, kreg[0][kk], sacc[c][0]);
                 sacc[c][1] = Mma<T>::mma(a, kreg[1][kk], sacc[c][1]);
             }
@@ -694,7 +690,7 @@ __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
         // element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4, key column of this lane
         const bool tail = mt + kQT2 > Q;                       // rows past the chunk end
         const bool diag = chunk_keys && mt <= last_nrel;       // tile may cross the diagonal
-        if (!tail && !diag && !(chunk_keys && p.new_mode)) {
+        if (!tail && !diag && !new_chunk) {
 #pragma unroll
             for (int c = 0; c < 2; c++) {
 #pragma unroll
@@ -751,7 +747,21 @@ __global__ void __launch_bounds__(256) colsum_mfma_kernel(ColsumParams p) {
                 acc[ks] = 0.f;
             }
         }
-        stage = stage == 2 ? 0 : stage + 1;
+    };
+
+    // two steps per trip: while stage s is consumed the copy of the next step fills stage s^1
+    if (n_steps > 0) issue(0, 0);
+    for (int step = 0; step < n_steps; step += 2) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        if (step + 1 < n_steps) issue(step + 1, 1);
+        tile_step(std::integral_constant<int, 0>{}, step);
+        if (step + 1 < n_steps) {
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+            if (step + 2 < n_steps) issue(step + 2, 0);
+            tile_step(std::integral_constant<int, 1>{}, step + 1);
+        }
     }
     if (n_steps == 0) {  // no query can see these keys (only possible for padding blocks)
         for (int g = 0; g < p.G; g++)
@@ -838,7 +848,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         cp.new_mode = mp.new_mode;
         cp.scale_log2 = scale_log2;
         const dim3 grid((unsigned)((n + 255) / 256), (unsigned)(mp.B * mp.KVH));
-        const int lds = 3 * kCsStage + (int)mp.Q * 4;
+        const int lds = 2 * kCsStage + (int)mp.Q * 4;
         CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(colsum_mfma_kernel<T>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         hipLaunchKernelGGL(colsum_mfma_kernel<T>, grid, dim3(256), lds, stream, cp);
