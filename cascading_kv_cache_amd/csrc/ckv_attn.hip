@@ -57,7 +57,12 @@ void contiguous_strides(int64_t* st, int64_t d1, int64_t d2, int64_t d3) {
 extern "C" int64_t ckv_attn_workspace_bytes(int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t D, int64_t num_sink,
                                             int64_t S, int32_t dtype) {
     if (B <= 0 || H <= 0 || KVH <= 0 || Q <= 0 || D <= 0 || num_sink < 0 || S < 0) return 0;
-    return ckv::carve_attn(nullptr, B, H, KVH, Q, D, num_sink, S, dtype).bytes;
+    int64_t bytes = ckv::carve_attn(nullptr, B, H, KVH, Q, D, num_sink, S, dtype).bytes;
+    if (Q == 1 && D == 128) {
+        const int64_t dec = ckv::decode_workspace_bytes(B, H, KVH, num_sink, S);
+        if (dec > bytes) bytes = dec;
+    }
+    return bytes;
 }
 
 extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
@@ -74,8 +79,10 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
     if (a.num_sink > 0 && (!a.sink_k || !a.sink_v || !a.sink_mask || !a.sink_pos)) return CKV_ERR_NULL;
     if (a.S > 0 && (!a.cache_k || !a.cache_v || !a.mask || !a.pos)) return CKV_ERR_NULL;
     if (!(a.beta > 0.0) || !(a.beta <= 1.0)) return CKV_ERR_SHAPE;
+    if (!a.workspace || a.workspace_bytes < ckv_attn_workspace_bytes(a.B, a.H, a.KVH, a.Q, a.D, a.num_sink, a.S, a.dtype))
+        return CKV_ERR_WORKSPACE;
+    if (decode_supported(a)) return launch_decode(a, stream);
     AttnWorkspace w = carve_attn(a.workspace, a.B, a.H, a.KVH, a.Q, a.D, a.num_sink, a.S, a.dtype);
-    if (!a.workspace || a.workspace_bytes < w.bytes) return CKV_ERR_WORKSPACE;
 
     const int64_t N = a.num_sink + a.S + a.Q;
     const bool want_scores = a.cache_s || a.new_scores;

@@ -1,0 +1,477 @@
+// Single-token decode attention (Q == 1, head_dim 128): bandwidth-bound kernels.
+//
+//   decode_q      rotate the B*H query rows, fold softmax scale * log2(e) in, keep them as fp32.
+//   decode_main   grid (key tiles of 128, groups of (batch, kv-head)).  A workgroup computes the
+//                 cos/sin of its 128 keys ONCE (registers) and then streams the K and V rows of
+//                 every (batch, kv-head) of its group: each row is read exactly once, 16 lanes per
+//                 row with 8-byte pieces, K is rotated in registers, the G query heads of the
+//                 group share the row.  Outputs: raw logits (log2 domain) per key and head, and one
+//                 (max, sum, weighted V) partial per (head, tile).
+//   decode_tail   combine the partials of a row: out, log-sum-exp.
+//   decode_scores P = exp2(logit - lse) exactly, head reduction, score EMA of every slot and the
+//                 new token's own score (cascade_attention.py:315-330 with q_len == 1).
+#include "ckv_attn_internal.h"
+
+namespace ckv {
+namespace {
+
+constexpr int kD = 128;
+constexpr int kTK = 128;     // keys per workgroup tile
+constexpr int kSteps = 8;    // a wavefront covers 32 keys as 8 steps of 4 keys (16 lanes per key)
+
+template <typename T>
+__device__ inline float round_t(float v) {
+    return Elem<T>::to_float(Elem<T>::from_float(v));
+}
+
+// all-reduce (sum) inside each row of 16 lanes with DPP: quad xor 1, quad xor 2, half mirror, mirror
+__device__ inline float row16_sum(float x) {
+    int v = __float_as_int(x);
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true));
+    v = __float_as_int(x);
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true));
+    v = __float_as_int(x);
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true));
+    v = __float_as_int(x);
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true));
+    return x;
+}
+
+// 4 consecutive elements of a row: raw load now, widening to fp32 later
+template <typename T>
+struct Piece;
+template <>
+struct Piece<float> {
+    using Raw = float4;
+    __device__ static void unpack(const Raw& v, float out[4]) { out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w; }
+};
+template <>
+struct Piece<__hip_bfloat16> {
+    using Raw = uint2;
+    __device__ static void unpack(const Raw& v, float out[4]) {
+        out[0] = __uint_as_float(v.x << 16); out[1] = __uint_as_float(v.x & 0xffff0000u);
+        out[2] = __uint_as_float(v.y << 16); out[3] = __uint_as_float(v.y & 0xffff0000u);
+    }
+};
+template <>
+struct Piece<__half> {
+    using Raw = uint2;
+    __device__ static void unpack(const Raw& v, float out[4]) {
+        const float2 fa = __half22float2(*reinterpret_cast<const __half2*>(&v.x));
+        const float2 fb = __half22float2(*reinterpret_cast<const __half2*>(&v.y));
+        out[0] = fa.x; out[1] = fa.y; out[2] = fb.x; out[3] = fb.y;
+    }
+};
+
+struct DecodeParams {
+    ckv_attn_args a;
+    float* qrot;       // (B, H, 128) rotated, pre-scaled queries
+    float* logits;     // (B, KVH, N, G) log2-domain logits, -inf for hidden keys
+    float* part_ml;    // (B, H, tiles, 2)
+    float* part_o;     // (B, H, tiles, 128)
+    float* lse2;       // (B, H)
+    int64_t N;         // num_sink + S + 1
+    int tiles;
+    int shared_pos;
+    float scale_log2;
+};
+
+template <typename T>
+__global__ void decode_q_kernel(DecodeParams p) {
+    const ckv_attn_args& a = p.a;
+    const int64_t row = blockIdx.x;  // b * H + h
+    const int j = threadIdx.x;       // 0..63: rotation pair
+    const int64_t b = row / a.H, h = row % a.H;
+    const T* q = (const T*)a.q + b * a.q_stride[0] + h * a.q_stride[1];
+    const float f = a.inv_freq ? a.inv_freq[j] : 1.0f / powf(a.rope_theta, (float)(2 * j) / (float)kD);
+    float sn, cs;
+    sincosf(__fmul_rn((float)a.q_pos[0], f), &sn, &cs);
+    const float x1 = Elem<T>::to_float(q[j * a.q_stride[3]]), x2 = Elem<T>::to_float(q[(j + 64) * a.q_stride[3]]);
+    // the eager path rotates in the tensor dtype (cascade_attention.py:31-35)
+    const float r1 = round_t<T>(x1 * cs - x2 * sn), r2 = round_t<T>(x2 * cs + x1 * sn);
+    p.qrot[row * kD + j] = r1 * p.scale_log2;
+    p.qrot[row * kD + 64 + j] = r2 * p.scale_log2;
+}
+
+// source row of key n: sink, cache slot or the new token
+template <typename T>
+__device__ inline bool key_source(const ckv_attn_args& a, int64_t n, int64_t b, int64_t kvh, const T*& kp, const T*& vp,
+                                  int64_t& pos) {
+    const int64_t NS = a.num_sink, S = a.S;
+    if (n < NS) {
+        const int64_t off = b * a.sink_stride[0] + kvh * a.sink_stride[1] + n * a.sink_stride[2];
+        kp = (const T*)a.sink_k + off;
+        vp = (const T*)a.sink_v + off;
+        pos = a.sink_pos[b * a.sink_pos_stride[0] + kvh * a.sink_pos_stride[1] + n];
+        return a.sink_mask[n] == 0;
+    }
+    if (n < NS + S) {
+        const int64_t slot = n - NS;
+        const int64_t off = b * a.cache_stride[0] + kvh * a.cache_stride[1] + slot * a.cache_stride[2];
+        kp = (const T*)a.cache_k + off;
+        vp = (const T*)a.cache_v + off;
+        pos = a.pos[b * a.pos_stride[0] + kvh * a.pos_stride[1] + slot] + a.pos_shift;
+        return a.mask[slot] == 0;
+    }
+    const int64_t off = b * a.kv_new_stride[0] + kvh * a.kv_new_stride[1];
+    kp = (const T*)a.k_new + off;
+    vp = (const T*)a.v_new + off;
+    pos = a.q_pos[0];
+    return true;
+}
+
+template <typename T, int G>
+__global__ void __launch_bounds__(256) decode_main_kernel(DecodeParams p) {
+    extern __shared__ __align__(16) float red[];  // [16][G][128] weighted-V partials, [16][G] max, [16][G] sum
+    float* red_o = red;
+    float* red_m = red + 16 * G * kD;
+    float* red_l = red_m + 16 * G;
+    using Raw = typename Piece<T>::Raw;
+    const ckv_attn_args& a = p.a;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int kg = lane >> 4, j = lane & 15;       // key within a step, piece index inside the row
+    const int grp = wave * 4 + kg;                 // 16-lane group id, 0..15
+    const int64_t tile = blockIdx.x;
+    const int64_t nbh = a.B * a.KVH;
+
+    // cos/sin of this lane's 8 keys x 4 frequencies, computed once when every (b, kvh) shares them
+    float cs[kSteps][4], sn[kSteps][4];
+    if (p.shared_pos) {
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) {
+            const int64_t n = tile * kTK + wave * 32 + s * 4 + kg;
+            const T *kp, *vp;
+            int64_t pos = 0;
+            if (n < p.N) key_source<T>(a, n, 0, 0, kp, vp, pos);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int f = 4 * j + e;
+                const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
+                sincosf(__fmul_rn((float)pos, fr), &sn[s][e], &cs[s][e]);
+            }
+        }
+    }
+
+    for (int64_t bh = blockIdx.y; bh < nbh; bh += gridDim.y) {
+        const int64_t b = bh / a.KVH, kvh = bh % a.KVH;
+        // ---- issue every row read of this (b, kvh) up front: 8 keys x (K, V) x 2 pieces
+        Raw kraw[kSteps][2], vraw[kSteps][2];
+        bool vis[kSteps];
+        int64_t posv[kSteps];
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) {
+            const int64_t n = tile * kTK + wave * 32 + s * 4 + kg;
+            const T *kp = nullptr, *vp = nullptr;
+            posv[s] = 0;
+            vis[s] = n < p.N && key_source<T>(a, n, b, kvh, kp, vp, posv[s]);
+            if (vis[s]) {
+                kraw[s][0] = *reinterpret_cast<const Raw*>(kp + 4 * j);
+                kraw[s][1] = *reinterpret_cast<const Raw*>(kp + 64 + 4 * j);
+                vraw[s][0] = *reinterpret_cast<const Raw*>(vp + 4 * j);
+                vraw[s][1] = *reinterpret_cast<const Raw*>(vp + 64 + 4 * j);
+            }
+        }
+        // this lane's 8 dims of the G rotated queries: [4j, 4j+4) and [64+4j, 64+4j+4)
+        float qa[G][4], qb[G][4];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const float* qr = p.qrot + ((b * a.H) + kvh * G + g) * kD;
+            const float4 va = *reinterpret_cast<const float4*>(qr + 4 * j);
+            const float4 vb = *reinterpret_cast<const float4*>(qr + 64 + 4 * j);
+            qa[g][0] = va.x; qa[g][1] = va.y; qa[g][2] = va.z; qa[g][3] = va.w;
+            qb[g][0] = vb.x; qb[g][1] = vb.y; qb[g][2] = vb.z; qb[g][3] = vb.w;
+        }
+        // ---- phase 1: logits of the 8 keys of this 16-lane group
+        float sreg[kSteps][G];
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) {
+            float ka[4] = {0.f, 0.f, 0.f, 0.f}, kb[4] = {0.f, 0.f, 0.f, 0.f};
+            if (vis[s]) {
+                Piece<T>::unpack(kraw[s][0], ka);
+                Piece<T>::unpack(kraw[s][1], kb);
+            }
+            float acc[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) acc[g] = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float c_ = cs[s][e], s_ = sn[s][e];
+                if (!p.shared_pos) {
+                    const int f = 4 * j + e;
+                    const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
+                    sincosf(__fmul_rn((float)posv[s], fr), &s_, &c_);
+                }
+                const float ra = ka[e] * c_ - kb[e] * s_;
+                const float rb = kb[e] * c_ + ka[e] * s_;
+#pragma unroll
+                for (int g = 0; g < G; g++) acc[g] = fmaf(ra, qa[g][e], fmaf(rb, qb[g][e], acc[g]));
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float tot = row16_sum(acc[g]);
+                sreg[s][g] = vis[s] ? tot : -INFINITY;
+            }
+            const int64_t n = tile * kTK + wave * 32 + s * 4 + kg;
+            if (j == 0 && n < p.N) {
+                float* lg = p.logits + ((b * a.KVH + kvh) * p.N + n) * G;
+#pragma unroll
+                for (int g = 0; g < G; g++) lg[g] = sreg[s][g];
+            }
+        }
+        // ---- phase 2: softmax partial of the group and its weighted V sum
+        float mg[G], lgp[G], o[G][8];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float m = sreg[0][g];
+#pragma unroll
+            for (int s = 1; s < kSteps; s++) m = fmaxf(m, sreg[s][g]);
+            mg[g] = m;
+            lgp[g] = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[g][e] = 0.f;
+        }
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) {
+            if (!vis[s]) continue;
+            float va[4], vb[4];
+            Piece<T>::unpack(vraw[s][0], va);
+            Piece<T>::unpack(vraw[s][1], vb);
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float pe = __builtin_amdgcn_exp2f(sreg[s][g] - mg[g]);  // mg is finite: the key is visible
+                lgp[g] += pe;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    o[g][e] = fmaf(pe, va[e], o[g][e]);
+                    o[g][4 + e] = fmaf(pe, vb[e], o[g][4 + e]);
+                }
+            }
+        }
+        // ---- combine the 16 groups of the workgroup
+        __syncthreads();  // the previous (b, kvh) has been written out
+        if (j == 0) {
+#pragma unroll
+            for (int g = 0; g < G; g++) red_m[grp * G + g] = mg[g];
+        }
+        __syncthreads();
+        float mt[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float m = red_m[g];
+#pragma unroll
+            for (int r = 1; r < 16; r++) m = fmaxf(m, red_m[r * G + g]);
+            mt[g] = m;
+            const float sc = mg[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mg[g] - m);
+            if (j == 0) red_l[grp * G + g] = lgp[g] * sc;
+            float* ro = red_o + (grp * G + g) * kD;
+            *reinterpret_cast<float4*>(ro + 4 * j) = make_float4(o[g][0] * sc, o[g][1] * sc, o[g][2] * sc, o[g][3] * sc);
+            *reinterpret_cast<float4*>(ro + 64 + 4 * j) =
+                make_float4(o[g][4] * sc, o[g][5] * sc, o[g][6] * sc, o[g][7] * sc);
+        }
+        __syncthreads();
+        for (int i = tid; i < G * kD; i += 256) {
+            const int g = i / kD, d = i % kD;
+            float acc = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc += red_o[(r * G + g) * kD + d];
+            p.part_o[(((b * a.H) + kvh * G + g) * p.tiles + tile) * kD + d] = acc;
+        }
+        if (tid < G) {
+            float l = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) l += red_l[r * G + tid];
+            float* ml = p.part_ml + (((b * a.H) + kvh * G + tid) * p.tiles + tile) * 2;
+            ml[0] = mt[tid];
+            ml[1] = l;
+        }
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(128) decode_tail_kernel(DecodeParams p) {
+    const ckv_attn_args& a = p.a;
+    const int64_t row = blockIdx.x;  // b * H + h
+    const int d = threadIdx.x;
+    const float* ml = p.part_ml + row * p.tiles * 2;
+    float M = -INFINITY;
+    for (int t = 0; t < p.tiles; t++) M = fmaxf(M, ml[2 * t]);
+    float L = 0.f, o = 0.f;
+    for (int t = 0; t < p.tiles; t++) {
+        const float m = ml[2 * t];
+        if (m == -INFINITY) continue;
+        const float sc = __builtin_amdgcn_exp2f(m - M);
+        L = fmaf(ml[2 * t + 1], sc, L);
+        o = fmaf(p.part_o[(row * p.tiles + t) * kD + d], sc, o);
+    }
+    const int64_t b = row / a.H, h = row % a.H;
+    T* out = (T*)a.out + b * a.out_stride[0] + h * a.out_stride[1];
+    out[d * a.out_stride[3]] = Elem<T>::from_float(o / L);
+    if (d == 0) {
+        const float l2 = M + __builtin_amdgcn_logf(L);
+        p.lse2[row] = l2;
+        if (a.lse) a.lse[row] = l2 * 0.6931471805599453f;
+    }
+}
+
+template <typename T, int G>
+__device__ inline float reduce_group(const float* v, int n, int mode) {
+    if (mode == CKV_REDUCE_MAX) {
+        float r = v[0];
+        for (int i = 1; i < n; i++) r = fmaxf(r, v[i]);
+        return r;
+    }
+    if (mode == CKV_REDUCE_MEAN) {
+        float r = 0.f;
+        for (int i = 0; i < n; i++) r = __fadd_rn(r, v[i]);
+        return round_t<T>(r / (float)n);
+    }
+    float tmp[128];
+    for (int i = 0; i < n; i++) {
+        const float x = v[i];
+        int k = i;
+        while (k > 0 && tmp[k - 1] > x) {
+            tmp[k] = tmp[k - 1];
+            k--;
+        }
+        tmp[k] = x;
+    }
+    return tmp[(n - 1) / 2];
+}
+
+// one thread per (b, kvh, key): P of the G (or all H) heads, dtype rounding like the eager path
+// (cascade_attention.py:319-323 with a single query row), head reduction, EMA / new-token score
+template <typename T, int G>
+__global__ void decode_scores_kernel(DecodeParams p, float w_one, float beta_pow) {
+    const ckv_attn_args& a = p.a;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t per = a.S + 1;
+    if (idx >= a.B * a.KVH * per) return;
+    const int64_t i = idx % per, kvh = (idx / per) % a.KVH, b = idx / (per * a.KVH);
+    const int64_t n = a.num_sink + i;
+    const bool is_new = i == a.S;
+    float vals[128];
+    int cnt = 0;
+    const int64_t kv0 = a.homogeneous_heads ? 0 : kvh, kv1 = a.homogeneous_heads ? a.KVH : kvh + 1;
+    for (int64_t kv = kv0; kv < kv1; kv++) {
+        const float* lg = p.logits + ((b * a.KVH + kv) * p.N + n) * G;
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            const float pt = round_t<T>(__builtin_amdgcn_exp2f(lg[g] - p.lse2[b * a.H + kv * G + g]));
+            // cached slots: fp32 product, cast; the new token: product in the tensor dtype
+            vals[cnt++] = round_t<T>(__fmul_rn(pt, is_new ? round_t<T>(w_one) : w_one));
+        }
+    }
+    const float red = reduce_group<T, G>(vals, cnt, a.head_reduction);
+    if (is_new) {
+        if (a.new_scores)
+            *((T*)a.new_scores + b * a.new_scores_stride[0] + kvh * a.new_scores_stride[1]) = Elem<T>::from_float(red);
+    } else if (a.cache_s) {
+        T* cs = (T*)a.cache_s + b * a.cache_s_stride[0] + kvh * a.cache_s_stride[1] + i * a.cache_s_stride[2];
+        const float decayed = round_t<T>(__fmul_rn(beta_pow, Elem<T>::to_float(*cs)));
+        *cs = Elem<T>::from_float(__fadd_rn(decayed, red));
+    }
+}
+
+template <typename T, int G>
+int run_decode(const DecodeParams& p, hipStream_t stream) {
+    const ckv_attn_args& a = p.a;
+    {
+        StageScope sc(CKV_STAGE_PREP, stream);
+        hipLaunchKernelGGL(decode_q_kernel<T>, dim3((unsigned)(a.B * a.H)), dim3(64), 0, stream, p);
+        CKV_HIP_TRY(hipGetLastError());
+    }
+    {
+        StageScope sc(CKV_STAGE_DECODE, stream);
+        const int64_t nbh = a.B * a.KVH;
+        // enough workgroups to fill the chip, few enough that cos/sin are amortised over many rows
+        int64_t groups = p.shared_pos ? (2048 + p.tiles - 1) / p.tiles : nbh;
+        if (groups < 1) groups = 1;
+        if (groups > nbh) groups = nbh;
+        const int lds = (16 * G * kD + 32 * G) * (int)sizeof(float);
+        if (lds > 48 * 1024) {
+            CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_main_kernel<T, G>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        }
+        hipLaunchKernelGGL((decode_main_kernel<T, G>), dim3((unsigned)p.tiles, (unsigned)groups), dim3(256), lds, stream,
+                           p);
+        CKV_HIP_TRY(hipGetLastError());
+    }
+    {
+        StageScope sc(CKV_STAGE_DECODE_TAIL, stream);
+        hipLaunchKernelGGL(decode_tail_kernel<T>, dim3((unsigned)(a.B * a.H)), dim3(128), 0, stream, p);
+        CKV_HIP_TRY(hipGetLastError());
+        if (a.cache_s || a.new_scores) {
+            // w_ema[0] == w_new[0] == (1 - beta) for a single query row; the new token's weight is
+            // built in the tensor dtype (cascade_attention.py:270-276)
+            const float w_one = (float)(1.0 - a.beta);
+            const int64_t items = a.B * a.KVH * (a.S + 1);
+            hipLaunchKernelGGL((decode_scores_kernel<T, G>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream,
+                               p, w_one, (float)a.beta);
+            CKV_HIP_TRY(hipGetLastError());
+        }
+    }
+    return CKV_OK;
+}
+
+template <typename T>
+int run_decode_g(const DecodeParams& p, int G, hipStream_t stream) {
+    switch (G) {
+        case 1: return run_decode<T, 1>(p, stream);
+        case 2: return run_decode<T, 2>(p, stream);
+        case 4: return run_decode<T, 4>(p, stream);
+        case 7: return run_decode<T, 7>(p, stream);
+        case 8: return run_decode<T, 8>(p, stream);
+        default: return CKV_ERR_UNSUPPORTED;
+    }
+}
+
+inline bool aligned(const void* p, int64_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+}  // namespace
+
+bool decode_supported(const ckv_attn_args& a) {
+    if (a.Q != 1 || a.D != kD) return false;
+    const int64_t G = a.H / a.KVH;
+    if (!(G == 1 || G == 2 || G == 4 || G == 7 || G == 8)) return false;
+    if ((a.homogeneous_heads ? a.H : G) > 128) return false;
+    const int64_t es = elem_bytes(a.dtype), vec = 4 * es;
+    // rows are read as 4-element vectors
+    if (a.cache_stride[3] != 1 || a.kv_new_stride[3] != 1 || (a.num_sink > 0 && a.sink_stride[3] != 1)) return false;
+    if (!aligned(a.cache_k, vec) || !aligned(a.cache_v, vec) || !aligned(a.k_new, vec) || !aligned(a.v_new, vec)) return false;
+    if (a.num_sink > 0 && (!aligned(a.sink_k, vec) || !aligned(a.sink_v, vec))) return false;
+    for (int i = 0; i < 3; i++) {
+        if ((a.cache_stride[i] * es) % vec || (a.kv_new_stride[i] * es) % vec) return false;
+        if (a.num_sink > 0 && (a.sink_stride[i] * es) % vec) return false;
+    }
+    return true;
+}
+
+int64_t decode_workspace_bytes(int64_t B, int64_t H, int64_t KVH, int64_t num_sink, int64_t S) {
+    const int64_t N = num_sink + S + 1, tiles = (N + kTK - 1) / kTK, G = H / KVH;
+    return align_up(B * H * kD * 4, 256) + align_up(B * KVH * N * G * 4, 256) + align_up(B * H * tiles * 2 * 4, 256) +
+           align_up(B * H * tiles * kD * 4, 256) + align_up(B * H * 4, 256);
+}
+
+int launch_decode(const ckv_attn_args& a, hipStream_t stream) {
+    DecodeParams p;
+    p.a = a;
+    p.N = a.num_sink + a.S + 1;
+    p.tiles = (int)((p.N + kTK - 1) / kTK);
+    const int64_t G = a.H / a.KVH;
+    char* w = reinterpret_cast<char*>(a.workspace);
+    p.qrot = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * kD * 4, 256);
+    p.logits = reinterpret_cast<float*>(w); w += align_up(a.B * a.KVH * p.N * G * 4, 256);
+    p.part_ml = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * p.tiles * 2 * 4, 256);
+    p.part_o = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * p.tiles * kD * 4, 256);
+    p.lse2 = reinterpret_cast<float*>(w);
+    p.shared_pos = a.sink_pos_stride[0] == 0 && a.sink_pos_stride[1] == 0 && a.pos_stride[0] == 0 && a.pos_stride[1] == 0;
+    p.scale_log2 = a.scale * 1.4426950408889634f;
+    switch (a.dtype) {
+        case CKV_F32: return run_decode_g<float>(p, (int)G, stream);
+        case CKV_F16: return run_decode_g<__half>(p, (int)G, stream);
+        case CKV_BF16: return run_decode_g<__hip_bfloat16>(p, (int)G, stream);
+        default: return CKV_ERR_DTYPE;
+    }
+}
+
+}  // namespace ckv

@@ -102,4 +102,9 @@ bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH, int64_t Q);
 int64_t mfma_n_pad(int64_t n);
 int launch_mfma(const MfmaProblem& p, hipStream_t stream);
 
+// ---- single-token decode family (Q == 1, head_dim 128) ----
+bool decode_supported(const ckv_attn_args& a);
+int64_t decode_workspace_bytes(int64_t B, int64_t H, int64_t KVH, int64_t num_sink, int64_t S);
+int launch_decode(const ckv_attn_args& a, hipStream_t stream);
+
 }  // namespace ckv

@@ -132,6 +132,43 @@ def test_mfma_prefill_head128(H, KVH, Q, W, C, NS, eager, dtype):
     print(f"{flips}/{compared} slots chose a different token")
 
 
+@pytest.mark.parametrize("H,KVH,W,C,NS,eager,dtype", [
+    (8, 2, 64, 4, 8, True, torch.bfloat16),      # G = 4
+    (14, 2, 32, 4, 4, False, torch.bfloat16),    # G = 7
+    (4, 4, 32, 2, 4, True, torch.float16),       # G = 1
+    (16, 2, 16, 8, 64, True, torch.bfloat16),    # G = 8
+    (8, 4, 64, 2, 6, True, torch.float32),       # G = 2, float32
+])
+def test_decode_head128(H, KVH, W, C, NS, eager, dtype):
+    """q == 1 with head_dim 128 takes the bandwidth-bound decode kernels: fill part of the cache
+    with a few chunks, then run single-token steps (cache still filling, then evicting)."""
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
+
+    B, D = 2, 128
+    gpu, cpu = make_pair(B, KVH, D, NS, W, C, dtype, eager=eager)
+    layer = OracleCascadeAttention(H, KVH, D, rope_theta=5e5)
+    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    gen = torch.Generator().manual_seed(21)
+    steps = [W * C // 2 + NS, 17] + [1] * (W * C // 2 + 40)
+    for c, qn in enumerate(steps):
+        q = (torch.randn(B, H, qn, D, generator=gen) * 0.7).to(dtype)
+        k = (torch.randn(B, KVH, qn, D, generator=gen) * 0.7).to(dtype)
+        v = (torch.randn(B, KVH, qn, D, generator=gen) * 0.7).to(dtype)
+        push_state(gpu, cpu)
+        out_g, new_g = cascade_attention(q.cuda(), k.cuda(), v.cuda(), gpu, 0, inv_freq)
+        if c == 0:
+            layer.query_pos = None
+        out_c = layer.forward(q, k, v, cpu)
+        torch.cuda.synchronize()
+        err = (out_g.float().cpu() - out_c.float()).abs().max().item()
+        assert err <= tol(dtype), f"step {c} (q={qn}): out max err {err:.3e}"
+        assert_scores_close(new_g, layer.last_new_scores[:, :KVH], dtype, f"step {c} new-token scores")
+        for name in META:
+            assert torch.equal(getattr(gpu, name)[0].cpu(), getattr(cpu, name)), f"step {c}: {name}"
+        if bool((gpu.og_pos[0].cpu() == cpu.og_pos).all()):
+            assert_scores_close(gpu.score_cache[0], cpu.score_cache, dtype, f"step {c} score cache")
+
+
 def dense_reference(q, k, v, mask, sm_scale):
     n_ctx, n_kv = q.size(2), k.size(2)
     logits = torch.matmul(q.float(), k.float().transpose(2, 3)) * sm_scale
