@@ -12,6 +12,8 @@
 //                 new token's own score (cascade_attention.py:315-330 with q_len == 1).
 #include "ckv_attn_internal.h"
 
+#include <type_traits>
+
 namespace ckv {
 namespace {
 
@@ -66,6 +68,7 @@ struct Piece<__half> {
 struct DecodeParams {
     ckv_attn_args a;
     float* qrot;       // (B, H, 128) rotated, pre-scaled queries
+    void* qrot_t;      // (B, H, 128) rotated queries in the tensor dtype (MFMA operand)
     float* logits;     // (B, KVH, N, G) log2-domain logits, -inf for hidden keys
     float* part_ml;    // (B, H, tiles, 2)
     float* part_o;     // (B, H, tiles, 128)
@@ -91,6 +94,8 @@ __global__ void decode_q_kernel(DecodeParams p) {
     const float r1 = round_t<T>(x1 * cs - x2 * sn), r2 = round_t<T>(x2 * cs + x1 * sn);
     p.qrot[row * kD + j] = r1 * p.scale_log2;
     p.qrot[row * kD + 64 + j] = r2 * p.scale_log2;
+    ((T*)p.qrot_t)[row * kD + j] = Elem<T>::from_float(r1);
+    ((T*)p.qrot_t)[row * kD + 64 + j] = Elem<T>::from_float(r2);
 }
 
 // source row of key n: sink, cache slot or the new token
@@ -139,7 +144,7 @@ __global__ void __launch_bounds__(256) decode_main_kernel(DecodeParams p) {
     if (p.shared_pos) {
 #pragma unroll
         for (int s = 0; s < kSteps; s++) {
-            const int64_t n = tile * kTK + wave * 32 + s * 4 + kg;
+            const int64_t n = tile * kTK + wave * (4 * kSteps) + s * 4 + kg;
             const T *kp, *vp;
             int64_t pos = 0;
             if (n < p.N) key_source<T>(a, n, 0, 0, kp, vp, pos);
@@ -160,7 +165,7 @@ __global__ void __launch_bounds__(256) decode_main_kernel(DecodeParams p) {
         int64_t posv[kSteps];
 #pragma unroll
         for (int s = 0; s < kSteps; s++) {
-            const int64_t n = tile * kTK + wave * 32 + s * 4 + kg;
+            const int64_t n = tile * kTK + wave * (4 * kSteps) + s * 4 + kg;
             const T *kp = nullptr, *vp = nullptr;
             posv[s] = 0;
             vis[s] = n < p.N && key_source<T>(a, n, b, kvh, kp, vp, posv[s]);
@@ -211,7 +216,7 @@ __global__ void __launch_bounds__(256) decode_main_kernel(DecodeParams p) {
                 const float tot = row16_sum(acc[g]);
                 sreg[s][g] = vis[s] ? tot : -INFINITY;
             }
-            const int64_t n = tile * kTK + wave * 32 + s * 4 + kg;
+            const int64_t n = tile * kTK + wave * (4 * kSteps) + s * 4 + kg;
             if (j == 0 && n < p.N) {
                 float* lg = p.logits + ((b * a.KVH + kvh) * p.N + n) * G;
 #pragma unroll
@@ -233,6 +238,275 @@ __global__ void __launch_bounds__(256) decode_main_kernel(DecodeParams p) {
 #pragma unroll
         for (int s = 0; s < kSteps; s++) {
             if (!vis[s]) continue;
+            float va[4], vb[4];
+            Piece<T>::unpack(vraw[s][0], va);
+            Piece<T>::unpack(vraw[s][1], vb);
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                const float pe = __builtin_amdgcn_exp2f(sreg[s][g] - mg[g]);  // mg is finite: the key is visible
+                lgp[g] += pe;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    o[g][e] = fmaf(pe, va[e], o[g][e]);
+                    o[g][4 + e] = fmaf(pe, vb[e], o[g][4 + e]);
+                }
+            }
+        }
+        // ---- combine the 16 groups of the workgroup
+        __syncthreads();  // the previous (b, kvh) has been written out
+        if (j == 0) {
+#pragma unroll
+            for (int g = 0; g < G; g++) red_m[grp * G + g] = mg[g];
+        }
+        __syncthreads();
+        float mt[G];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float m = red_m[g];
+#pragma unroll
+            for (int r = 1; r < 16; r++) m = fmaxf(m, red_m[r * G + g]);
+            mt[g] = m;
+            const float sc = mg[g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mg[g] - m);
+            if (j == 0) red_l[grp * G + g] = lgp[g] * sc;
+            float* ro = red_o + (grp * G + g) * kD;
+            *reinterpret_cast<float4*>(ro + 4 * j) = make_float4(o[g][0] * sc, o[g][1] * sc, o[g][2] * sc, o[g][3] * sc);
+            *reinterpret_cast<float4*>(ro + 64 + 4 * j) =
+                make_float4(o[g][4] * sc, o[g][5] * sc, o[g][6] * sc, o[g][7] * sc);
+        }
+        __syncthreads();
+        for (int i = tid; i < G * kD; i += 256) {
+            const int g = i / kD, d = i % kD;
+            float acc = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc += red_o[(r * G + g) * kD + d];
+            p.part_o[(((b * a.H) + kvh * G + g) * p.tiles + tile) * kD + d] = acc;
+        }
+        if (tid < G) {
+            float l = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) l += red_l[r * G + tid];
+            float* ml = p.part_ml + (((b * a.H) + kvh * G + tid) * p.tiles + tile) * 2;
+            ml[0] = mt[tid];
+            ml[1] = l;
+        }
+    }
+}
+
+// ---- 16-bit dtypes: the logits come from v_mfma_f32_16x16x32 (16 head rows, G real, x 16 keys),
+// so the dot products cost no vector ALU work and need no cross-lane reduction.  Lane
+// (key = lane % 16, kq = lane / 16) holds dims 32*ks + 8*kq + [0, 8) of its key for ks = 0..3:
+// the rotation partner of dim d (d + 64) is the same lane's ks + 2 piece.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+template <typename T>
+struct Mma16;
+template <>
+struct Mma16<__hip_bfloat16> {
+    __device__ static f32x4 mma(uint4 a, uint4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
+                                                       0, 0, 0);
+    }
+    __device__ static float lo(uint32_t w) { return __uint_as_float(w << 16); }
+    __device__ static float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+    __device__ static uint32_t pack2(float a, float b) {
+        f32x2_t f = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+    }
+};
+template <>
+struct Mma16<__half> {
+    __device__ static f32x4 mma(uint4 a, uint4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0,
+                                                      0, 0);
+    }
+    __device__ static float lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2_t, w)[0]; }
+    __device__ static float hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2_t, w)[1]; }
+    __device__ static uint32_t pack2(float a, float b) {
+        f32x2_t f = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2_t));
+    }
+};
+
+template <typename T, int G>
+__global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p) {
+    extern __shared__ __align__(16) float red[];  // [16][G][128] partials, [16][G] max, [16][G] sum, [4][32][8] logits
+    float* red_o = red;
+    float* red_m = red + 16 * G * kD;
+    float* red_l = red_m + 16 * G;
+    float* s_lds = red_l + 16 * G;
+    using Raw = typename Piece<T>::Raw;
+    const ckv_attn_args& a = p.a;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int kg = lane >> 4, j = lane & 15;  // phase 2: key within a step, piece index inside the row
+    const int grp = wave * 4 + kg;
+    const int key16 = lane & 15, kq = lane >> 4;  // phase 1: MFMA column (key) and k-quarter
+    const int64_t tile = blockIdx.x;
+    const int64_t nbh = a.B * a.KVH;
+    const int64_t n_wave = tile * kTK + wave * 32;  // first key of this wavefront
+    float* s_wave = s_lds + wave * 32 * 8;
+
+    // phase-1 keys of this lane: n_wave + 16*gi + key16; their source row offset (shared by every
+    // (b, kvh) up to the segment base), visibility and rotation factors
+    int64_t koff1[2];
+    int seg1[2];
+    bool vis1[2];
+    float cs[2][2][8], sn[2][2][8];
+#pragma unroll
+    for (int gi = 0; gi < 2; gi++) {
+        const int64_t n = n_wave + 16 * gi + key16;
+        const int64_t NS = a.num_sink, S = a.S;
+        int64_t pos = 0;
+        seg1[gi] = 0;
+        koff1[gi] = 0;
+        vis1[gi] = false;
+        if (n < NS) {
+            seg1[gi] = 0; koff1[gi] = n * a.sink_stride[2]; vis1[gi] = a.sink_mask[n] == 0;
+            if (p.shared_pos) pos = a.sink_pos[n];
+        } else if (n < NS + S) {
+            seg1[gi] = 1; koff1[gi] = (n - NS) * a.cache_stride[2]; vis1[gi] = a.mask[n - NS] == 0;
+            if (p.shared_pos) pos = a.pos[n - NS] + a.pos_shift;
+        } else if (n < p.N) {
+            seg1[gi] = 2; koff1[gi] = 0; vis1[gi] = true;
+            pos = a.q_pos[0];
+        }
+        if (p.shared_pos) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int f = 32 * ks + 8 * kq + e;
+                    const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
+                    sincosf(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
+                }
+        }
+    }
+    // phase-2 keys of this lane: n_wave + 4*s + kg
+    int64_t koff2[kSteps];
+    int seg2[kSteps];
+    bool vis2[kSteps];
+#pragma unroll
+    for (int s = 0; s < kSteps; s++) {
+        const int64_t n = n_wave + 4 * s + kg;
+        const int64_t NS = a.num_sink, S = a.S;
+        seg2[s] = 0; koff2[s] = 0; vis2[s] = false;
+        if (n < NS) { seg2[s] = 0; koff2[s] = n * a.sink_stride[2]; vis2[s] = a.sink_mask[n] == 0; }
+        else if (n < NS + S) { seg2[s] = 1; koff2[s] = (n - NS) * a.cache_stride[2]; vis2[s] = a.mask[n - NS] == 0; }
+        else if (n < p.N) { seg2[s] = 2; koff2[s] = 0; vis2[s] = true; }
+    }
+
+    for (int64_t bh = blockIdx.y; bh < nbh; bh += gridDim.y) {
+        const int64_t b = bh / a.KVH, kvh = bh % a.KVH;
+        const T* kseg[3] = {(const T*)a.sink_k + b * a.sink_stride[0] + kvh * a.sink_stride[1],
+                            (const T*)a.cache_k + b * a.cache_stride[0] + kvh * a.cache_stride[1],
+                            (const T*)a.k_new + b * a.kv_new_stride[0] + kvh * a.kv_new_stride[1]};
+        const T* vseg[3] = {(const T*)a.sink_v + b * a.sink_stride[0] + kvh * a.sink_stride[1],
+                            (const T*)a.cache_v + b * a.cache_stride[0] + kvh * a.cache_stride[1],
+                            (const T*)a.v_new + b * a.kv_new_stride[0] + kvh * a.kv_new_stride[1]};
+        // ---- issue every row read of this (b, kvh) up front
+        uint4 kraw[2][4];
+#pragma unroll
+        for (int gi = 0; gi < 2; gi++) {
+            const T* kp = kseg[seg1[gi]] + koff1[gi];
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++)
+                kraw[gi][ks] = vis1[gi] ? *reinterpret_cast<const uint4*>(kp + 32 * ks + 8 * kq) : make_uint4(0, 0, 0, 0);
+        }
+        Raw vraw[kSteps][2];
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) {
+            if (vis2[s]) {
+                const T* vp = vseg[seg2[s]] + koff2[s];
+                vraw[s][0] = *reinterpret_cast<const Raw*>(vp + 4 * j);
+                vraw[s][1] = *reinterpret_cast<const Raw*>(vp + 64 + 4 * j);
+            }
+        }
+        // A operand: rotated queries of the group's heads (rows >= G are zero)
+        uint4 qop[4];
+        {
+            const T* qr = (const T*)p.qrot_t + ((b * a.H) + kvh * G + key16) * kD;
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++)
+                qop[ks] = key16 < G ? *reinterpret_cast<const uint4*>(qr + 32 * ks + 8 * kq) : make_uint4(0, 0, 0, 0);
+        }
+        // ---- phase 1: rotate K in registers, logits by MFMA, share them through LDS
+#pragma unroll
+        for (int gi = 0; gi < 2; gi++) {
+            if (!p.shared_pos && vis1[gi]) {
+                const int64_t n = n_wave + 16 * gi + key16;
+                int64_t pos;
+                if (seg1[gi] == 0) pos = a.sink_pos[b * a.sink_pos_stride[0] + kvh * a.sink_pos_stride[1] + n];
+                else if (seg1[gi] == 1)
+                    pos = a.pos[b * a.pos_stride[0] + kvh * a.pos_stride[1] + (n - a.num_sink)] + a.pos_shift;
+                else pos = a.q_pos[0];
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const int f = 32 * ks + 8 * kq + e;
+                        const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
+                        sincosf(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
+                    }
+            }
+            uint4 kop[4];
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&kraw[gi][ks]);
+                const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&kraw[gi][ks + 2]);
+                uint32_t o1[4], o2[4];
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const float a0 = Mma16<T>::lo(w1[w]), a1 = Mma16<T>::hi(w1[w]);
+                    const float b0 = Mma16<T>::lo(w2[w]), b1 = Mma16<T>::hi(w2[w]);
+                    const float c0 = cs[gi][ks][2 * w], s0 = sn[gi][ks][2 * w];
+                    const float c1 = cs[gi][ks][2 * w + 1], s1 = sn[gi][ks][2 * w + 1];
+                    o1[w] = Mma16<T>::pack2(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+                    o2[w] = Mma16<T>::pack2(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+                }
+                kop[ks] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+                kop[ks + 2] = make_uint4(o2[0], o2[1], o2[2], o2[3]);
+            }
+            f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) sacc = Mma16<T>::mma(qop[ks], kop[ks], sacc);
+            // lane holds heads 4*kq + v of key (16*gi + key16)
+            const int64_t n = n_wave + 16 * gi + key16;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int g = 4 * kq + v;
+                if (g < G) {
+                    const float sv = vis1[gi] ? sacc[v] * p.scale_log2 : -INFINITY;
+                    s_wave[(16 * gi + key16) * 8 + g] = sv;
+                    if (n < p.N) p.logits[((b * a.KVH + kvh) * p.N + n) * G + g] = sv;
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront's LDS writes are done
+        __builtin_amdgcn_wave_barrier();
+        // ---- phase 2: softmax partial of each 16-lane group and its weighted V sum
+        float sreg[kSteps][G];
+#pragma unroll
+        for (int s = 0; s < kSteps; s++)
+#pragma unroll
+            for (int g = 0; g < G; g++) sreg[s][g] = s_wave[(4 * s + kg) * 8 + g];
+        float mg[G], lgp[G], o[G][8];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float m = sreg[0][g];
+#pragma unroll
+            for (int s = 1; s < kSteps; s++) m = fmaxf(m, sreg[s][g]);
+            mg[g] = m;
+            lgp[g] = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[g][e] = 0.f;
+        }
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) {
+            if (!vis2[s]) continue;
             float va[4], vb[4];
             Piece<T>::unpack(vraw[s][0], va);
             Piece<T>::unpack(vraw[s][1], vb);
@@ -387,13 +661,22 @@ int run_decode(const DecodeParams& p, hipStream_t stream) {
         int64_t groups = p.shared_pos ? (2048 + p.tiles - 1) / p.tiles : nbh;
         if (groups < 1) groups = 1;
         if (groups > nbh) groups = nbh;
-        const int lds = (16 * G * kD + 32 * G) * (int)sizeof(float);
-        if (lds > 48 * 1024) {
-            CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_main_kernel<T, G>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        const int lds = (16 * G * kD + 32 * G + 4 * 32 * 8) * (int)sizeof(float);
+        if constexpr (std::is_same<T, float>::value) {
+            if (lds > 48 * 1024) {
+                CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_main_kernel<T, G>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            }
+            hipLaunchKernelGGL((decode_main_kernel<T, G>), dim3((unsigned)p.tiles, (unsigned)groups), dim3(256), lds,
+                               stream, p);
+        } else {
+            if (lds > 48 * 1024) {
+                CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_main_mfma_kernel<T, G>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            }
+            hipLaunchKernelGGL((decode_main_mfma_kernel<T, G>), dim3((unsigned)p.tiles, (unsigned)groups), dim3(256), lds,
+                               stream, p);
         }
-        hipLaunchKernelGGL((decode_main_kernel<T, G>), dim3((unsigned)p.tiles, (unsigned)groups), dim3(256), lds, stream,
-                           p);
         CKV_HIP_TRY(hipGetLastError());
     }
     {
@@ -434,8 +717,8 @@ bool decode_supported(const ckv_attn_args& a) {
     const int64_t G = a.H / a.KVH;
     if (!(G == 1 || G == 2 || G == 4 || G == 7 || G == 8)) return false;
     if ((a.homogeneous_heads ? a.H : G) > 128) return false;
-    const int64_t es = elem_bytes(a.dtype), vec = 4 * es;
-    // rows are read as 4-element vectors
+    const int64_t es = elem_bytes(a.dtype), vec = 16;
+    // rows are read as 16-byte (K of 16-bit caches, all of float32) or 8-byte vectors
     if (a.cache_stride[3] != 1 || a.kv_new_stride[3] != 1 || (a.num_sink > 0 && a.sink_stride[3] != 1)) return false;
     if (!aligned(a.cache_k, vec) || !aligned(a.cache_v, vec) || !aligned(a.k_new, vec) || !aligned(a.v_new, vec)) return false;
     if (a.num_sink > 0 && (!aligned(a.sink_k, vec) || !aligned(a.sink_v, vec))) return false;
@@ -448,7 +731,7 @@ bool decode_supported(const ckv_attn_args& a) {
 
 int64_t decode_workspace_bytes(int64_t B, int64_t H, int64_t KVH, int64_t num_sink, int64_t S) {
     const int64_t N = num_sink + S + 1, tiles = (N + kTK - 1) / kTK, G = H / KVH;
-    return align_up(B * H * kD * 4, 256) + align_up(B * KVH * N * G * 4, 256) + align_up(B * H * tiles * 2 * 4, 256) +
+    return 2 * align_up(B * H * kD * 4, 256) + align_up(B * KVH * N * G * 4, 256) + align_up(B * H * tiles * 2 * 4, 256) +
            align_up(B * H * tiles * kD * 4, 256) + align_up(B * H * 4, 256);
 }
 
@@ -460,6 +743,7 @@ int launch_decode(const ckv_attn_args& a, hipStream_t stream) {
     const int64_t G = a.H / a.KVH;
     char* w = reinterpret_cast<char*>(a.workspace);
     p.qrot = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * kD * 4, 256);
+    p.qrot_t = w; w += align_up(a.B * a.H * kD * 4, 256);
     p.logits = reinterpret_cast<float*>(w); w += align_up(a.B * a.KVH * p.N * G * 4, 256);
     p.part_ml = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * p.tiles * 2 * 4, 256);
     p.part_o = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * p.tiles * kD * 4, 256);
