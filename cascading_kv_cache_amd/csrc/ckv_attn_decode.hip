@@ -561,22 +561,37 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
     }
 }
 
+// one workgroup per (b, h): 4 quarters of 128 threads walk every 4th tile, then merge through LDS
 template <typename T>
-__global__ void __launch_bounds__(128) decode_tail_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
+    __shared__ float sh_m[512], sh_l[4], sh_o[4][kD];
     const ckv_attn_args& a = p.a;
     const int64_t row = blockIdx.x;  // b * H + h
-    const int d = threadIdx.x;
+    const int tid = threadIdx.x, d = tid & 127, qtr = tid >> 7;
     const float* ml = p.part_ml + row * p.tiles * 2;
     float M = -INFINITY;
-    for (int t = 0; t < p.tiles; t++) M = fmaxf(M, ml[2 * t]);
+    for (int t = tid; t < p.tiles; t += 512) M = fmaxf(M, ml[2 * t]);
+    sh_m[tid] = M;
+    __syncthreads();
+    for (int off = 256; off > 0; off >>= 1) {
+        if (tid < off) sh_m[tid] = fmaxf(sh_m[tid], sh_m[tid + off]);
+        __syncthreads();
+    }
+    M = sh_m[0];
     float L = 0.f, o = 0.f;
-    for (int t = 0; t < p.tiles; t++) {
+    for (int t = qtr; t < p.tiles; t += 4) {
         const float m = ml[2 * t];
         if (m == -INFINITY) continue;
         const float sc = __builtin_amdgcn_exp2f(m - M);
         L = fmaf(ml[2 * t + 1], sc, L);
         o = fmaf(p.part_o[(row * p.tiles + t) * kD + d], sc, o);
     }
+    sh_o[qtr][d] = o;
+    if (d == 0) sh_l[qtr] = L;
+    __syncthreads();
+    if (qtr != 0) return;
+    o = sh_o[0][d] + sh_o[1][d] + sh_o[2][d] + sh_o[3][d];
+    L = sh_l[0] + sh_l[1] + sh_l[2] + sh_l[3];
     const int64_t b = row / a.H, h = row % a.H;
     T* out = (T*)a.out + b * a.out_stride[0] + h * a.out_stride[1];
     out[d * a.out_stride[3]] = Elem<T>::from_float(o / L);
@@ -681,7 +696,7 @@ int run_decode(const DecodeParams& p, hipStream_t stream) {
     }
     {
         StageScope sc(CKV_STAGE_DECODE_TAIL, stream);
-        hipLaunchKernelGGL(decode_tail_kernel<T>, dim3((unsigned)(a.B * a.H)), dim3(128), 0, stream, p);
+        hipLaunchKernelGGL(decode_tail_kernel<T>, dim3((unsigned)(a.B * a.H)), dim3(512), 0, stream, p);
         CKV_HIP_TRY(hipGetLastError());
         if (a.cache_s || a.new_scores) {
             // w_ema[0] == w_new[0] == (1 - beta) for a single query row; the new token's weight is

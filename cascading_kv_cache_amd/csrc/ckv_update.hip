@@ -517,7 +517,8 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
         p.token_offset = off;
         p.k_sub = ksub;
         p.do_pos = (off + ksub == A.K) ? 1 : 0;
-        const int T = ksub <= 64 ? 64 : (ksub <= 256 ? 256 : 1024);
+        // small calls still rewrite max_seq_len position ids per (n, h): keep enough lanes for that
+        const int T = ksub <= 256 ? 256 : 1024;
         const size_t lds = plan_lds_bytes(ksub);
         if (lds > 48 * 1024) {
             CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(ckv_update_plan_kernel),
