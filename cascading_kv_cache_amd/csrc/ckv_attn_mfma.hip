@@ -586,6 +586,7 @@ struct ColsumParams {
     int G;
     int new_mode;
     float scale_log2;
+    int nkb, first_chunk_blk, nbkv, xcd_aware;  // block order, see the kernel
 };
 
 constexpr int kQT2 = 64;                      // query rows per LDS tile of the column pass
@@ -603,10 +604,35 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, half = lane >> 5;
-    const int64_t bkv = blockIdx.y;
+    // Block order.  Key blocks that hold chunk keys cost the most per step (masking on the
+    // diagonal, per-element weights), so they are handed out first and never form the tail of
+    // the launch.  Workgroup ids go round the 8 XCDs; when the kv heads divide evenly, every
+    // block of one kv head runs on one XCD so that head's query stream stays in that XCD's L2.
+    int bkv_i, kb_i;
+    {
+        const int nkb = p.nkb, cb0 = p.first_chunk_blk, heavy = nkb - cb0;
+        int id = blockIdx.x, nb = p.nbkv, first = 0, stride = 1;
+        if (p.xcd_aware) {
+            first = id & 7;
+            stride = 8;
+            id >>= 3;
+            nb >>= 3;
+        }
+        int i;
+        if (id < nb * heavy) {
+            i = id / heavy;
+            kb_i = cb0 + id % heavy;
+        } else {
+            id -= nb * heavy;
+            i = id / cb0;
+            kb_i = id % cb0;
+        }
+        bkv_i = first + stride * i;
+    }
+    const int64_t bkv = bkv_i;
     const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
     const int Q = (int)p.Q;
-    const int64_t key_blk = (int64_t)blockIdx.x * 256;   // first key of the workgroup
+    const int64_t key_blk = (int64_t)kb_i * 256;          // first key of the workgroup
     const int64_t key_w = key_blk + wave * 64;            // first key of this wavefront
 
     uint4 kreg[2][8];
@@ -631,6 +657,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     const bool chunk_keys = key_blk + 255 >= p.Nc;  // some key of the workgroup belongs to the chunk
     const int last_nrel = (int)(key_blk + 255 - p.Nc);
     const bool new_chunk = chunk_keys && p.new_mode;
+    const bool pure_chunk = key_blk >= p.Nc;        // no cached key in the workgroup
     if (new_chunk) {
         for (int i = tid; i < Q; i += 256) wnew_lds[i] = p.w_new[i];
     }
@@ -650,8 +677,9 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
 #pragma unroll
     for (int kk = 0; kk < 8; kk++) q_off[kk] = k_lds_off(col, 2 * kk + half);
     const int64_t head_row0 = (b * p.H + kvh * p.G) * p.Q;
-    auto issue = [&](int step, int stage) {
-        const int g = step / nmt, mt = m_first + (step % nmt) * kQT2;
+    // (head, query tile) of a step are tracked incrementally: integer division per step would
+    // cost more scalar instructions than the step's matrix work leaves room for
+    auto issue = [&](int g, int mt, int stage) {
         const int64_t row0 = head_row0 + (int64_t)g * p.Q + mt;
         const char* qt = (const char*)p.qr + row0 * (kD * (int64_t)sizeof(T));
         const uint32_t st = smem_addr + stage * kCsStage;
@@ -664,12 +692,11 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     };
 
     float acc[2] = {0.f, 0.f};
-    auto tile_step = [&](auto stage_tag, int step) {
+    auto tile_step = [&](auto stage_tag, int g, int mt) {
         constexpr int ST = decltype(stage_tag)::value;
         const unsigned char* q_lds = smem + ST * kCsStage;
         const float* lse_lds = reinterpret_cast<const float*>(q_lds + 16384);
         const float* w_lds = lse_lds + 64;
-        const int g = step / nmt, mt = m_first + (step % nmt) * kQT2;
 
         f32x16 sacc[2][2];  // [c = query subtile][ks]
 #pragma unroll
@@ -690,7 +717,41 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
         // element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4, key column of this lane
         const bool tail = mt + kQT2 > Q;                       // rows past the chunk end
         const bool diag = chunk_keys && mt <= last_nrel;       // tile may cross the diagonal
-        if (!tail && !diag && !new_chunk) {
+        if (!tail && !diag && new_chunk) {
+            // every row is later than every key of the block: no masks.  A chunk key takes the
+            // weight of its distance m - n and the eager path's roundings; a cached key (only in
+            // the block that straddles the chunk start) takes the row's EMA weight unrounded.
+            const float* wb[2];
+            bool chunk_lane[2];
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                chunk_lane[ks] = nrel[ks] >= 0;
+                wb[ks] = chunk_lane[ks] ? wnew_lds + (mt + 4 * half - nrel[ks]) : w_lds + 4 * half;
+            }
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+#pragma unroll
+                for (int v4 = 0; v4 < 4; v4++) {
+                    const int r0 = 32 * c + 8 * v4;
+                    const float4 l4 = *reinterpret_cast<const float4*>(lse_lds + r0 + 4 * half);
+                    const float ls[4] = {l4.x, l4.y, l4.z, l4.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+#pragma unroll
+                        for (int ks = 0; ks < 2; ks++) {
+                            const float pe = __builtin_amdgcn_exp2f(fmaf(sacc[c][ks][4 * v4 + e], p.scale_log2, -ls[e]));
+                            const float w = wb[ks][r0 + e];
+                            if (pure_chunk) {
+                                acc[ks] += Mma<T>::round1(Mma<T>::round1(pe) * w);
+                            } else {
+                                const float prod = (chunk_lane[ks] ? Mma<T>::round1(pe) : pe) * w;
+                                acc[ks] += chunk_lane[ks] ? Mma<T>::round1(prod) : prod;
+                            }
+                        }
+                    }
+                }
+            }
+        } else if (!tail && !diag && !new_chunk) {
 #pragma unroll
             for (int c = 0; c < 2; c++) {
 #pragma unroll
@@ -737,7 +798,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
                 }
             }
         }
-        if ((step % nmt) == nmt - 1) {  // head finished: combine the two lane halves and store
+        if (mt + kQT2 >= Q) {  // head finished: combine the two lane halves and store
             const int64_t h = kvh * p.G + g;
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
@@ -750,17 +811,31 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     };
 
     // two steps per trip: while stage s is consumed the copy of the next step fills stage s^1
-    if (n_steps > 0) issue(0, 0);
+    int g_cur = 0, mt_cur = m_first;          // step being consumed
+    auto advance = [&](int& g, int& mt) {
+        mt += kQT2;
+        if (mt >= Q) {
+            mt = m_first;
+            g++;
+        }
+    };
+    if (n_steps > 0) issue(0, m_first, 0);
     for (int step = 0; step < n_steps; step += 2) {
+        int g_n = g_cur, mt_n = mt_cur;
+        advance(g_n, mt_n);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
-        if (step + 1 < n_steps) issue(step + 1, 1);
-        tile_step(std::integral_constant<int, 0>{}, step);
+        if (step + 1 < n_steps) issue(g_n, mt_n, 1);
+        tile_step(std::integral_constant<int, 0>{}, g_cur, mt_cur);
         if (step + 1 < n_steps) {
+            int g_n2 = g_n, mt_n2 = mt_n;
+            advance(g_n2, mt_n2);
             __builtin_amdgcn_s_waitcnt(0x0F70);
             __syncthreads();
-            if (step + 2 < n_steps) issue(step + 2, 0);
-            tile_step(std::integral_constant<int, 1>{}, step + 1);
+            if (step + 2 < n_steps) issue(g_n2, mt_n2, 0);
+            tile_step(std::integral_constant<int, 1>{}, g_n, mt_n);
+            g_cur = g_n2;
+            mt_cur = mt_n2;
         }
     }
     if (n_steps == 0) {  // no query can see these keys (only possible for padding blocks)
@@ -847,7 +922,11 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         cp.G = G;
         cp.new_mode = mp.new_mode;
         cp.scale_log2 = scale_log2;
-        const dim3 grid((unsigned)((n + 255) / 256), (unsigned)(mp.B * mp.KVH));
+        cp.nkb = (int)((n + 255) / 256);
+        cp.first_chunk_blk = (int)(cp.Nc / 256);
+        cp.nbkv = (int)(mp.B * mp.KVH);
+        cp.xcd_aware = cp.nbkv % 8 == 0;
+        const dim3 grid((unsigned)(cp.nkb * cp.nbkv));
         const int lds = 2 * kCsStage + (int)mp.Q * 4;
         CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(colsum_mfma_kernel<T>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
