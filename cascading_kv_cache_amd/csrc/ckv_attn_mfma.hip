@@ -236,6 +236,8 @@ struct StageQParams {
     void* qr;                // (B*H, Q, D) contiguous
     int64_t rows;            // B*H*Q
     int64_t H, Q;
+    float qscale;            // softmax scale * log2(e), folded into the staged queries
+    int vec;                 // source rows can be read 16 bytes at a time
 };
 
 template <typename T>
@@ -247,11 +249,21 @@ __global__ void __launch_bounds__(256) stage_q_kernel(StageQParams p) {
     const int64_t m = row % p.Q, h = (row / p.Q) % p.H, b = row / (p.Q * p.H);
     const T* src = (const T*)p.q + b * p.stride[0] + h * p.stride[1] + m * p.stride[2];
     T lo[16], hi[16];
+    if (p.vec) {  // unit stride and 16-byte aligned rows
+        reinterpret_cast<uint4*>(lo)[0] = *reinterpret_cast<const uint4*>(src + 16 * quarter);
+        reinterpret_cast<uint4*>(lo)[1] = *reinterpret_cast<const uint4*>(src + 16 * quarter + 8);
+        reinterpret_cast<uint4*>(hi)[0] = *reinterpret_cast<const uint4*>(src + 64 + 16 * quarter);
+        reinterpret_cast<uint4*>(hi)[1] = *reinterpret_cast<const uint4*>(src + 64 + 16 * quarter + 8);
+    } else {
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-        lo[i] = src[(16 * quarter + i) * p.stride[3]];
-        hi[i] = src[(64 + 16 * quarter + i) * p.stride[3]];
+        for (int i = 0; i < 16; i++) {
+            lo[i] = src[(16 * quarter + i) * p.stride[3]];
+            hi[i] = src[(64 + 16 * quarter + i) * p.stride[3]];
+        }
     }
+    // the softmax scale (times log2 e) rides on the staged queries: one rounding to the tensor
+    // dtype after rotation and scaling, and the attention kernels exponentiate the products as
+    // they come out of the matrix pipe
     if (p.q_pos) {
         const int64_t pos = p.q_pos[m];
 #pragma unroll
@@ -261,8 +273,14 @@ __global__ void __launch_bounds__(256) stage_q_kernel(StageQParams p) {
             float sn, cs;
             sincosf(__fmul_rn((float)pos, f), &sn, &cs);
             const float x1 = Elem<T>::to_float(lo[i]), x2 = Elem<T>::to_float(hi[i]);
-            lo[i] = Elem<T>::from_float(x1 * cs - x2 * sn);
-            hi[i] = Elem<T>::from_float(x2 * cs + x1 * sn);
+            lo[i] = Elem<T>::from_float((x1 * cs - x2 * sn) * p.qscale);
+            hi[i] = Elem<T>::from_float((x2 * cs + x1 * sn) * p.qscale);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            lo[i] = Elem<T>::from_float(Elem<T>::to_float(lo[i]) * p.qscale);
+            hi[i] = Elem<T>::from_float(Elem<T>::to_float(hi[i]) * p.qscale);
         }
     }
     T* dst = (T*)p.qr + row * kD;
@@ -571,6 +589,352 @@ __global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
     }
 }
 
+// max over the two lane halves (lane l and lane l ^ 32) without a trip through LDS
+__device__ inline float half_max(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
+// Software-pipelined forward: eight wavefronts, 32 (head, position) rows each.  Iteration i runs
+// the softmax of tile i on the vector ALU while the matrix pipe adds the P.V product of tile i-1
+// and computes the logits of tile i+1; neither depends on the softmax in flight, so the two pipes
+// overlap inside one wavefront.  LDS: two K stages and three V^T stages.  Iteration i copies K
+// tile i+2 and V^T tile i+1, so everything an iteration reads was complete one barrier earlier
+// and its first operands can be fetched before the barrier.
+constexpr int kPipeStage = 16384;
+constexpr int kPipeLds = 5 * kPipeStage;   // K0 K1 V0 V1 V2
+constexpr int kPipeSrc = 4 * 512 * 4;      // copy source offsets, 4 per lane
+
+template <typename T>
+__global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int kThreads = 512, kBlocksPerWave = 2, kAhead = 3;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 31, half = lane >> 5;
+    const int64_t bkv = blockIdx.y;
+    const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
+    const int m0 = (int)blockIdx.x * p.QT;
+
+    int m_hi = m0 + p.QT - 1;
+    if (m_hi > (int)p.Q - 1) m_hi = (int)p.Q - 1;
+    const int n_tiles = (int)((p.Nc + m_hi) / kBN) + 1;
+    const int tiles_cap = (int)(p.n_pad / kBN);
+    unsigned long long* vis_lds = reinterpret_cast<unsigned long long*>(smem + kPipeLds + kPipeSrc);
+    uint32_t* src_lds = reinterpret_cast<uint32_t*>(smem + kPipeLds);   // per-lane source offsets of the copies
+    int* list_lds = reinterpret_cast<int*>(smem + kPipeLds + kPipeSrc + 8 * tiles_cap);
+    const uint32_t smem_addr = lds_address(smem);
+
+    // ---- work list: tiles with at least one visible key; bit 31 marks tiles that need masking
+    for (int i = tid; i < n_tiles; i += kThreads) vis_lds[i] = p.tile_vis[i];
+    __syncthreads();
+    if (wave == 0) {
+        int cnt = 0;
+        for (int base = 0; base < n_tiles; base += 64) {
+            const int t = base + lane;
+            const unsigned long long v = t < n_tiles ? vis_lds[t] : 0ull;
+            const unsigned long long bal = __ballot(v != 0ull);
+            if (v != 0ull) {
+                const bool partial = (v != ~0ull) || (t * kBN + kBN - 1 - (int)p.Nc > m0);
+                list_lds[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = t | (partial ? (int)0x80000000 : 0);
+            }
+            cnt += __popcll(bal);
+        }
+        if (lane == 0) list_lds[tiles_cap] = cnt;
+    }
+    __syncthreads();
+    const int n_work = __builtin_amdgcn_readfirstlane(list_lds[tiles_cap]);
+
+    // ---- the query row this lane owns as MFMA column `col`
+    int row_m;
+    uint4 qreg[8];
+    {
+        const int r = wave * 32 + col;
+        const int g = r / p.QT, mloc = r % p.QT;
+        row_m = m0 + mloc;
+        const int64_t row_h = kvh * p.G + g;
+        const bool row_ok = g < p.G && row_m < p.Q;
+        const T* qrow = (const T*)p.qr + ((b * p.H + row_h) * p.Q + row_m) * kD;
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++) {
+            qreg[kk] = row_ok ? *reinterpret_cast<const uint4*>(qrow + 16 * kk + 8 * half) : make_uint4(0, 0, 0, 0);
+        }
+    }
+    f32x16 oacc[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) oacc[dt][v] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;  // l_run: partial over this lane's keys; halves are added at the end
+
+    // ---- per-lane constants of the copies (source offsets) and of the operand reads (LDS offsets)
+    // (kept in LDS: a register spilled to scratch would make every reload wait for the copies in flight)
+#pragma unroll
+    for (int j = 0; j < kBlocksPerWave; j++) {
+        const int blk = wave * kBlocksPerWave + j;
+        const int pos = blk * 64 + lane;                     // piece position inside the LDS tile
+        const int kr_ = pos >> 4, kc = (pos & 15) ^ (kr_ & 15);
+        src_lds[(2 + j) * kThreads + tid] = kr_ * 256 + kc * 16;
+        const int vd = pos >> 3, vc = (pos & 7) ^ ((vd >> 1) & 7);
+        src_lds[j * kThreads + tid] = vd * 128 + vc * 16;
+    }
+    int k_off[8], v_off[4];  // key row `col` (+32 rows = +8192 B), dim row `col` (+32 rows = +4096 B)
+#pragma unroll
+    for (int kk = 0; kk < 8; kk++) k_off[kk] = k_lds_off(col, 2 * kk + half);
+#pragma unroll
+    for (int s = 0; s < 4; s++) v_off[s] = v_lds_off(col, 2 * s + half);
+    const char* kbase = (const char*)uniform_ptr((const char*)p.kr + bkv * p.n_pad * kD * (int64_t)sizeof(T));
+    const char* vbase = (const char*)uniform_ptr((const char*)p.vt + bkv * p.n_pad * kD * (int64_t)sizeof(T));
+    constexpr int kTileBytes = kBN * kD * (int)sizeof(T);
+
+    // one 1 KiB block (j = 0, 1) of a tile into K stage `stage` (0, 1) / V^T stage `stage` (0..2)
+    auto copy_k = [&](int t, int stage, int j, uint32_t src) {
+        async_copy16(kbase + (int64_t)t * kTileBytes, src, smem_addr + stage * kPipeStage + (wave * kBlocksPerWave + j) * 1024);
+    };
+    auto copy_v = [&](int t, int stage, int j, uint32_t src) {
+        async_copy16(vbase + (int64_t)t * kTileBytes, src,
+                     smem_addr + (2 + stage) * kPipeStage + (wave * kBlocksPerWave + j) * 1024);
+    };
+    auto work = [&](int j) { return __builtin_amdgcn_readfirstlane(list_lds[j < n_work ? j : n_work - 1]); };
+
+    // logits of the K tile in stage ST: s[ks][v] = key 32ks + 8(v/4) + 4half + v%4, query column col
+    auto qk = [&](auto stage_tag, f32x16(&s)[2]) {
+        constexpr int ST = decltype(stage_tag)::value;
+        const unsigned char* k_lds = smem + ST * kPipeStage;
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) s[ks][v] = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+                const uint4 a = *reinterpret_cast<const uint4*>(k_lds + k_off[kk] + ks * 8192);
+                s[ks] = Mma<T>::mma(a, qreg[kk], s[ks]);
+            }
+        }
+    };
+    uint32_t pk[4][4];  // P^T of one tile as the B operands of the four P.V contraction steps
+    // O^T += V^T P^T with the V^T tile in stage `stage` (0..2)
+    auto pv = [&](int stage) {
+        const unsigned char* v_lds = smem + (2 + stage) * kPipeStage;
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                const uint4 a = *reinterpret_cast<const uint4*>(v_lds + v_off[s] + dt * 4096);
+                const uint4 bq = make_uint4(pk[s][0], pk[s][1], pk[s][2], pk[s][3]);
+                oacc[dt] = Mma<T>::mma(a, bq, oacc[dt]);
+            }
+        }
+    };
+    auto mask_tile = [&](int entry, f32x16(&s)[2]) {
+        const int t = entry & 0x7fffffff;
+        const unsigned long long vis = vis_lds[t];
+        const int key0 = t * kBN;
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int kidx = 32 * ks + 8 * (v >> 2) + 4 * half + (v & 3);
+                const int nrel = key0 - (int)p.Nc + kidx;  // >= 0: key of the chunk
+                const bool ok = ((vis >> kidx) & 1ull) && (nrel < 0 || nrel <= row_m);
+                s[ks][v] = ok ? s[ks][v] : -INFINITY;
+            }
+    };
+    float alpha = 1.f;  // rescale of the accumulator owed since the last softmax
+    // the running maximum settles after a few tiles: rescale only when some row of the wavefront moved
+    auto rescale = [&]() {
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0ull) {
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) oacc[dt][v] *= alpha;
+        }
+    };
+
+    // Iteration i, written in issue order: 32 slots, each one matrix instruction (slots 0..15: P.V of
+    // tile i-1 out of V^T stage v_rd, slots 16..31: logits of tile i+1 out of K stage ST), the LDS
+    // read of the operand kAhead slots ahead, and a slice of the softmax of tile i.  Scheduling
+    // barriers keep the slots as written, so matrix and vector instructions alternate inside the
+    // wavefront.  The probabilities of tile i overwrite those of tile i-1 piece by piece, each after
+    // its last use by the P.V product.  The copies (V^T tile t_v into stage v_wr, K tile t_k into
+    // the other K stage) go out one at a time, a quarter of the slots apart.
+    // pre[]: on entry the operands of slots 0..kAhead-1, read before the barrier; on exit those
+    // of the next iteration.
+    auto iteration = [&](auto stage_tag, auto with_pv, int entry, int t_v, int t_k, int v_rd, int v_wr, f32x16(&s_cur)[2],
+                         f32x16(&s_nxt)[2], uint4(&pre)[kAhead]) {
+        constexpr int ST = decltype(stage_tag)::value;
+        constexpr bool kPV = decltype(with_pv)::value;
+        constexpr int kSlots = kPV ? 32 : 16, kQk0 = kPV ? 16 : 0;
+        constexpr int kCopyStep = kSlots / 4;
+        const unsigned char* k_lds = smem + ST * kPipeStage;
+        int v_addr[4];
+#pragma unroll
+        for (int s = 0; s < 4; s++) v_addr[s] = v_off[s] + (2 + v_rd) * kPipeStage;
+        if (entry < 0) mask_tile(entry, s_cur);
+        rescale();  // tile i-2 is in the accumulator; tile i-1, scaled for the newer maximum, is added below
+        auto operand = [&](int k) -> uint4 {
+            if (k >= kQk0) {
+                const int j = k - kQk0;  // K piece (kk, ks) = (j / 2, j % 2)
+                return *reinterpret_cast<const uint4*>(k_lds + k_off[j >> 1] + (j & 1) * 8192);
+            }
+            return *reinterpret_cast<const uint4*>(smem + v_addr[k >> 2] + (k & 3) * 4096);  // V^T piece (s, dt)
+        };
+        uint4 ops[kSlots];
+#pragma unroll
+        for (int k = 0; k < kAhead; k++) ops[k] = kPV ? pre[k] : operand(k);
+        float mx[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+        float m_use = 0.f, rs0 = 0.f, rs1 = 0.f;
+        constexpr int kMaxSlots = kPV ? 8 : 4;             // slots with running maxima
+        constexpr int kMaxPer = 32 / kMaxSlots;            // logits per such slot
+        constexpr int kExpFirst = kMaxSlots + 1;           // first slot with probabilities
+        constexpr int kExpPer = kPV ? 1 : 2;               // pairs per slot
+        float q0[kExpPer], q1[kExpPer];                    // exponentials of the previous slot, packed one slot later
+        // the source offset of a copy is read from LDS two slots before the copy, so that waiting
+        // for it does not also wait for the operand reads issued since
+        uint32_t src = src_lds[tid];
+#pragma unroll
+        for (int k = 0; k < kSlots; k++) {
+            if (k + kAhead < kSlots) ops[k + kAhead] = operand(k + kAhead);
+            if (k % kCopyStep == 1) {
+                const int q = k / kCopyStep;               // 0, 1: V^T blocks; 2, 3: K blocks
+                if (q < 2) copy_v(t_v, v_wr, q, src);
+                else copy_k(t_k, 1 - ST, q - 2, src);
+            }
+            if (k % kCopyStep == kCopyStep - 1 && k + 2 < kSlots) src = src_lds[((k + 2) / kCopyStep) * kThreads + tid];
+            if (k >= kQk0) {
+                const int j = k - kQk0;
+                const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                s_nxt[j & 1] = Mma<T>::mma(ops[k], qreg[j >> 1], j < 2 ? zero : s_nxt[j & 1]);
+            } else {
+                const int st = k >> 2, dt = k & 3;
+                const uint4 bq = make_uint4(pk[st][0], pk[st][1], pk[st][2], pk[st][3]);
+                oacc[dt] = Mma<T>::mma(ops[k], bq, oacc[dt]);
+            }
+            if (k < kMaxSlots) {
+#pragma unroll
+                for (int e = 0; e < kMaxPer; e++) {
+                    const int idx = k * kMaxPer + e;
+                    mx[e & 3] = fmaxf(mx[e & 3], s_cur[idx >> 4][idx & 15]);
+                }
+            } else if (k == kMaxSlots) {
+                float m = fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3]));
+                m = half_max(m) * p.scale_log2;  // scale > 0 commutes with max
+                const float m_new = fmaxf(m_run, m);
+                m_use = m_new == -INFINITY ? 0.f : m_new;
+                alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+                m_run = m_new;
+            } else {
+#pragma unroll
+                for (int r = 0; r < kExpPer; r++) {
+                    const int prev = (k - 1 - kExpFirst) * kExpPer + r;  // pair computed one slot ago
+                    if (prev >= 0 && prev < 16) {
+                        const int ks = prev >> 3, v = 2 * (prev & 7);
+                        rs0 += q0[r];
+                        rs1 += q1[r];
+                        pk[2 * ks + (v >> 3)][(v & 7) >> 1] = Mma<T>::pack2(q0[r], q1[r]);
+                    }
+                    const int pair = (k - kExpFirst) * kExpPer + r;      // (ks, v) = (pair / 8, 2 * (pair % 8))
+                    if (pair < 16) {
+                        const int ks = pair >> 3, v = 2 * (pair & 7);
+                        q0[r] = __builtin_amdgcn_exp2f(fmaf(s_cur[ks][v], p.scale_log2, -m_use));
+                        q1[r] = __builtin_amdgcn_exp2f(fmaf(s_cur[ks][v + 1], p.scale_log2, -m_use));
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        l_run = l_run * alpha + (rs0 + rs1);
+        // first operands of the next iteration: V^T tile i, complete since the last barrier
+        {
+            const int v_next = v_rd == 2 ? 0 : v_rd + 1;
+#pragma unroll
+            for (int k = 0; k < kAhead; k++) {
+                pre[k] = *reinterpret_cast<const uint4*>(smem + v_off[k >> 2] + (2 + v_next) * kPipeStage + (k & 3) * 4096);
+            }
+        }
+        // keep the packed probabilities in this region (they are next read after the barrier)
+#pragma unroll
+        for (int st = 0; st < 4; st++) asm volatile("" ::"v"(pk[st][0]), "v"(pk[st][1]), "v"(pk[st][2]), "v"(pk[st][3]));
+    };
+
+    f32x16 sA[2], sB[2];
+    uint4 pre[kAhead];
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    if (n_work > 0) {
+#pragma unroll
+        for (int j = 0; j < kBlocksPerWave; j++) {
+            copy_k(work(0) & 0x7fffffff, 0, j, src_lds[(2 + j) * kThreads + tid]);
+            copy_k(work(1) & 0x7fffffff, 1, j, src_lds[(2 + j) * kThreads + tid]);
+            copy_v(work(0) & 0x7fffffff, 0, j, src_lds[j * kThreads + tid]);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        qk(S0{}, sA);
+        // iteration 0: nothing to multiply by V yet
+        int e = work(0), tv = work(1) & 0x7fffffff, tk = work(2) & 0x7fffffff;
+        __syncthreads();                     // every wavefront is done with K stage 0
+        iteration(S1{}, std::false_type{}, e, tv, tk, 2, 1, sA, sB, pre);
+        int v_rd = 0;                        // (i - 1) % 3
+        auto next3 = [](int x) { return x == 2 ? 0 : x + 1; };
+        for (int i = 1; i < n_work; i += 2) {
+            // odd iteration: K stage 0 is read, K stage 1 refilled
+            e = work(i);
+            tv = work(i + 1) & 0x7fffffff;
+            tk = work(i + 2) & 0x7fffffff;
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+            iteration(S0{}, std::true_type{}, e, tv, tk, v_rd, next3(next3(v_rd)), sB, sA, pre);
+            v_rd = next3(v_rd);
+            if (i + 1 < n_work) {
+                e = work(i + 1);
+                tv = work(i + 2) & 0x7fffffff;
+                tk = work(i + 3) & 0x7fffffff;
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+                __syncthreads();
+                iteration(S1{}, std::true_type{}, e, tv, tk, v_rd, next3(next3(v_rd)), sA, sB, pre);
+                v_rd = next3(v_rd);
+            }
+        }
+        // the P.V product of the last tile; the copies still in flight are repeats that nobody reads
+        rescale();
+        pv(v_rd);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+
+    // epilogue: lane owns d = 32dt + 8(v/4) + 4half + v%4 of its query row
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const int g_row = (wave * 32 + col) / p.QT;
+    const int64_t row_h = kvh * p.G + g_row;
+    if (g_row < p.G && row_m < p.Q) {
+        const float inv = 1.f / l_tot;
+        T* orow = (T*)p.out + b * p.out_stride[0] + row_h * p.out_stride[1] + row_m * p.out_stride[2];
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+#pragma unroll
+            for (int v4 = 0; v4 < 4; v4++) {
+                const int d = 32 * dt + 8 * v4 + 4 * half;
+                if (p.out_stride[3] == 1) {
+                    uint2 w;
+                    w.x = Mma<T>::pack2(oacc[dt][4 * v4] * inv, oacc[dt][4 * v4 + 1] * inv);
+                    w.y = Mma<T>::pack2(oacc[dt][4 * v4 + 2] * inv, oacc[dt][4 * v4 + 3] * inv);
+                    *reinterpret_cast<uint2*>(orow + d) = w;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) orow[(d + e) * p.out_stride[3]] = Elem<T>::from_float(oacc[dt][4 * v4 + e] * inv);
+                }
+            }
+        }
+        if (half == 0) {
+            const float l2 = m_run + __builtin_amdgcn_logf(l_tot);  // v_log_f32 is log2
+            p.lse[(b * p.H + row_h) * p.Q + row_m] = l2 * 0.6931471805599453f;
+            p.lse2[(b * p.H + row_h) * p.Q + row_m] = l2;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // score sums
 // ---------------------------------------------------------------------------------------------
@@ -851,6 +1215,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
 template <typename T>
 int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
     const int64_t n = mp.n, n_pad = mp.n_pad;
+    const float scale_log2 = mp.scale * 1.4426950408889634f;
     {
         StageScope sc(CKV_STAGE_PREP, stream);
         StageParams sp;
@@ -887,11 +1252,13 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         sq.qr = mp.qr;
         sq.rows = mp.B * mp.H * mp.Q;
         sq.H = mp.H; sq.Q = mp.Q;
+        sq.qscale = scale_log2;
+        sq.vec = mp.q_stride[3] == 1 && reinterpret_cast<uintptr_t>(mp.q) % 16 == 0 && mp.q_stride[0] % 8 == 0 &&
+                 mp.q_stride[1] % 8 == 0 && mp.q_stride[2] % 8 == 0;
         hipLaunchKernelGGL(stage_q_kernel<T>, dim3((unsigned)((sq.rows * 4 + 255) / 256)), dim3(256), 0, stream, sq);
         CKV_HIP_TRY(hipGetLastError());
     }
     const int G = (int)(mp.H / mp.KVH);
-    const float scale_log2 = mp.scale * 1.4426950408889634f;
     {
         StageScope sc(CKV_STAGE_FWD, stream);
         FwdParams fp;
@@ -905,12 +1272,20 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         constexpr int kNC = 1, kNW = 8;
         constexpr int kWgRows = 32 * kNC * kNW;
         fp.QT = kWgRows / G;
-        fp.scale_log2 = scale_log2;
+        fp.scale_log2 = 1.f;  // already on the staged queries
         const dim3 grid((unsigned)((mp.Q + fp.QT - 1) / fp.QT), (unsigned)(mp.B * mp.KVH));
         const int lds = 2 * kStageBytes + (int)(n_pad / kBN) * 12 + 16;
         CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fwd_mfma_kernel<T, kNC, kNW>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        hipLaunchKernelGGL((fwd_mfma_kernel<T, kNC, kNW>), grid, dim3(64 * kNW), lds, stream, fp);
+        static const bool old_fwd = getenv("CKV_FWD_OLD") != nullptr;
+        if (old_fwd) {
+            hipLaunchKernelGGL((fwd_mfma_kernel<T, kNC, kNW>), grid, dim3(64 * kNW), lds, stream, fp);
+        } else {
+            const int lds_pipe = kPipeLds + kPipeSrc + (int)(n_pad / kBN) * 12 + 16;
+            CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fwd_pipe_kernel<T>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_pipe));
+            hipLaunchKernelGGL(fwd_pipe_kernel<T>, grid, dim3(512), lds_pipe, stream, fp);
+        }
         CKV_HIP_TRY(hipGetLastError());
     }
     if (mp.colsum) {
@@ -921,7 +1296,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         cp.B = mp.B; cp.H = mp.H; cp.KVH = mp.KVH; cp.Q = mp.Q; cp.N = n; cp.Nc = n - mp.Q; cp.n_pad = n_pad;
         cp.G = G;
         cp.new_mode = mp.new_mode;
-        cp.scale_log2 = scale_log2;
+        cp.scale_log2 = 1.f;  // already on the staged queries
         cp.nkb = (int)((n + 255) / 256);
         cp.first_chunk_blk = (int)(cp.Nc / 256);
         cp.nbkv = (int)(mp.B * mp.KVH);
