@@ -91,7 +91,7 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
         rc = launch_weights(w.w_ema, w.w_new, a.Q, a.beta, a.dtype, stream);
         if (rc) return rc;
     }
-    const bool use_mfma = mfma_supported(a.dtype, a.D, a.H, a.KVH, a.Q) && a.Q > 1;
+    const bool use_mfma = mfma_supported(a.dtype, a.D, a.H, a.KVH, a.Q) && a.Q > 1 && mfma_fits(N);
     if (use_mfma) {
         MfmaProblem mp;
         mp.seg[0] = MfmaSegment{a.sink_k, a.sink_v, {a.sink_stride[0], a.sink_stride[1], a.sink_stride[2], a.sink_stride[3]},

@@ -100,6 +100,7 @@ struct MfmaProblem {
 
 bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH, int64_t Q);
 int64_t mfma_n_pad(int64_t n);
+bool mfma_fits(int64_t n);  // the per-tile bookkeeping of n keys fits in LDS
 int launch_mfma(const MfmaProblem& p, hipStream_t stream);
 
 // ---- single-token decode family (Q == 1, head_dim 128) ----

@@ -331,7 +331,6 @@ __device__ inline uint32_t lds_address(const void* p) {
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
 }
 
-constexpr int kStageBytes = 32768;   // one K tile (64 x 256 B) + one V^T tile (128 x 128 B)
 
 // LDS tiles are unpadded (the async copy writes 1 KiB per wavefront contiguously); bank conflicts
 // are avoided by XOR-swizzling the 16-byte piece index with the row:
@@ -339,255 +338,6 @@ constexpr int kStageBytes = 32768;   // one K tile (64 x 256 B) + one V^T tile (
 //   V^T tile piece c of dim row d   lives at d*128 + ((c ^ ((d >> 1) & 7)) << 4)
 __device__ inline int k_lds_off(int r, int c) { return r * 256 + ((c ^ (r & 15)) << 4); }
 __device__ inline int v_lds_off(int d, int c) { return d * 128 + ((c ^ ((d >> 1) & 7)) << 4); }
-
-// NC = 32-row query subtiles per wavefront, NW = wavefronts per workgroup; a workgroup covers
-// 32 * NC * NW (head, position) rows of one kv head.  LDS: two tile stages, then the visibility
-// words of the key tiles and the compacted list of tiles that hold at least one visible key.
-template <typename T, int NC, int NW>
-__global__ void __launch_bounds__(64 * NW) fwd_mfma_kernel(FwdParams p) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int kThreads = 64 * NW;
-    constexpr int kBlocksPerWave = 16 / NW;  // 1 KiB blocks of each 16 KiB tile copied by one wavefront
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int col = lane & 31, half = lane >> 5;
-    const int64_t bkv = blockIdx.y;
-    const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
-    const int m0 = (int)blockIdx.x * p.QT;
-
-    int m_hi = m0 + p.QT - 1;
-    if (m_hi > (int)p.Q - 1) m_hi = (int)p.Q - 1;
-    const int n_tiles = (int)((p.Nc + m_hi) / kBN) + 1;
-    const int tiles_cap = (int)(p.n_pad / kBN);
-    unsigned long long* vis_lds = reinterpret_cast<unsigned long long*>(smem + 2 * kStageBytes);
-    int* list_lds = reinterpret_cast<int*>(smem + 2 * kStageBytes + 8 * tiles_cap);
-    const uint32_t smem_addr = lds_address(smem);
-
-    // ---- work list: tiles with at least one visible key; bit 31 marks tiles that need masking
-    for (int i = tid; i < n_tiles; i += kThreads) vis_lds[i] = p.tile_vis[i];
-    __syncthreads();
-    if (wave == 0) {
-        int cnt = 0;
-        for (int base = 0; base < n_tiles; base += 64) {
-            const int t = base + lane;
-            const unsigned long long v = t < n_tiles ? vis_lds[t] : 0ull;
-            const unsigned long long bal = __ballot(v != 0ull);
-            if (v != 0ull) {
-                const bool partial = (v != ~0ull) || (t * kBN + kBN - 1 - (int)p.Nc > m0);
-                list_lds[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = t | (partial ? (int)0x80000000 : 0);
-            }
-            cnt += __popcll(bal);
-        }
-        if (lane == 0) list_lds[tiles_cap] = cnt;
-    }
-    __syncthreads();
-    const int n_work = __builtin_amdgcn_readfirstlane(list_lds[tiles_cap]);
-
-    // ---- the query rows (one per 32-row subtile) this lane owns as MFMA column `col`
-    int row_m[NC];
-    int64_t row_h[NC];
-    bool row_ok[NC];
-    uint4 qreg[NC][8];
-#pragma unroll
-    for (int c = 0; c < NC; c++) {
-        const int r = wave * (32 * NC) + c * 32 + col;
-        const int g = r / p.QT, mloc = r % p.QT;
-        row_m[c] = m0 + mloc;
-        row_h[c] = kvh * p.G + g;
-        row_ok[c] = g < p.G && row_m[c] < p.Q;
-        const T* qrow = (const T*)p.qr + ((b * p.H + row_h[c]) * p.Q + row_m[c]) * kD;
-#pragma unroll
-        for (int kk = 0; kk < 8; kk++) {
-            qreg[c][kk] = row_ok[c] ? *reinterpret_cast<const uint4*>(qrow + 16 * kk + 8 * half) : make_uint4(0, 0, 0, 0);
-        }
-    }
-
-    f32x16 oacc[4][NC];
-#pragma unroll
-    for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-        for (int c = 0; c < NC; c++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) oacc[dt][c][v] = 0.f;
-    float m_run[NC], l_run[NC];  // l_run: partial over this lane's keys; halves are added at the end
-#pragma unroll
-    for (int c = 0; c < NC; c++) {
-        m_run[c] = -INFINITY;
-        l_run[c] = 0.f;
-    }
-
-    // ---- per-lane constants of the copy (source offsets) and of the operand reads (LDS offsets)
-    uint32_t k_src[kBlocksPerWave], v_src[kBlocksPerWave];
-#pragma unroll
-    for (int j = 0; j < kBlocksPerWave; j++) {
-        const int blk = wave * kBlocksPerWave + j;
-        const int pos = blk * 64 + lane;                     // piece position inside the LDS tile
-        const int kr_ = pos >> 4, kc = (pos & 15) ^ (kr_ & 15);
-        k_src[j] = kr_ * 256 + kc * 16;
-        const int vd = pos >> 3, vc = (pos & 7) ^ ((vd >> 1) & 7);
-        v_src[j] = vd * 128 + vc * 16;
-    }
-    int k_off[8], v_off[4];  // key row `col` (+32 rows = +8192 B), dim row `col` (+32 rows = +4096 B)
-#pragma unroll
-    for (int kk = 0; kk < 8; kk++) k_off[kk] = k_lds_off(col, 2 * kk + half);
-#pragma unroll
-    for (int s = 0; s < 4; s++) v_off[s] = v_lds_off(col, 2 * s + half);
-    const char* kbase = (const char*)uniform_ptr((const char*)p.kr + bkv * p.n_pad * kD * (int64_t)sizeof(T));
-    const char* vbase = (const char*)uniform_ptr((const char*)p.vt + bkv * p.n_pad * kD * (int64_t)sizeof(T));
-
-    auto issue = [&](int t, int stage) {  // t, stage uniform
-        const char* kt = kbase + (int64_t)t * (kBN * kD * (int)sizeof(T));
-        const char* vtile = vbase + (int64_t)t * (kBN * kD * (int)sizeof(T));
-        const uint32_t st = smem_addr + stage * kStageBytes;
-#pragma unroll
-        for (int j = 0; j < kBlocksPerWave; j++) {
-            const int blk = wave * kBlocksPerWave + j;
-            async_copy16(kt, k_src[j], st + blk * 1024);
-            async_copy16(vtile, v_src[j], st + 16384 + blk * 1024);
-        }
-    };
-    auto work = [&](int j) { return __builtin_amdgcn_readfirstlane(list_lds[j]); };
-
-    // one key tile out of LDS stage ST (compile-time so that every LDS read is register + immediate)
-    auto tile_step = [&](auto stage_tag, int entry) {
-        constexpr int ST = decltype(stage_tag)::value;
-        const unsigned char* k_lds = smem + ST * kStageBytes;
-        const unsigned char* v_lds = k_lds + 16384;
-        const int t = entry & 0x7fffffff;
-
-        // S^T tile: sacc[ks][c][v] = logit of key 32ks + 8(v/4) + 4half + v%4 for query column col
-        f32x16 sacc[2][NC];
-#pragma unroll
-        for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-            for (int c = 0; c < NC; c++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) sacc[ks][c][v] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < 8; kk++) {
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
-                const uint4 a = *reinterpret_cast<const uint4*>(k_lds + k_off[kk] + ks * 8192);
-#pragma unroll
-                for (int c = 0; c < NC; c++) sacc[ks][c] = Mma<T>::mma(a, qreg[c][kk], sacc[ks][c]);
-            }
-        }
-
-        if (entry < 0) {  // hidden keys in the tile, or the tile reaches past the diagonal
-            const unsigned long long vis = vis_lds[t];
-            const int key0 = t * kBN;
-#pragma unroll
-            for (int c = 0; c < NC; c++)
-#pragma unroll
-                for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-                    for (int v = 0; v < 16; v++) {
-                        const int kidx = 32 * ks + 8 * (v >> 2) + 4 * half + (v & 3);
-                        const int nrel = key0 - (int)p.Nc + kidx;  // >= 0: key of the chunk
-                        const bool ok = ((vis >> kidx) & 1ull) && (nrel < 0 || nrel <= row_m[c]);
-                        sacc[ks][c][v] = ok ? sacc[ks][c][v] : -INFINITY;
-                    }
-        }
-        uint32_t pk[NC][4][4];  // P^T as MFMA B operands: [query subtile][step][4 x 2 elements]
-#pragma unroll
-        for (int c = 0; c < NC; c++) {
-            float mx = -INFINITY;
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) mx = fmaxf(mx, sacc[ks][c][v]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32)) * p.scale_log2;  // scale > 0 commutes with max
-            const float m_new = fmaxf(m_run[c], mx);
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m_run[c] - m_use);
-            m_run[c] = m_new;
-            float rs = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
-#pragma unroll
-                for (int v = 0; v < 16; v += 2) {
-                    const float p0 = __builtin_amdgcn_exp2f(fmaf(sacc[ks][c][v], p.scale_log2, -m_use));
-                    const float p1 = __builtin_amdgcn_exp2f(fmaf(sacc[ks][c][v + 1], p.scale_log2, -m_use));
-                    rs += p0 + p1;
-                    // step = 2ks + v/8, element = v%8
-                    pk[c][2 * ks + (v >> 3)][(v & 7) >> 1] = Mma<T>::pack2(p0, p1);
-                }
-            }
-            l_run[c] = l_run[c] * alpha + rs;
-            // the running maximum settles after a few tiles: skip the accumulator rescale
-            // whenever no row of the wavefront moved (alpha == 1 everywhere)
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0ull) {
-#pragma unroll
-                for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-                    for (int v = 0; v < 16; v++) oacc[dt][c][v] *= alpha;
-            }
-        }
-
-        // O^T += V^T P^T
-#pragma unroll
-        for (int s = 0; s < 4; s++) {
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
-                const uint4 a = *reinterpret_cast<const uint4*>(v_lds + v_off[s] + dt * 4096);
-#pragma unroll
-                for (int c = 0; c < NC; c++) {
-                    const uint4 bq = make_uint4(pk[c][s][0], pk[c][s][1], pk[c][s][2], pk[c][s][3]);
-                    oacc[dt][c] = Mma<T>::mma(a, bq, oacc[dt][c]);
-                }
-            }
-        }
-    };
-
-    // ---- main loop, two tiles per trip: while stage s is consumed the copy of the next tile
-    //      fills stage s^1
-    if (n_work > 0) issue(work(0) & 0x7fffffff, 0);
-    for (int j = 0; j < n_work; j += 2) {
-        const int e0 = work(j);
-        const int e1 = j + 1 < n_work ? work(j + 1) : 0;
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's pieces of tile j landed
-        __syncthreads();                     // ... everyone's did, and stage 1 is free again
-        if (j + 1 < n_work) issue(e1 & 0x7fffffff, 1);
-        tile_step(std::integral_constant<int, 0>{}, e0);
-        if (j + 1 < n_work) {
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-            __syncthreads();
-            if (j + 2 < n_work) issue(work(j + 2) & 0x7fffffff, 0);
-            tile_step(std::integral_constant<int, 1>{}, e1);
-        }
-    }
-
-    // epilogue: lane owns d = 32dt + 8(v/4) + 4half + v%4 of its query row
-#pragma unroll
-    for (int c = 0; c < NC; c++) {
-        const float l_tot = l_run[c] + __shfl_xor(l_run[c], 32);
-        if (!row_ok[c]) continue;
-        const float inv = 1.f / l_tot;
-        T* orow = (T*)p.out + b * p.out_stride[0] + row_h[c] * p.out_stride[1] + row_m[c] * p.out_stride[2];
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-#pragma unroll
-            for (int v4 = 0; v4 < 4; v4++) {
-                const int d = 32 * dt + 8 * v4 + 4 * half;
-                if (p.out_stride[3] == 1) {
-                    uint2 w;
-                    w.x = Mma<T>::pack2(oacc[dt][c][4 * v4] * inv, oacc[dt][c][4 * v4 + 1] * inv);
-                    w.y = Mma<T>::pack2(oacc[dt][c][4 * v4 + 2] * inv, oacc[dt][c][4 * v4 + 3] * inv);
-                    *reinterpret_cast<uint2*>(orow + d) = w;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        orow[(d + e) * p.out_stride[3]] = Elem<T>::from_float(oacc[dt][c][4 * v4 + e] * inv);
-                }
-            }
-        }
-        if (half == 0) {
-            const float l2 = m_run[c] + __builtin_amdgcn_logf(l_tot);  // v_log_f32 is log2
-            p.lse[(b * p.H + row_h[c]) * p.Q + row_m[c]] = l2 * 0.6931471805599453f;
-            p.lse2[(b * p.H + row_h[c]) * p.Q + row_m[c]] = l2;
-        }
-    }
-}
 
 // max over the two lane halves (lane l and lane l ^ 32) without a trip through LDS
 __device__ inline float half_max(float x) {
@@ -604,6 +354,9 @@ __device__ inline float half_max(float x) {
 constexpr int kPipeStage = 16384;
 constexpr int kPipeLds = 5 * kPipeStage;   // K0 K1 V0 V1 V2
 constexpr int kPipeSrc = 4 * 512 * 4;      // copy source offsets, 4 per lane
+// stages, copy offsets, one visibility word and one work-list entry per key tile, the list length
+inline int64_t pipe_lds_bytes(int64_t n_pad) { return kPipeLds + kPipeSrc + (n_pad / kBN) * 12 + 16; }
+constexpr int64_t kLdsLimit = 160 * 1024;
 
 template <typename T>
 __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
@@ -1269,23 +1022,13 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         fp.lse2 = mp.lse2;
         fp.B = mp.B; fp.H = mp.H; fp.KVH = mp.KVH; fp.Q = mp.Q; fp.N = n; fp.Nc = n - mp.Q; fp.n_pad = n_pad;
         fp.G = G;
-        constexpr int kNC = 1, kNW = 8;
-        constexpr int kWgRows = 32 * kNC * kNW;
-        fp.QT = kWgRows / G;
+        fp.QT = kRows / G;
         fp.scale_log2 = 1.f;  // already on the staged queries
         const dim3 grid((unsigned)((mp.Q + fp.QT - 1) / fp.QT), (unsigned)(mp.B * mp.KVH));
-        const int lds = 2 * kStageBytes + (int)(n_pad / kBN) * 12 + 16;
-        CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fwd_mfma_kernel<T, kNC, kNW>),
+        const int lds = pipe_lds_bytes(n_pad);
+        CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fwd_pipe_kernel<T>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        static const bool old_fwd = getenv("CKV_FWD_OLD") != nullptr;
-        if (old_fwd) {
-            hipLaunchKernelGGL((fwd_mfma_kernel<T, kNC, kNW>), grid, dim3(64 * kNW), lds, stream, fp);
-        } else {
-            const int lds_pipe = kPipeLds + kPipeSrc + (int)(n_pad / kBN) * 12 + 16;
-            CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fwd_pipe_kernel<T>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_pipe));
-            hipLaunchKernelGGL(fwd_pipe_kernel<T>, grid, dim3(512), lds_pipe, stream, fp);
-        }
+        hipLaunchKernelGGL(fwd_pipe_kernel<T>, grid, dim3(512), lds, stream, fp);
         CKV_HIP_TRY(hipGetLastError());
     }
     if (mp.colsum) {
@@ -1322,6 +1065,10 @@ bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH, int64_t Q) {
 }
 
 int64_t mfma_n_pad(int64_t n) { return align_up(n, 256); }
+
+// the forward kernel keeps per-tile bookkeeping of all N keys in LDS
+bool mfma_fits(int64_t n) { return pipe_lds_bytes(mfma_n_pad(n)) <= kLdsLimit; }
+
 
 int launch_mfma(const MfmaProblem& mp, hipStream_t stream) {
     if (mp.dtype == CKV_BF16) return run_mfma<__hip_bfloat16>(mp, stream);
