@@ -561,6 +561,313 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Streaming variant of the main kernel (16-bit caches, shared positions, G <= 4).
+//
+// The (key tile, batch x kv-head) items are dealt out in equal contiguous runs, one workgroup per
+// CU, so the launch has no tail.  K and V rows reach LDS by asynchronous copies, double buffered:
+// while item i is computed the rows of item i+1 are in flight and occupy no registers.  Each of the
+// eight wavefronts copies exactly the 16 key rows it consumes, so the staging needs no workgroup
+// barrier, only the wavefront's own vmcnt wait.  That wait is vmcnt(0) at the top of an iteration;
+// to keep it from stalling on stores, the partial results of an item are written out one iteration
+// late, just before the next copies are issued, and the query operand of the next item is loaded
+// (and waited for) at the same point.
+// ---------------------------------------------------------------------------------------------
+constexpr int kSK = 128;                       // keys per tile
+constexpr int kStreamStage = 2 * kSK * 256;    // K rows then V rows of one tile (16-bit, 256 B per row)
+
+__device__ inline uint32_t lds_address(const void* p) {
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
+}
+
+// 16 bytes per lane from a per-lane global address to LDS (wave base in M0, lane i at +16 i)
+__device__ inline void async_row_copy16(const void* src, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(src)
+                 : "memory");
+}
+
+// the same with a uniform base (SGPR pair) plus a 32-bit per-lane byte offset
+__device__ inline void async_copy16_s(const void* sbase, uint32_t voff, uint32_t lds_wave_base) {
+    const uint64_t v = reinterpret_cast<uint64_t>(sbase);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(voff),
+                   "s"(reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo))
+                 : "memory");
+}
+
+// sum / max over the four 16-lane rows of a wavefront (lanes l, l^16, l^32, l^48)
+__device__ inline float rows4_sum(float x) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    const auto q = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(q[0]) + __uint_as_float(q[1]);
+}
+__device__ inline float rows4_max(float x) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    const auto q = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
+}
+
+inline int stream_lds_bytes(int G) { return 2 * kStreamStage + (8 * G * kD + 8 * G * 2 + 8 * 16 * 8) * (int)sizeof(float); }
+
+template <typename T, int G>
+__global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* red_o = reinterpret_cast<float*>(smem + 2 * kStreamStage);  // [8 waves][G][128]
+    float* red_ml = red_o + 8 * G * kD;                                // [8][G][2]
+    float* s_lds = red_ml + 8 * G * 2;                                 // [8][16 keys][8] logits, then [16][4] probabilities
+    const uint32_t smem_addr = lds_address(smem);
+    const ckv_attn_args& a = p.a;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int key16 = lane & 15, kq = lane >> 4;  // phase 1: MFMA column (key) and k-quarter
+    const int pkey = lane >> 2, pg = lane & 3;    // softmax: one (key, head) per lane
+    float* s_wave = s_lds + wave * 16 * 8;
+    const int64_t nbh = a.B * a.KVH, total = (int64_t)p.tiles * nbh;
+    const int64_t item0 = total * blockIdx.x / gridDim.x, item1 = total * (blockIdx.x + 1) / gridDim.x;
+    const int64_t NS = a.num_sink, S = a.S;
+    const bool cache_small = S * a.cache_stride[2] * (int64_t)sizeof(T) < (1ll << 31);  // 32-bit byte offsets reach every row
+
+    // LDS read offsets inside a stage.  K row r keeps source piece c at slot c ^ (r & 15), which
+    // makes the 16-byte operand reads conflict free; V rows are linear (a row is read as one
+    // 256-byte line, 4 bytes per lane).
+    int kaddr[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) kaddr[ks] = (wave * 16 + key16) * 256 + (((4 * ks + kq) ^ key16) << 4);
+    const int vaddr = kSK * 256 + wave * 16 * 256 + lane * 4;
+
+    for (int64_t item = item0; item < item1;) {
+        const int64_t tile = item / nbh, bh0 = item % nbh;
+        const int64_t bh1 = (tile + 1) * nbh > item1 ? item1 - tile * nbh : nbh;
+        item = tile * nbh + bh1;
+        const int64_t n_wave = tile * kSK + wave * 16;  // first key of this wavefront
+
+        // ---- per-tile constants (the same for every (b, kvh): positions are shared)
+        bool vis1 = false;
+        float cs[2][8], sn[2][8];
+        {
+            const int64_t n = n_wave + key16;
+            int64_t pos = 0;
+            if (n < NS) { vis1 = a.sink_mask[n] == 0; pos = a.sink_pos[n]; }
+            else if (n < NS + S) { vis1 = a.mask[n - NS] == 0; pos = a.pos[n - NS] + a.pos_shift; }
+            else if (n < p.N) { vis1 = true; pos = a.q_pos[0]; }
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int f = 32 * ks + 8 * kq + e;
+                    const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
+                    sincosf(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
+                }
+        }
+        // bit k: key n_wave + k is visible (lanes 0..15 are the sixteen keys)
+        const uint32_t vis_keys = __builtin_amdgcn_readfirstlane((uint32_t)(__builtin_amdgcn_ballot_w64(vis1) & 0xffffull));
+        // copy rows of this lane: block jb holds rows 4 jb .. 4 jb + 3 of the wavefront's 16.
+        // Usual case: all 16 rows are cache slots and byte offsets fit 32 bits -> uniform base plus
+        // a per-lane offset, no address arithmetic per copy.
+        const bool one_seg = cache_small && n_wave >= NS && n_wave + 16 <= NS + S;
+        int seg_c[4];
+        int64_t koff_c[4], voff_c[4];  // element offsets inside the (b, kvh) slab, source piece included
+        uint32_t koff32[4], voff32[4]; // the same in bytes for the usual case
+#pragma unroll
+        for (int jb = 0; jb < 4; jb++) {
+            const int r = 4 * jb + (lane >> 4);
+            const int64_t n = n_wave + r;
+            int64_t row_off;
+            if (n < NS) { seg_c[jb] = 0; row_off = n * a.sink_stride[2]; }
+            else if (n < NS + S) { seg_c[jb] = 1; row_off = (n - NS) * a.cache_stride[2]; }
+            else { seg_c[jb] = 2; row_off = 0; }  // the new token; rows past the end repeat it and stay hidden
+            koff_c[jb] = row_off + (((lane & 15) ^ (r & 15)) << 3);
+            voff_c[jb] = row_off + ((lane & 15) << 3);
+            koff32[jb] = (uint32_t)(koff_c[jb] * (int64_t)sizeof(T));
+            voff32[jb] = (uint32_t)(voff_c[jb] * (int64_t)sizeof(T));
+        }
+
+        auto issue = [&](int64_t bh, int stage) {
+            const int64_t b = bh / a.KVH, kvh = bh % a.KVH;
+            const uint32_t st = smem_addr + stage * kStreamStage;
+            if (one_seg) {
+                const T* kb = (const T*)a.cache_k + b * a.cache_stride[0] + kvh * a.cache_stride[1];
+                const T* vb = (const T*)a.cache_v + b * a.cache_stride[0] + kvh * a.cache_stride[1];
+#pragma unroll
+                for (int jb = 0; jb < 4; jb++) {
+                    async_copy16_s(kb, koff32[jb], st + (wave * 4 + jb) * 1024);
+                    async_copy16_s(vb, voff32[jb], st + kSK * 256 + (wave * 4 + jb) * 1024);
+                }
+                return;
+            }
+            const T* kseg[3] = {(const T*)a.sink_k + b * a.sink_stride[0] + kvh * a.sink_stride[1],
+                                (const T*)a.cache_k + b * a.cache_stride[0] + kvh * a.cache_stride[1],
+                                (const T*)a.k_new + b * a.kv_new_stride[0] + kvh * a.kv_new_stride[1]};
+            const T* vseg[3] = {(const T*)a.sink_v + b * a.sink_stride[0] + kvh * a.sink_stride[1],
+                                (const T*)a.cache_v + b * a.cache_stride[0] + kvh * a.cache_stride[1],
+                                (const T*)a.v_new + b * a.kv_new_stride[0] + kvh * a.kv_new_stride[1]};
+#pragma unroll
+            for (int jb = 0; jb < 4; jb++) {
+                const T* kb = seg_c[jb] == 0 ? kseg[0] : (seg_c[jb] == 1 ? kseg[1] : kseg[2]);
+                const T* vb = seg_c[jb] == 0 ? vseg[0] : (seg_c[jb] == 1 ? vseg[1] : vseg[2]);
+                async_row_copy16(kb + koff_c[jb], st + (wave * 4 + jb) * 1024);
+                async_row_copy16(vb + voff_c[jb], st + kSK * 256 + (wave * 4 + jb) * 1024);
+            }
+        };
+        // A operand: rotated queries of the group's heads (rows >= G are zero)
+        auto load_q = [&](int64_t bh, uint4(&q)[4]) {
+            const int64_t b = bh / a.KVH, kvh = bh % a.KVH;
+            const T* qr = (const T*)p.qrot_t + ((b * a.H) + kvh * G + key16) * kD;
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++)
+                q[ks] = key16 < G ? *reinterpret_cast<const uint4*>(qr + 32 * ks + 8 * kq) : make_uint4(0, 0, 0, 0);
+        };
+
+        uint4 q_next[4];
+        load_q(bh0, q_next);
+        issue(bh0, 0);
+        bool pending = false;
+        int64_t pend_bh = 0;
+        float pend_o = 0.f, pend_m = 0.f, pend_l = 0.f;
+        auto flush = [&]() {
+            if (!pending) return;
+            const int64_t b = pend_bh / a.KVH, kvh = pend_bh % a.KVH;
+            if (tid < G * kD) {
+                const int g = tid >> 7, d = tid & 127;
+                const int64_t row = (b * a.H + kvh * G + g) * p.tiles + tile;
+                p.part_o[row * kD + d] = pend_o;
+                if (d == 0) {
+                    p.part_ml[row * 2] = pend_m;
+                    p.part_ml[row * 2 + 1] = pend_l;
+                }
+            }
+        };
+        int stage = 0;
+        for (int64_t bh = bh0; bh < bh1; bh++, stage ^= 1) {
+            const int64_t b = bh / a.KVH, kvh = bh % a.KVH;
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the rows of this item are in LDS
+            uint4 qop[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                qop[ks] = q_next[ks];
+                // use the operand here so that the wait for its load is placed here too, ahead of the next copies
+                asm volatile("" : "+v"(qop[ks].x), "+v"(qop[ks].y), "+v"(qop[ks].z), "+v"(qop[ks].w));
+            }
+            if (bh + 1 < bh1) load_q(bh + 1, q_next);
+            flush();
+            if (bh + 1 < bh1) issue(bh + 1, stage ^ 1);
+            const unsigned char* st = smem + stage * kStreamStage;
+
+            // ---- phase 1: rotate K in registers, logits by MFMA, share them through LDS
+            {
+                uint4 kraw[4];
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) kraw[ks] = *reinterpret_cast<const uint4*>(st + kaddr[ks]);
+                uint4 kop[4];
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&kraw[ks]);
+                    const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&kraw[ks + 2]);
+                    uint32_t o1[4], o2[4];
+#pragma unroll
+                    for (int w = 0; w < 4; w++) {
+                        const float a0 = Mma16<T>::lo(w1[w]), a1 = Mma16<T>::hi(w1[w]);
+                        const float b0 = Mma16<T>::lo(w2[w]), b1 = Mma16<T>::hi(w2[w]);
+                        const float c0 = cs[ks][2 * w], s0 = sn[ks][2 * w];
+                        const float c1 = cs[ks][2 * w + 1], s1 = sn[ks][2 * w + 1];
+                        o1[w] = Mma16<T>::pack2(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+                        o2[w] = Mma16<T>::pack2(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+                    }
+                    kop[ks] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+                    kop[ks + 2] = make_uint4(o2[0], o2[1], o2[2], o2[3]);
+                }
+                f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) sacc = Mma16<T>::mma(qop[ks], kop[ks], sacc);
+                // lane holds heads 4 kq + v of key key16
+                const int64_t n = n_wave + key16;
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int g = 4 * kq + v;
+                    if (g < G) {
+                        const float sv = vis1 ? sacc[v] * p.scale_log2 : -INFINITY;
+                        s_wave[key16 * 8 + g] = sv;
+                        if (n < p.N) p.logits[((b * a.KVH + kvh) * p.N + n) * G + g] = sv;
+                    }
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront's LDS writes are done
+            __builtin_amdgcn_wave_barrier();
+            // ---- phase 2a: softmax of the wavefront's 16 keys, one (key, head) per lane
+            {
+                const float sv = pg < G ? s_wave[pkey * 8 + pg] : -INFINITY;
+                // all-reduce over the 16 keys of a head: lanes pg, pg + 4, ... of every 16-lane row, then the rows
+                float m = sv;
+                m = fmaxf(m, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(m), 0x124, 0xF, 0xF, true)));  // row_ror:4
+                m = fmaxf(m, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(m), 0x128, 0xF, 0xF, true)));  // row_ror:8
+                m = rows4_max(m);
+                const float pe = __builtin_amdgcn_exp2f(sv - (m == -INFINITY ? 0.f : m));  // hidden keys and idle lanes: 0
+                float l = pe;
+                l += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(l), 0x124, 0xF, 0xF, true));
+                l += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(l), 0x128, 0xF, 0xF, true));
+                l = rows4_sum(l);
+                __builtin_amdgcn_wave_barrier();      // every lane has read its logit
+                s_wave[pkey * 4 + pg] = pe;           // probabilities, 4 per key
+                if (pkey == 0 && pg < G) {
+                    red_ml[(wave * G + pg) * 2] = m;
+                    red_ml[(wave * G + pg) * 2 + 1] = l;
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier();
+            // ---- phase 2b: weighted V sum; lane owns dims 2 lane, 2 lane + 1 of every row
+            float o[G][2];
+#pragma unroll
+            for (int g = 0; g < G; g++) o[g][0] = o[g][1] = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < 16; kk++) {
+                if (!((vis_keys >> kk) & 1u)) continue;  // hidden slots may hold anything
+                const float4 p4 = *reinterpret_cast<const float4*>(s_wave + kk * 4);
+                const uint32_t vv = *reinterpret_cast<const uint32_t*>(st + vaddr + kk * 256);
+                const float v0 = Mma16<T>::lo(vv), v1 = Mma16<T>::hi(vv);
+                const float pp[4] = {p4.x, p4.y, p4.z, p4.w};
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    o[g][0] = fmaf(pp[g], v0, o[g][0]);
+                    o[g][1] = fmaf(pp[g], v1, o[g][1]);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++)
+                *reinterpret_cast<float2*>(red_o + (wave * G + g) * kD + 2 * lane) = make_float2(o[g][0], o[g][1]);
+            __syncthreads();
+            // ---- combine the eight wavefronts; the result is stored at the top of the next iteration
+            if (tid < G * kD) {
+                const int g = tid >> 7, d = tid & 127;
+                float M = -INFINITY;
+#pragma unroll
+                for (int w = 0; w < 8; w++) M = fmaxf(M, red_ml[(w * G + g) * 2]);
+                float acc = 0.f, L = 0.f;
+#pragma unroll
+                for (int w = 0; w < 8; w++) {
+                    const float mw = red_ml[(w * G + g) * 2];
+                    const float sc = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M);
+                    acc = fmaf(red_o[(w * G + g) * kD + d], sc, acc);
+                    L = fmaf(red_ml[(w * G + g) * 2 + 1], sc, L);
+                }
+                pend_o = acc;
+                pend_m = M;
+                pend_l = L;
+            }
+            pending = true;
+            pend_bh = bh;
+            __syncthreads();  // red_* may be overwritten
+        }
+        flush();
+    }
+}
+
 // one workgroup per (b, h): 4 quarters of 128 threads walk every 4th tile, then merge through LDS
 template <typename T>
 __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
@@ -684,6 +991,19 @@ int run_decode(const DecodeParams& p, hipStream_t stream) {
             }
             hipLaunchKernelGGL((decode_main_kernel<T, G>), dim3((unsigned)p.tiles, (unsigned)groups), dim3(256), lds,
                                stream, p);
+        } else if (G <= 4 && p.shared_pos && !getenv("CKV_DECODE_OLD")) {
+            // streaming kernel: one workgroup per CU, items dealt out evenly
+            if constexpr (G <= 4) {
+                const int lds_s = stream_lds_bytes(G);
+                CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stream_kernel<T, G>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_s));
+                int dev = 0, cus = 0;
+                CKV_HIP_TRY(hipGetDevice(&dev));
+                CKV_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+                int64_t wgs = cus > 0 ? cus : 256;
+                if (wgs > p.tiles * nbh) wgs = p.tiles * nbh;
+                hipLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(512), lds_s, stream, p);
+            }
         } else {
             if (lds > 48 * 1024) {
                 CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_main_mfma_kernel<T, G>),
