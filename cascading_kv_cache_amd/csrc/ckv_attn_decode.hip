@@ -302,6 +302,8 @@ typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
 
 template <typename T>
 struct Mma16;
@@ -317,6 +319,11 @@ struct Mma16<__hip_bfloat16> {
         f32x2_t f = {a, b};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
     }
+    // 16x16x16: four 16-bit values per lane and operand
+    __device__ static f32x4 mma_k16(uint2 a, uint2 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a), __builtin_bit_cast(s16x4_t, b), c, 0,
+                                                         0, 0);
+    }
 };
 template <>
 struct Mma16<__half> {
@@ -329,6 +336,9 @@ struct Mma16<__half> {
     __device__ static uint32_t pack2(float a, float b) {
         f32x2_t f = {a, b};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2_t));
+    }
+    __device__ static f32x4 mma_k16(uint2 a, uint2 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a), __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
     }
 };
 
@@ -565,39 +575,15 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
 // Streaming variant of the main kernel (16-bit caches, shared positions, G <= 4).
 //
 // The (key tile, batch x kv-head) items are dealt out in equal contiguous runs, one workgroup per
-// CU, so the launch has no tail.  K and V rows reach LDS by asynchronous copies, double buffered:
-// while item i is computed the rows of item i+1 are in flight and occupy no registers.  Each of the
-// eight wavefronts copies exactly the 16 key rows it consumes, so the staging needs no workgroup
-// barrier, only the wavefront's own vmcnt wait.  That wait is vmcnt(0) at the top of an iteration;
-// to keep it from stalling on stores, the partial results of an item are written out one iteration
-// late, just before the next copies are issued, and the query operand of the next item is loaded
-// (and waited for) at the same point.
+// CU, so the launch has no tail.  K and V rows are read with fully coalesced 16-byte loads (1 KiB
+// per wavefront instruction) one item ahead into registers, then written to LDS, from where the
+// MFMA operand layout (K) and the dims-per-lane layout (V) are read back.  Each of the eight
+// wavefronts stages exactly the 16 key rows it consumes, so staging needs no workgroup barrier.
+// The partial results of an item are written out one iteration late, off the critical path.
 // ---------------------------------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kSK = 128;                       // keys per tile
 constexpr int kStreamStage = 2 * kSK * 256;    // K rows then V rows of one tile (16-bit, 256 B per row)
-
-__device__ inline uint32_t lds_address(const void* p) {
-    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
-}
-
-// 16 bytes per lane from a per-lane global address to LDS (wave base in M0, lane i at +16 i)
-__device__ inline void async_row_copy16(const void* src, uint32_t lds_wave_base) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                 :
-                 : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(src)
-                 : "memory");
-}
-
-// the same with a uniform base (SGPR pair) plus a 32-bit per-lane byte offset
-__device__ inline void async_copy16_s(const void* sbase, uint32_t voff, uint32_t lds_wave_base) {
-    const uint64_t v = reinterpret_cast<uint64_t>(sbase);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(voff),
-                   "s"(reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo))
-                 : "memory");
-}
 
 // sum / max over the four 16-lane rows of a wavefront (lanes l, l^16, l^32, l^48)
 __device__ inline float rows4_sum(float x) {
@@ -613,15 +599,15 @@ __device__ inline float rows4_max(float x) {
     return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
 }
 
-inline int stream_lds_bytes(int G) { return 2 * kStreamStage + (8 * G * kD + 8 * G * 2 + 8 * 16 * 8) * (int)sizeof(float); }
+inline int stream_lds_bytes(int G) { return kStreamStage + (8 * G * kD + 8 * G * 2 + 8 * 16 * 8) * (int)sizeof(float); }
 
 template <typename T, int G>
 __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    float* red_o = reinterpret_cast<float*>(smem + 2 * kStreamStage);  // [8 waves][G][128]
+    float* red_o = reinterpret_cast<float*>(smem + kStreamStage);  // [8 waves][G][128]
     float* red_ml = red_o + 8 * G * kD;                                // [8][G][2]
     float* s_lds = red_ml + 8 * G * 2;                                 // [8][16 keys][8] logits, then [16][4] probabilities
-    const uint32_t smem_addr = lds_address(smem);
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)smem;
     const ckv_attn_args& a = p.a;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -631,15 +617,26 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
     const int64_t nbh = a.B * a.KVH, total = (int64_t)p.tiles * nbh;
     const int64_t item0 = total * blockIdx.x / gridDim.x, item1 = total * (blockIdx.x + 1) / gridDim.x;
     const int64_t NS = a.num_sink, S = a.S;
-    const bool cache_small = S * a.cache_stride[2] * (int64_t)sizeof(T) < (1ll << 31);  // 32-bit byte offsets reach every row
 
-    // LDS read offsets inside a stage.  K row r keeps source piece c at slot c ^ (r & 15), which
-    // makes the 16-byte operand reads conflict free; V rows are linear (a row is read as one
-    // 256-byte line, 4 bytes per lane).
+    // LDS read offsets.  K row r keeps source piece c at slot c ^ (r & 15), which makes the 16-byte
+    // operand reads conflict free.  V row r keeps piece c at slot c ^ ((r & 7) << 1): the transposing
+    // reads below take 32 bytes from each of four rows, and this puts the rows on different banks.
     int kaddr[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) kaddr[ks] = (wave * 16 + key16) * 256 + (((4 * ks + kq) ^ key16) << 4);
-    const int vaddr = kSK * 256 + wave * 16 * 256 + lane * 4;
+    // P.V on the matrix pipe, 16x16x16: A = V^T block (16 dims x 16 keys), B = P^T (16 keys x 16 heads).
+    // ds_read_b64_tr_b16 hands lane i of a 16-lane group element [4e + i/4][i%4] (e = 0..3) of the
+    // 16 x 4 matrix whose row r is the 8 bytes lane r points at.  With lane r of group q pointing at
+    // dims 16 blk + 4 (r%4) .. +3 of key 4q + r/4, lane i receives dim 16 blk + i of keys 4q .. 4q+3:
+    // the A operand.
+    int vt_addr[8];
+    {
+        const int r_l = lane & 15, key = 4 * (lane >> 4) + (r_l >> 2);
+#pragma unroll
+        for (int blk = 0; blk < 8; blk++) {
+            vt_addr[blk] = kSK * 256 + (wave * 16 + key) * 256 + 32 * (blk ^ (key & 7)) + 16 * ((r_l & 3) >> 1) + 8 * (r_l & 1);
+        }
+    }
 
     for (int64_t item = item0; item < item1;) {
         const int64_t tile = item / nbh, bh0 = item % nbh;
@@ -667,13 +664,9 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
         }
         // bit k: key n_wave + k is visible (lanes 0..15 are the sixteen keys)
         const uint32_t vis_keys = __builtin_amdgcn_readfirstlane((uint32_t)(__builtin_amdgcn_ballot_w64(vis1) & 0xffffull));
-        // copy rows of this lane: block jb holds rows 4 jb .. 4 jb + 3 of the wavefront's 16.
-        // Usual case: all 16 rows are cache slots and byte offsets fit 32 bits -> uniform base plus
-        // a per-lane offset, no address arithmetic per copy.
-        const bool one_seg = cache_small && n_wave >= NS && n_wave + 16 <= NS + S;
+        // rows loaded by this lane: block jb holds rows 4 jb .. 4 jb + 3 of the wavefront's 16, piece lane % 16
         int seg_c[4];
-        int64_t koff_c[4], voff_c[4];  // element offsets inside the (b, kvh) slab, source piece included
-        uint32_t koff32[4], voff32[4]; // the same in bytes for the usual case
+        int64_t off_c[4];  // element offset inside the (b, kvh) slab of the row's segment
 #pragma unroll
         for (int jb = 0; jb < 4; jb++) {
             const int r = 4 * jb + (lane >> 4);
@@ -682,25 +675,11 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
             if (n < NS) { seg_c[jb] = 0; row_off = n * a.sink_stride[2]; }
             else if (n < NS + S) { seg_c[jb] = 1; row_off = (n - NS) * a.cache_stride[2]; }
             else { seg_c[jb] = 2; row_off = 0; }  // the new token; rows past the end repeat it and stay hidden
-            koff_c[jb] = row_off + (((lane & 15) ^ (r & 15)) << 3);
-            voff_c[jb] = row_off + ((lane & 15) << 3);
-            koff32[jb] = (uint32_t)(koff_c[jb] * (int64_t)sizeof(T));
-            voff32[jb] = (uint32_t)(voff_c[jb] * (int64_t)sizeof(T));
+            off_c[jb] = row_off + ((lane & 15) << 3);
         }
-
-        auto issue = [&](int64_t bh, int stage) {
-            const int64_t b = bh / a.KVH, kvh = bh % a.KVH;
-            const uint32_t st = smem_addr + stage * kStreamStage;
-            if (one_seg) {
-                const T* kb = (const T*)a.cache_k + b * a.cache_stride[0] + kvh * a.cache_stride[1];
-                const T* vb = (const T*)a.cache_v + b * a.cache_stride[0] + kvh * a.cache_stride[1];
-#pragma unroll
-                for (int jb = 0; jb < 4; jb++) {
-                    async_copy16_s(kb, koff32[jb], st + (wave * 4 + jb) * 1024);
-                    async_copy16_s(vb, voff32[jb], st + kSK * 256 + (wave * 4 + jb) * 1024);
-                }
-                return;
-            }
+        // rows of one item: eight 16-byte pieces per lane (four K, four V blocks of 1 KiB per wavefront),
+        // loaded one item ahead into registers and written to LDS at the top of the item's iteration
+        auto load_rows = [&](int b, int kvh, u32x4(&kr)[4], u32x4(&vr)[4]) {
             const T* kseg[3] = {(const T*)a.sink_k + b * a.sink_stride[0] + kvh * a.sink_stride[1],
                                 (const T*)a.cache_k + b * a.cache_stride[0] + kvh * a.cache_stride[1],
                                 (const T*)a.k_new + b * a.kv_new_stride[0] + kvh * a.kv_new_stride[1]};
@@ -711,31 +690,33 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
             for (int jb = 0; jb < 4; jb++) {
                 const T* kb = seg_c[jb] == 0 ? kseg[0] : (seg_c[jb] == 1 ? kseg[1] : kseg[2]);
                 const T* vb = seg_c[jb] == 0 ? vseg[0] : (seg_c[jb] == 1 ? vseg[1] : vseg[2]);
-                async_row_copy16(kb + koff_c[jb], st + (wave * 4 + jb) * 1024);
-                async_row_copy16(vb + voff_c[jb], st + kSK * 256 + (wave * 4 + jb) * 1024);
+                kr[jb] = *reinterpret_cast<const u32x4*>(kb + off_c[jb]);
+                vr[jb] = *reinterpret_cast<const u32x4*>(vb + off_c[jb]);
             }
         };
         // A operand: rotated queries of the group's heads (rows >= G are zero)
-        auto load_q = [&](int64_t bh, uint4(&q)[4]) {
-            const int64_t b = bh / a.KVH, kvh = bh % a.KVH;
-            const T* qr = (const T*)p.qrot_t + ((b * a.H) + kvh * G + key16) * kD;
+        auto load_q = [&](int b, int kvh, uint4(&q)[4]) {
+            const T* qr = (const T*)p.qrot_t + (((int64_t)b * a.H) + kvh * G + key16) * kD;
 #pragma unroll
             for (int ks = 0; ks < 4; ks++)
                 q[ks] = key16 < G ? *reinterpret_cast<const uint4*>(qr + 32 * ks + 8 * kq) : make_uint4(0, 0, 0, 0);
         };
 
         uint4 q_next[4];
-        load_q(bh0, q_next);
-        issue(bh0, 0);
+        u32x4 k_next[4], v_next[4];  // plain vectors: an aggregate copied to LDS would be kept in scratch
+        // (batch, kv head) of the item in hand and of the next one, stepped without divisions
+        const int KVH = (int)a.KVH;
+        int b = (int)(bh0 / KVH), kvh = (int)(bh0 % KVH);
+        load_q(b, kvh, q_next);
+        load_rows(b, kvh, k_next, v_next);
         bool pending = false;
-        int64_t pend_bh = 0;
+        int pend_b = 0, pend_kvh = 0;
         float pend_o = 0.f, pend_m = 0.f, pend_l = 0.f;
         auto flush = [&]() {
             if (!pending) return;
-            const int64_t b = pend_bh / a.KVH, kvh = pend_bh % a.KVH;
             if (tid < G * kD) {
                 const int g = tid >> 7, d = tid & 127;
-                const int64_t row = (b * a.H + kvh * G + g) * p.tiles + tile;
+                const int64_t row = ((int64_t)pend_b * a.H + pend_kvh * G + g) * p.tiles + tile;
                 p.part_o[row * kD + d] = pend_o;
                 if (d == 0) {
                     p.part_ml[row * 2] = pend_m;
@@ -743,21 +724,29 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
                 }
             }
         };
-        int stage = 0;
-        for (int64_t bh = bh0; bh < bh1; bh++, stage ^= 1) {
-            const int64_t b = bh / a.KVH, kvh = bh % a.KVH;
-            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the rows of this item are in LDS
+        for (int64_t bh = bh0; bh < bh1; bh++) {
+            // this wavefront's 16 rows go to LDS (it is their only reader, so no workgroup barrier);
+            // K piece c of row r lands in slot c ^ (r & 15)
+#pragma unroll
+            for (int jb = 0; jb < 4; jb++) {
+                const int r = 4 * jb + (lane >> 4);
+                *reinterpret_cast<u32x4*>(smem + (wave * 16 + r) * 256 + (((lane & 15) ^ (r & 15)) << 4)) = k_next[jb];
+                *reinterpret_cast<u32x4*>(smem + kSK * 256 + (wave * 16 + r) * 256 + (((lane & 15) ^ ((r & 7) << 1)) << 4)) = v_next[jb];
+            }
             uint4 qop[4];
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                qop[ks] = q_next[ks];
-                // use the operand here so that the wait for its load is placed here too, ahead of the next copies
-                asm volatile("" : "+v"(qop[ks].x), "+v"(qop[ks].y), "+v"(qop[ks].z), "+v"(qop[ks].w));
+            for (int ks = 0; ks < 4; ks++) qop[ks] = q_next[ks];
+            int b_nx = b, kvh_nx = kvh;
+            if (bh + 1 < bh1) {  // the last item of a run loads itself again: cheaper than a branch around the loads
+                kvh_nx = kvh + 1 == KVH ? 0 : kvh + 1;
+                b_nx = kvh + 1 == KVH ? b + 1 : b;
             }
-            if (bh + 1 < bh1) load_q(bh + 1, q_next);
+            load_q(b_nx, kvh_nx, q_next);
+            load_rows(b_nx, kvh_nx, k_next, v_next);
             flush();
-            if (bh + 1 < bh1) issue(bh + 1, stage ^ 1);
-            const unsigned char* st = smem + stage * kStreamStage;
+            const unsigned char* st = smem;
+            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the rows are in LDS
+            __builtin_amdgcn_wave_barrier();
 
             // ---- phase 1: rotate K in registers, logits by MFMA, share them through LDS
             {
@@ -793,7 +782,7 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
                     if (g < G) {
                         const float sv = vis1 ? sacc[v] * p.scale_log2 : -INFINITY;
                         s_wave[key16 * 8 + g] = sv;
-                        if (n < p.N) p.logits[((b * a.KVH + kvh) * p.N + n) * G + g] = sv;
+                        if (n < p.N) p.logits[(((int64_t)b * KVH + kvh) * p.N + n) * G + g] = sv;
                     }
                 }
             }
@@ -813,7 +802,8 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
                 l += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(l), 0x128, 0xF, 0xF, true));
                 l = rows4_sum(l);
                 __builtin_amdgcn_wave_barrier();      // every lane has read its logit
-                s_wave[pkey * 4 + pg] = pe;           // probabilities, 4 per key
+                // probabilities in the tensor dtype, [head][16 keys] (hidden keys: 0)
+                reinterpret_cast<unsigned short*>(s_wave)[pg * 16 + pkey] = (unsigned short)Mma16<T>::pack2(pe, 0.f);
                 if (pkey == 0 && pg < G) {
                     red_ml[(wave * G + pg) * 2] = m;
                     red_ml[(wave * G + pg) * 2 + 1] = l;
@@ -821,26 +811,31 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
-            // ---- phase 2b: weighted V sum; lane owns dims 2 lane, 2 lane + 1 of every row
-            float o[G][2];
+            // ---- phase 2b: weighted V sum on the matrix pipe.  Lane 16 q + g (g < G) ends up with
+            //      dims 16 blk + 4 q .. + 3 of head g.  Rows of hidden slots may hold anything (their
+            //      probability is zero, but 0 * NaN is not), so they are zeroed on the way in.
+            {
+                const int g = lane & 15, q4 = lane >> 4;
+                uint2 pb = make_uint2(0u, 0u);
+                if (g < G) pb = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned char*>(s_wave) + g * 32 + q4 * 8);
+                // this lane's operand pieces are keys 4 q4 .. 4 q4 + 3
+                const uint32_t vk = (vis_keys >> (4 * q4)) & 0xfu;
+                const uint32_t m01 = ((vk & 1u) ? 0x0000ffffu : 0u) | ((vk & 2u) ? 0xffff0000u : 0u);
+                const uint32_t m23 = ((vk & 4u) ? 0x0000ffffu : 0u) | ((vk & 8u) ? 0xffff0000u : 0u);
 #pragma unroll
-            for (int g = 0; g < G; g++) o[g][0] = o[g][1] = 0.f;
-#pragma unroll
-            for (int kk = 0; kk < 16; kk++) {
-                if (!((vis_keys >> kk) & 1u)) continue;  // hidden slots may hold anything
-                const float4 p4 = *reinterpret_cast<const float4*>(s_wave + kk * 4);
-                const uint32_t vv = *reinterpret_cast<const uint32_t*>(st + vaddr + kk * 256);
-                const float v0 = Mma16<T>::lo(vv), v1 = Mma16<T>::hi(vv);
-                const float pp[4] = {p4.x, p4.y, p4.z, p4.w};
-#pragma unroll
-                for (int g = 0; g < G; g++) {
-                    o[g][0] = fmaf(pp[g], v0, o[g][0]);
-                    o[g][1] = fmaf(pp[g], v1, o[g][1]);
+                for (int blk = 0; blk < 8; blk++) {
+                    const s16x4_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(lds_base + vt_addr[blk]));
+                    uint2 av = __builtin_bit_cast(uint2, va);
+                    av.x &= m01;
+                    av.y &= m23;
+                    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                    const f32x4 acc = Mma16<T>::mma_k16(av, pb, zero);
+                    if (g < G)
+                        *reinterpret_cast<float4*>(red_o + (wave * G + g) * kD + 16 * blk + 4 * q4) =
+                            make_float4(acc[0], acc[1], acc[2], acc[3]);
                 }
             }
-#pragma unroll
-            for (int g = 0; g < G; g++)
-                *reinterpret_cast<float2*>(red_o + (wave * G + g) * kD + 2 * lane) = make_float2(o[g][0], o[g][1]);
             __syncthreads();
             // ---- combine the eight wavefronts; the result is stored at the top of the next iteration
             if (tid < G * kD) {
@@ -861,7 +856,10 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
                 pend_l = L;
             }
             pending = true;
-            pend_bh = bh;
+            pend_b = b;
+            pend_kvh = kvh;
+            b = b_nx;
+            kvh = kvh_nx;
             __syncthreads();  // red_* may be overwritten
         }
         flush();
