@@ -27,6 +27,10 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
+# HBM bytes per launch of the dominant kernels on the bench workloads, measured with rocprofv3 --pmc
+# FETCH_SIZE and WRITE_SIZE (one pass each), each scaled by the reading for a 512 MiB device copy in the
+# same run (profiles/hbm_traffic_bench_kernels.md).  Counters cannot be read inside this process.
+TRAFFIC_BYTES = {"fwd_pipe_kernel": 1.125e9, "decode_stream_kernel": 2.322e9}
 
 PREFILL = dict(B=2, H=32, KVH=8, D=128, NS=64, S=16384, C=8, Q=2048, theta=5e5, seed=2)
 DECODE = dict(B=16, H=32, KVH=8, D=128, NS=64, S=32768, C=4, Q=1, theta=5e5, seed=3)
@@ -106,7 +110,7 @@ def run_prefill(steps, warmup, dtype, device):
         ms_per_step=dt / steps * 1e3,
         tokens_per_s=B * Q * steps / dt,
         roofline=dict(bound="mfma", achieved=achieved, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                      frac=achieved / PEAK_BF16_TFLOPS, traffic=None, kernel="fwd_mfma_kernel",
+                      frac=achieved / PEAK_BF16_TFLOPS, traffic=TRAFFIC_BYTES["fwd_pipe_kernel"], kernel="fwd_pipe_kernel",
                       kernel_ms=fwd_avg_ms, algorithmic_tflop_per_launch=flops_fwd / 1e12),
         stage_ms=stage_ms,
         attention_tflops_all_stages=(flops_fwd + 2.0 * B * H * Q * (n_cached + Q)) / (attn_ms * 1e-3) / 1e12
@@ -171,7 +175,8 @@ def run_decode(steps, warmup, dtype, device):
         ms_per_step=dt / steps * 1e3,
         tokens_per_s=B * steps / dt,
         roofline=dict(bound="hbm", achieved=achieved, peak=PEAK_HBM_GBPS, unit="GB/s", frac=achieved / PEAK_HBM_GBPS,
-                      traffic=None, kernel_ms=main_ms, algorithmic_gb_per_launch=algo_bytes / 1e9),
+                      traffic=TRAFFIC_BYTES["decode_stream_kernel"], kernel="decode_stream_kernel", kernel_ms=main_ms,
+                      algorithmic_gb_per_launch=algo_bytes / 1e9),
         stage_ms=stage_ms,
     )
 
@@ -215,6 +220,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 512 MiB device copy, the known-size reference that scales the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU mode (every (batch, kv-head) unit is "
@@ -230,6 +238,13 @@ def main():
     del cache, pool
     torch.cuda.empty_cache()
     dec = None if args.no_decode else run_decode(max(args.steps, 20), args.warmup, dtype, device)
+    if args.calibrate_copy:
+        src = torch.ones(512 << 20, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     line = {
         "metric": "prefill+decode tokens/s (8B-shape, C=8, 64K window); MFMA% and HBM GB/s vs peak",
         "value": pre["tokens_per_s"],
