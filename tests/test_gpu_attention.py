@@ -169,6 +169,52 @@ def test_decode_head128(H, KVH, W, C, NS, eager, dtype):
             assert_scores_close(gpu.score_cache[0], cpu.score_cache, dtype, f"step {c} score cache")
 
 
+@pytest.mark.parametrize("H,KVH,dtype,fill", [
+    (32, 8, torch.bfloat16, 3000),   # G = 4, cache partly filled: hidden slots inside most tiles
+    (32, 8, torch.bfloat16, 6000),   # G = 4, cache full and evicting
+    (16, 8, torch.float16, 2500),    # G = 2
+    (8, 8, torch.bfloat16, 3500),    # G = 1
+])
+def test_decode_streaming_many_items(H, KVH, dtype, fill):
+    """Decode over a few thousand slots with 16 (batch, kv-head) units: more (tile, unit) items than
+    workgroups, so a workgroup walks several items and crosses key-tile boundaries.  The cache is
+    filled through the oracle's update alone (random keys, values and scores), and the hidden slots of
+    the GPU copy are poisoned with NaN: nothing of a hidden slot may reach the output."""
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
+
+    B, D, NS, W, C = 2, 128, 4, 1024, 4
+    gpu, cpu = make_pair(B, KVH, D, NS, W, C, dtype)
+    layer = OracleCascadeAttention(H, KVH, D, rope_theta=5e5)
+    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    gen = torch.Generator().manual_seed(5)
+    done = 0
+    while done < fill:
+        n = min(512, fill - done)
+        k = (torch.randn(B, KVH, n, D, generator=gen) * 0.7).to(dtype)
+        v = (torch.randn(B, KVH, n, D, generator=gen) * 0.7).to(dtype)
+        s = torch.rand(B, KVH, n, generator=gen).to(dtype)
+        cpu.update(k, v, s)
+        done += n
+    layer.query_pos = torch.arange(0, 512, dtype=torch.long).view(1, -1)  # what a first prefill chunk leaves behind
+    for step in range(3):
+        q = (torch.randn(B, H, 1, D, generator=gen) * 0.7).to(dtype)
+        k = (torch.randn(B, KVH, 1, D, generator=gen) * 0.7).to(dtype)
+        v = (torch.randn(B, KVH, 1, D, generator=gen) * 0.7).to(dtype)
+        push_state(gpu, cpu)
+        hidden = gpu.mask[0].bool().expand(gpu.key_cache[0].shape[:-1])
+        gpu.key_cache[0][hidden] = float("nan")
+        gpu.value_cache[0][hidden] = float("nan")
+        out_g, new_g = cascade_attention(q.cuda(), k.cuda(), v.cuda(), gpu, 0, inv_freq)
+        out_c = layer.forward(q, k, v, cpu)
+        torch.cuda.synchronize()
+        assert torch.isfinite(out_g.float()).all(), f"step {step}: a hidden slot leaked into the output"
+        err = (out_g.float().cpu() - out_c.float()).abs().max().item()
+        assert err <= tol(dtype), f"step {step}: out max err {err:.3e}"
+        assert_scores_close(new_g, layer.last_new_scores[:, :KVH], dtype, f"step {step} new-token scores")
+        for name in META:
+            assert torch.equal(getattr(gpu, name)[0].cpu(), getattr(cpu, name)), f"step {step}: {name}"
+
+
 def dense_reference(q, k, v, mask, sm_scale):
     n_ctx, n_kv = q.size(2), k.size(2)
     logits = torch.matmul(q.float(), k.float().transpose(2, 3)) * sm_scale
