@@ -391,7 +391,7 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
                 for (int e = 0; e < 8; e++) {
                     const int f = 32 * ks + 8 * kq + e;
                     const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                    sincosf(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
+                    fast_sincos(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
                 }
         }
     }
@@ -459,7 +459,7 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
                     for (int e = 0; e < 8; e++) {
                         const int f = 32 * ks + 8 * kq + e;
                         const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                        sincosf(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
+                        fast_sincos(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
                     }
             }
             uint4 kop[4];
@@ -659,7 +659,7 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
                 for (int e = 0; e < 8; e++) {
                     const int f = 32 * ks + 8 * kq + e;
                     const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                    sincosf(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
+                    fast_sincos(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
                 }
         }
         // bit k: key n_wave + k is visible (lanes 0..15 are the sixteen keys)

@@ -135,7 +135,7 @@ __global__ void __launch_bounds__(256) stage_keys_kernel(StageParams p) {
         for (int i = 0; i < 16; i++) {
             const int j = 16 * quarter + i;
             const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
-            sincosf(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
+            fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
         }
     }
     const int64_t nbh = p.B * p.KVH;
@@ -176,7 +176,7 @@ __global__ void __launch_bounds__(256) stage_keys_kernel(StageParams p) {
                     for (int i = 0; i < 16; i++) {
                         const int j = 16 * quarter + i;
                         const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
-                        sincosf(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
+                        fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
                     }
                 }
                 T* l0 = reinterpret_cast<T*>(lo);
@@ -240,54 +240,61 @@ struct StageQParams {
     int vec;                 // source rows can be read 16 bytes at a time
 };
 
+// thread = (position m, quarter of the rotation pairs); the cos/sin of the position are computed once
+// and reused for the batch x head rows of the block's share (blockIdx.y of gridDim.y)
 template <typename T>
 __global__ void __launch_bounds__(256) stage_q_kernel(StageQParams p) {
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t row = idx >> 2;
+    const int64_t m = idx >> 2;
     const int quarter = idx & 3;
-    if (row >= p.rows) return;
-    const int64_t m = row % p.Q, h = (row / p.Q) % p.H, b = row / (p.Q * p.H);
-    const T* src = (const T*)p.q + b * p.stride[0] + h * p.stride[1] + m * p.stride[2];
-    T lo[16], hi[16];
-    if (p.vec) {  // unit stride and 16-byte aligned rows
-        reinterpret_cast<uint4*>(lo)[0] = *reinterpret_cast<const uint4*>(src + 16 * quarter);
-        reinterpret_cast<uint4*>(lo)[1] = *reinterpret_cast<const uint4*>(src + 16 * quarter + 8);
-        reinterpret_cast<uint4*>(hi)[0] = *reinterpret_cast<const uint4*>(src + 64 + 16 * quarter);
-        reinterpret_cast<uint4*>(hi)[1] = *reinterpret_cast<const uint4*>(src + 64 + 16 * quarter + 8);
-    } else {
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            lo[i] = src[(16 * quarter + i) * p.stride[3]];
-            hi[i] = src[(64 + 16 * quarter + i) * p.stride[3]];
-        }
-    }
-    // the softmax scale (times log2 e) rides on the staged queries: one rounding to the tensor
-    // dtype after rotation and scaling, and the attention kernels exponentiate the products as
-    // they come out of the matrix pipe
+    if (m >= p.Q) return;
+    float cs[16], sn[16];
     if (p.q_pos) {
         const int64_t pos = p.q_pos[m];
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const int j = 16 * quarter + i;
             const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
-            float sn, cs;
-            sincosf(__fmul_rn((float)pos, f), &sn, &cs);
-            const float x1 = Elem<T>::to_float(lo[i]), x2 = Elem<T>::to_float(hi[i]);
-            lo[i] = Elem<T>::from_float((x1 * cs - x2 * sn) * p.qscale);
-            hi[i] = Elem<T>::from_float((x2 * cs + x1 * sn) * p.qscale);
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            lo[i] = Elem<T>::from_float(Elem<T>::to_float(lo[i]) * p.qscale);
-            hi[i] = Elem<T>::from_float(Elem<T>::to_float(hi[i]) * p.qscale);
+            fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
         }
     }
-    T* dst = (T*)p.qr + row * kD;
-    *reinterpret_cast<uint4*>(dst + 16 * quarter) = reinterpret_cast<uint4*>(lo)[0];
-    *reinterpret_cast<uint4*>(dst + 16 * quarter + 8) = reinterpret_cast<uint4*>(lo)[1];
-    *reinterpret_cast<uint4*>(dst + 64 + 16 * quarter) = reinterpret_cast<uint4*>(hi)[0];
-    *reinterpret_cast<uint4*>(dst + 64 + 16 * quarter + 8) = reinterpret_cast<uint4*>(hi)[1];
+    const int64_t nbh = p.rows / p.Q;
+    for (int64_t bh = blockIdx.y; bh < nbh; bh += gridDim.y) {
+        const int64_t b = bh / p.H, h = bh % p.H;
+        const T* src = (const T*)p.q + b * p.stride[0] + h * p.stride[1] + m * p.stride[2];
+        T lo[16], hi[16];
+        if (p.vec) {  // unit stride and 16-byte aligned rows
+            reinterpret_cast<uint4*>(lo)[0] = *reinterpret_cast<const uint4*>(src + 16 * quarter);
+            reinterpret_cast<uint4*>(lo)[1] = *reinterpret_cast<const uint4*>(src + 16 * quarter + 8);
+            reinterpret_cast<uint4*>(hi)[0] = *reinterpret_cast<const uint4*>(src + 64 + 16 * quarter);
+            reinterpret_cast<uint4*>(hi)[1] = *reinterpret_cast<const uint4*>(src + 64 + 16 * quarter + 8);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                lo[i] = src[(16 * quarter + i) * p.stride[3]];
+                hi[i] = src[(64 + 16 * quarter + i) * p.stride[3]];
+            }
+        }
+        // the softmax scale (times log2 e) rides on the staged queries: one rounding to the tensor
+        // dtype after rotation and scaling, and the attention kernels exponentiate the products as
+        // they come out of the matrix pipe
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float x1 = Elem<T>::to_float(lo[i]), x2 = Elem<T>::to_float(hi[i]);
+            if (p.q_pos) {
+                lo[i] = Elem<T>::from_float((x1 * cs[i] - x2 * sn[i]) * p.qscale);
+                hi[i] = Elem<T>::from_float((x2 * cs[i] + x1 * sn[i]) * p.qscale);
+            } else {
+                lo[i] = Elem<T>::from_float(x1 * p.qscale);
+                hi[i] = Elem<T>::from_float(x2 * p.qscale);
+            }
+        }
+        T* dst = (T*)p.qr + (bh * p.Q + m) * kD;
+        *reinterpret_cast<uint4*>(dst + 16 * quarter) = reinterpret_cast<uint4*>(lo)[0];
+        *reinterpret_cast<uint4*>(dst + 16 * quarter + 8) = reinterpret_cast<uint4*>(lo)[1];
+        *reinterpret_cast<uint4*>(dst + 64 + 16 * quarter) = reinterpret_cast<uint4*>(hi)[0];
+        *reinterpret_cast<uint4*>(dst + 64 + 16 * quarter + 8) = reinterpret_cast<uint4*>(hi)[1];
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1008,7 +1015,14 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         sq.qscale = scale_log2;
         sq.vec = mp.q_stride[3] == 1 && reinterpret_cast<uintptr_t>(mp.q) % 16 == 0 && mp.q_stride[0] % 8 == 0 &&
                  mp.q_stride[1] % 8 == 0 && mp.q_stride[2] % 8 == 0;
-        hipLaunchKernelGGL(stage_q_kernel<T>, dim3((unsigned)((sq.rows * 4 + 255) / 256)), dim3(256), 0, stream, sq);
+        {
+            // enough blocks to fill the chip; the rest of batch x heads is looped over inside, sharing cos/sin
+            const int64_t bx = (mp.Q * 4 + 255) / 256, nbh_q = mp.B * mp.H;
+            int64_t by = (1024 + bx - 1) / bx;
+            if (by > nbh_q) by = nbh_q;
+            if (by < 1) by = 1;
+            hipLaunchKernelGGL(stage_q_kernel<T>, dim3((unsigned)bx, (unsigned)by), dim3(256), 0, stream, sq);
+        }
         CKV_HIP_TRY(hipGetLastError());
     }
     const int G = (int)(mp.H / mp.KVH);
