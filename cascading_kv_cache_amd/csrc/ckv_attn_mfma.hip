@@ -308,7 +308,7 @@ struct FwdParams {
     void* out;
     int64_t out_stride[4];
     float* lse;       // (B*H, Q) natural log
-    float* lse2;      // (B*H, Q) log2 domain, consumed by the column pass
+    float* lse2;      // (B*H, Q) minus the log2-domain normaliser, consumed by the column pass
     int64_t B, H, KVH, Q, N, Nc, n_pad;
     int G, QT;        // heads per kv head, positions per workgroup (G * QT <= 256)
     float scale_log2; // softmax scale * log2(e)
@@ -690,7 +690,7 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
         if (half == 0) {
             const float l2 = m_run + __builtin_amdgcn_logf(l_tot);  // v_log_f32 is log2
             p.lse[(b * p.H + row_h) * p.Q + row_m] = l2 * 0.6931471805599453f;
-            p.lse2[(b * p.H + row_h) * p.Q + row_m] = l2;
+            p.lse2[(b * p.H + row_h) * p.Q + row_m] = -l2;
         }
     }
 }
@@ -702,7 +702,7 @@ struct ColsumParams {
     const void* qr;       // (B*H*Q + 64 rows of slack, D)
     const void* kr;
     const unsigned long long* tile_vis;
-    const float* lse2;    // (B*H*Q + 64) log2-domain row normalisers
+    const float* lse2;    // (B*H*Q + 64) minus the log2-domain row normalisers
     const float* w_ema;   // (Q + 64), zero beyond Q
     const float* w_new;   // (Q)
     float* colsum;        // (B*H, N)
@@ -822,13 +822,24 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
         const float* lse_lds = reinterpret_cast<const float*>(q_lds + 16384);
         const float* w_lds = lse_lds + 64;
 
+        // The accumulators start from minus the row normaliser, so the matrix pipe hands back
+        // log2 P directly (the softmax scale is already on the staged queries).
+        // Element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4.
         f32x16 sacc[2][2];  // [c = query subtile][ks]
 #pragma unroll
-        for (int c = 0; c < 2; c++)
+        for (int c = 0; c < 2; c++) {
+            f32x16 init;
 #pragma unroll
-            for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) sacc[c][ks][v] = 0.f;
+            for (int v4 = 0; v4 < 4; v4++) {
+                const float4 l4 = *reinterpret_cast<const float4*>(lse_lds + 32 * c + 8 * v4 + 4 * half);
+                init[4 * v4] = l4.x;
+                init[4 * v4 + 1] = l4.y;
+                init[4 * v4 + 2] = l4.z;
+                init[4 * v4 + 3] = l4.w;
+            }
+            sacc[c][0] = init;
+            sacc[c][1] = init;
+        }
 #pragma unroll
         for (int kk = 0; kk < 8; kk++) {
 #pragma unroll
@@ -857,13 +868,11 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
 #pragma unroll
                 for (int v4 = 0; v4 < 4; v4++) {
                     const int r0 = 32 * c + 8 * v4;
-                    const float4 l4 = *reinterpret_cast<const float4*>(lse_lds + r0 + 4 * half);
-                    const float ls[4] = {l4.x, l4.y, l4.z, l4.w};
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
 #pragma unroll
                         for (int ks = 0; ks < 2; ks++) {
-                            const float pe = __builtin_amdgcn_exp2f(fmaf(sacc[c][ks][4 * v4 + e], p.scale_log2, -ls[e]));
+                            const float pe = __builtin_amdgcn_exp2f(sacc[c][ks][4 * v4 + e]);
                             const float w = wb[ks][r0 + e];
                             if (pure_chunk) {
                                 acc[ks] += Mma<T>::round1(Mma<T>::round1(pe) * w);
@@ -881,15 +890,13 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
 #pragma unroll
                 for (int v4 = 0; v4 < 4; v4++) {
                     const int r0 = 32 * c + 8 * v4 + 4 * half;
-                    const float4 l4 = *reinterpret_cast<const float4*>(lse_lds + r0);
                     const float4 w4 = *reinterpret_cast<const float4*>(w_lds + r0);
-                    const float ls[4] = {l4.x, l4.y, l4.z, l4.w};
                     const float ws[4] = {w4.x, w4.y, w4.z, w4.w};
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
 #pragma unroll
                         for (int ks = 0; ks < 2; ks++) {
-                            const float pe = __builtin_amdgcn_exp2f(fmaf(sacc[c][ks][4 * v4 + e], p.scale_log2, -ls[e]));
+                            const float pe = __builtin_amdgcn_exp2f(sacc[c][ks][4 * v4 + e]);
                             acc[ks] = fmaf(ws[e], pe, acc[ks]);
                         }
                     }
@@ -903,11 +910,10 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
                     const int r = 32 * c + 8 * (v >> 2) + 4 * half + (v & 3);
                     const int m = mt + r;
                     const bool row_in = m < Q;
-                    const float l2 = lse_lds[r];
                     const float we = w_lds[r];
 #pragma unroll
                     for (int ks = 0; ks < 2; ks++) {
-                        float pe = __builtin_amdgcn_exp2f(fmaf(sacc[c][ks][v], p.scale_log2, -l2));
+                        float pe = __builtin_amdgcn_exp2f(sacc[c][ks][v]);
                         const bool is_chunk = nrel[ks] >= 0;
                         const bool vis = row_in && (!is_chunk || m >= nrel[ks]);
                         pe = vis ? pe : 0.f;
