@@ -170,12 +170,19 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
     return CKV_OK;
 }
 
+namespace ckv {
+// 16-bit, head_dim 128, more than one query row: the dense operator runs on the MFMA kernels too
+static bool dense_uses_mfma(int dtype, int64_t D, int64_t H, int64_t n_ctx, int64_t n_kv) {
+    return n_ctx > 1 && mfma_supported(dtype, D, H, H, n_ctx) && mfma_fits(n_kv);
+}
+}  // namespace ckv
+
 extern "C" int64_t ckv_dense_workspace_bytes(int64_t B, int64_t H, int64_t n_ctx, int64_t n_kv, int64_t D,
                                              int32_t dtype) {
-    (void)D;
-    (void)dtype;
     if (B <= 0 || H <= 0 || n_ctx <= 0 || n_kv < n_ctx) return 0;
     using ckv::align_up;
+    if (ckv::dense_uses_mfma(dtype, D, H, n_ctx, n_kv))  // staged Q / K / V^T and the column pass's scratch
+        return ckv::carve_attn(nullptr, B, H, H, n_ctx, D, 0, n_kv - n_ctx, dtype).bytes;
     return align_up(B * H * n_ctx * 4, 256) + align_up(B * H * n_kv * 4, 256) + 2 * align_up((n_ctx + 64) * 4, 256);
 }
 
@@ -191,6 +198,48 @@ extern "C" int ckv_attn_dense(const ckv_dense_args* args, void* stream_) {
     if (!(a.beta > 0.0) || !(a.beta <= 1.0)) return CKV_ERR_SHAPE;
     const int64_t need = ckv_dense_workspace_bytes(a.B, a.H, a.n_ctx, a.n_kv, a.D, a.dtype);
     if (!a.workspace || a.workspace_bytes < need) return CKV_ERR_WORKSPACE;
+    if (dense_uses_mfma(a.dtype, a.D, a.H, a.n_ctx, a.n_kv)) {
+        // keys and queries arrive rotated (no position ids); every head is its own kv head
+        const int64_t n_cache = a.n_kv - a.n_ctx;
+        AttnWorkspace w = carve_attn(a.workspace, a.B, a.H, a.H, a.n_ctx, a.D, 0, n_cache, a.dtype);
+        int rc;
+        if (a.scores) {
+            rc = launch_weights(w.w_ema, w.w_new, a.n_ctx, a.beta, a.dtype, stream);
+            if (rc) return rc;
+        }
+        const int64_t es = a.dtype == CKV_F32 ? 4 : 2;
+        MfmaProblem mp;
+        const MfmaSegment none{nullptr, nullptr, {0, 0, 0, 0}, nullptr, {0, 0}, 0, nullptr, 0};
+        mp.seg[0] = MfmaSegment{a.k, a.v, {a.kv_stride[0], a.kv_stride[1], a.kv_stride[2], a.kv_stride[3]},
+                                nullptr, {0, 0}, 0, n_cache > 0 ? a.mask : nullptr, n_cache};
+        mp.seg[1] = none;
+        mp.seg[2] = MfmaSegment{(const char*)a.k + n_cache * a.kv_stride[2] * es, (const char*)a.v + n_cache * a.kv_stride[2] * es,
+                                {a.kv_stride[0], a.kv_stride[1], a.kv_stride[2], a.kv_stride[3]},
+                                nullptr, {0, 0}, 0, nullptr, a.n_ctx};
+        mp.q = a.q;
+        for (int i = 0; i < 4; i++) { mp.q_stride[i] = a.q_stride[i]; mp.out_stride[i] = a.out_stride[i]; }
+        mp.q_pos = nullptr;
+        mp.inv_freq = nullptr;
+        mp.theta = 1.f;
+        mp.shared_pos = 1;
+        mp.qr = w.qr; mp.kr = w.kr; mp.vt = w.vc; mp.tile_vis = w.tile_vis;
+        mp.out = a.out;
+        mp.lse = w.lse;
+        mp.lse2 = w.lse2;
+        mp.colsum = a.scores ? w.colsum : nullptr;
+        mp.w_ema = w.w_ema; mp.w_new = w.w_new;
+        mp.new_mode = 0;  // every key is weighted by the query row alone (flash_attention.py:73-77)
+        mp.B = a.B; mp.H = a.H; mp.KVH = a.H; mp.Q = a.n_ctx; mp.n = a.n_kv; mp.n_pad = mfma_n_pad(a.n_kv);
+        mp.scale = a.scale;
+        mp.dtype = a.dtype;
+        rc = launch_mfma(mp, stream);
+        if (rc) return rc;
+        if (a.scores) {
+            rc = launch_cast_scores(w.colsum, a.scores, a.scores_stride, a.B, a.H, a.n_kv, a.dtype, stream);
+            if (rc) return rc;
+        }
+        return CKV_OK;
+    }
     Carver c(a.workspace);
     float* lse = (float*)c.take(a.B * a.H * a.n_ctx * 4);
     float* colsum = (float*)c.take(a.B * a.H * a.n_kv * 4);

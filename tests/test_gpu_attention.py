@@ -228,6 +228,8 @@ def dense_reference(q, k, v, mask, sm_scale):
 @pytest.mark.parametrize("Z,H,N_CTX,N_KV,HEAD_DIM", [
     (1, 2, 128, 128, 64), (1, 2, 256, 256, 64), (1, 1, 128, 128 + 128, 64), (1, 2, 512, 2560, 64),
     (1, 2, 500, 2048 + 500, 64), (1, 2, 500, 2048 + 64 + 500, 64), (2, 4, 256, 1024 + 256, 128),
+    # head_dim 128 in 16-bit runs on the matrix-core kernels: ragged sizes, no cache at all, long cache
+    (1, 2, 500, 2048 + 64 + 500, 128), (2, 3, 384, 384, 128), (1, 2, 130, 4096 + 130, 128),
 ])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_dense_operator_forward(Z, H, N_CTX, N_KV, HEAD_DIM, dtype):
