@@ -522,8 +522,10 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     // the other K stage) go out one at a time, a quarter of the slots apart.
     // pre[]: on entry the operands of slots 0..kAhead-1, read before the barrier; on exit those
     // of the next iteration.
+    // fetch_idx / fetched: the work-list entry three tiles ahead is read from LDS in the middle of the
+    // slots, so its latency is never waited for.
     auto iteration = [&](auto stage_tag, auto with_pv, int entry, int t_v, int t_k, int v_rd, int v_wr, f32x16(&s_cur)[2],
-                         f32x16(&s_nxt)[2], uint4(&pre)[kAhead]) {
+                         f32x16(&s_nxt)[2], uint4(&pre)[kAhead], int fetch_idx, int& fetched) {
         constexpr int ST = decltype(stage_tag)::value;
         constexpr bool kPV = decltype(with_pv)::value;
         constexpr int kSlots = kPV ? 32 : 16, kQk0 = kPV ? 16 : 0;
@@ -554,6 +556,7 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
         // the source offset of a copy is read from LDS two slots before the copy, so that waiting
         // for it does not also wait for the operand reads issued since
         uint32_t src = src_lds[tid];
+        int raw_entry = 0;
 #pragma unroll
         for (int k = 0; k < kSlots; k++) {
             if (k + kAhead < kSlots) ops[k + kAhead] = operand(k + kAhead);
@@ -563,6 +566,7 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
                 else copy_k(t_k, 1 - ST, q - 2, src);
             }
             if (k % kCopyStep == kCopyStep - 1 && k + 2 < kSlots) src = src_lds[((k + 2) / kCopyStep) * kThreads + tid];
+            if (k == 4) raw_entry = list_lds[fetch_idx];
             if (k >= kQk0) {
                 const int j = k - kQk0;
                 const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -606,6 +610,7 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
             __builtin_amdgcn_sched_barrier(0);
         }
         l_run = l_run * alpha + (rs0 + rs1);
+        fetched = __builtin_amdgcn_readfirstlane(raw_entry);
         // first operands of the next iteration: V^T tile i, complete since the last barrier
         {
             const int v_next = v_rd == 2 ? 0 : v_rd + 1;
@@ -633,28 +638,27 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
         qk(S0{}, sA);
-        // iteration 0: nothing to multiply by V yet
-        int e = work(0), tv = work(1) & 0x7fffffff, tk = work(2) & 0x7fffffff;
+        // iteration 0: nothing to multiply by V yet.  e0 / e1 / e2: work-list entries of tiles i, i+1, i+2
+        auto clamp_idx = [&](int j) { return j < n_work ? j : n_work - 1; };
+        int e0 = work(0), e1 = work(1), e2 = work(2), e3 = 0;
         __syncthreads();                     // every wavefront is done with K stage 0
-        iteration(S1{}, std::false_type{}, e, tv, tk, 2, 1, sA, sB, pre);
+        iteration(S1{}, std::false_type{}, e0, e1 & 0x7fffffff, e2 & 0x7fffffff, 2, 1, sA, sB, pre, clamp_idx(3), e3);
         int v_rd = 0;                        // (i - 1) % 3
         auto next3 = [](int x) { return x == 2 ? 0 : x + 1; };
         for (int i = 1; i < n_work; i += 2) {
             // odd iteration: K stage 0 is read, K stage 1 refilled
-            e = work(i);
-            tv = work(i + 1) & 0x7fffffff;
-            tk = work(i + 2) & 0x7fffffff;
+            e0 = e1; e1 = e2; e2 = e3;
             __builtin_amdgcn_s_waitcnt(0x0F70);
             __syncthreads();
-            iteration(S0{}, std::true_type{}, e, tv, tk, v_rd, next3(next3(v_rd)), sB, sA, pre);
+            iteration(S0{}, std::true_type{}, e0, e1 & 0x7fffffff, e2 & 0x7fffffff, v_rd, next3(next3(v_rd)), sB, sA, pre,
+                      clamp_idx(i + 3), e3);
             v_rd = next3(v_rd);
             if (i + 1 < n_work) {
-                e = work(i + 1);
-                tv = work(i + 2) & 0x7fffffff;
-                tk = work(i + 3) & 0x7fffffff;
+                e0 = e1; e1 = e2; e2 = e3;
                 __builtin_amdgcn_s_waitcnt(0x0F70);
                 __syncthreads();
-                iteration(S1{}, std::true_type{}, e, tv, tk, v_rd, next3(next3(v_rd)), sA, sB, pre);
+                iteration(S1{}, std::true_type{}, e0, e1 & 0x7fffffff, e2 & 0x7fffffff, v_rd, next3(next3(v_rd)), sA, sB, pre,
+                          clamp_idx(i + 4), e3);
                 v_rd = next3(v_rd);
             }
         }
