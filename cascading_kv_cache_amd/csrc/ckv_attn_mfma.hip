@@ -714,7 +714,7 @@ struct ColsumParams {
     int G;
     int new_mode;
     float scale_log2;
-    int nkb, first_chunk_blk, nbkv, xcd_aware;  // block order, see the kernel
+    int nkb, first_chunk_blk, nbkv, xcd_aware, gsplit;  // block order and head split, see the kernel
 };
 
 constexpr int kQT2 = 64;                      // query rows per LDS tile of the column pass
@@ -736,9 +736,12 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     // diagonal, per-element weights), so they are handed out first and never form the tail of
     // the launch.  Workgroup ids go round the 8 XCDs; when the kv heads divide evenly, every
     // block of one kv head runs on one XCD so that head's query stream stays in that XCD's L2.
-    int bkv_i, kb_i;
+    // A key block is shared out over gsplit workgroups, each taking G / gsplit heads: units small
+    // enough that the last round of workgroups costs little.
+    int bkv_i, kb_i, g_first;
+    const int g_cnt = p.G / p.gsplit;
     {
-        const int nkb = p.nkb, cb0 = p.first_chunk_blk, heavy = nkb - cb0;
+        const int nkb = p.nkb * p.gsplit, cb0 = p.first_chunk_blk * p.gsplit, heavy = nkb - cb0;
         int id = blockIdx.x, nb = p.nbkv, first = 0, stride = 1;
         if (p.xcd_aware) {
             first = id & 7;
@@ -756,6 +759,8 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
             kb_i = id % cb0;
         }
         bkv_i = first + stride * i;
+        g_first = (kb_i % p.gsplit) * g_cnt;
+        kb_i /= p.gsplit;
     }
     const int64_t bkv = bkv_i;
     const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
@@ -790,7 +795,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
         for (int i = tid; i < Q; i += 256) wnew_lds[i] = p.w_new[i];
     }
     const int nmt = (Q - m_first + kQT2 - 1) / kQT2;  // query tiles per head
-    const int n_steps = nmt * p.G;
+    const int n_steps = nmt * g_cnt;
 
     // async copy assignments: the Q tile is 16 blocks of 1 KiB (4 per wavefront); wavefront 0 also
     // brings the tile's 64 normalisers, wavefront 1 its 64 weights (16 lanes x 16 bytes each)
@@ -825,13 +830,9 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
         const unsigned char* q_lds = smem + ST * kCsStage;
         const float* lse_lds = reinterpret_cast<const float*>(q_lds + 16384);
         const float* w_lds = lse_lds + 64;
-
-        // The accumulators start from minus the row normaliser, so the matrix pipe hands back
-        // log2 P directly (the softmax scale is already on the staged queries).
-        // Element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4.
-        f32x16 sacc[2][2];  // [c = query subtile][ks]
-#pragma unroll
-        for (int c = 0; c < 2; c++) {
+        const bool tail = mt + kQT2 > Q;                       // rows past the chunk end
+        const bool diag = chunk_keys && mt <= last_nrel;       // tile may cross the diagonal
+        auto row_init = [&](int c) {
             f32x16 init;
 #pragma unroll
             for (int v4 = 0; v4 < 4; v4++) {
@@ -841,9 +842,63 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
                 init[4 * v4 + 2] = l4.z;
                 init[4 * v4 + 3] = l4.w;
             }
-            sacc[c][0] = init;
-            sacc[c][1] = init;
-        }
+            return init;
+        };
+        if (!tail && !diag && !new_chunk) {
+            // The common case, written in issue order: the logits of the second 32 rows go through
+            // the matrix pipe while the vector ALU turns the first 32 rows into weighted probabilities.
+            // Accumulators start from minus the row normaliser, so the matrix pipe hands back log2 P.
+            f32x16 s0[2], s1[2];
+            s0[0] = s0[1] = row_init(0);
+            uint4 a1[8];
+#pragma unroll
+            for (int kk = 0; kk < 8; kk++) {
+                const uint4 a = *reinterpret_cast<const uint4*>(q_lds + q_off[kk]);
+                s0[0] = Mma<T>::mma(a, kreg[0][kk], s0[0]);
+                s0[1] = Mma<T>::mma(a, kreg[1][kk], s0[1]);
+            }
+            s1[0] = s1[1] = row_init(1);
+#pragma unroll
+            for (int kk = 0; kk < 8; kk++) a1[kk] = *reinterpret_cast<const uint4*>(q_lds + q_off[kk] + 8192);
+            float ws[16];
+#pragma unroll
+            for (int v4 = 0; v4 < 4; v4++) {
+                const float4 w4 = *reinterpret_cast<const float4*>(w_lds + 8 * v4 + 4 * half);
+                ws[4 * v4] = w4.x; ws[4 * v4 + 1] = w4.y; ws[4 * v4 + 2] = w4.z; ws[4 * v4 + 3] = w4.w;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int slot = 0; slot < 16; slot++) {
+                const int kk = slot >> 1, ks = slot & 1;
+                s1[ks] = Mma<T>::mma(a1[kk], kreg[ks][kk], s1[ks]);
+#pragma unroll
+                for (int r = 0; r < 2; r++) {
+                    const int j = 2 * slot + r, ksv = j >> 4, v = j & 15;
+                    const float pe = __builtin_amdgcn_exp2f(s0[ksv][v]);
+                    acc[ksv] = fmaf(ws[v], pe, acc[ksv]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int v4 = 0; v4 < 4; v4++) {
+                const float4 w4 = *reinterpret_cast<const float4*>(w_lds + 32 + 8 * v4 + 4 * half);
+                const float wv[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+#pragma unroll
+                    for (int ks = 0; ks < 2; ks++) {
+                        const float pe = __builtin_amdgcn_exp2f(s1[ks][4 * v4 + e]);
+                        acc[ks] = fmaf(wv[e], pe, acc[ks]);
+                    }
+                }
+            }
+        } else {
+        // The accumulators start from minus the row normaliser, so the matrix pipe hands back
+        // log2 P directly (the softmax scale is already on the staged queries).
+        // Element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4.
+        f32x16 sacc[2][2];  // [c = query subtile][ks]
+#pragma unroll
+        for (int c = 0; c < 2; c++) sacc[c][0] = sacc[c][1] = row_init(c);
 #pragma unroll
         for (int kk = 0; kk < 8; kk++) {
 #pragma unroll
@@ -854,8 +909,6 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
             }
         }
         // element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4, key column of this lane
-        const bool tail = mt + kQT2 > Q;                       // rows past the chunk end
-        const bool diag = chunk_keys && mt <= last_nrel;       // tile may cross the diagonal
         if (!tail && !diag && new_chunk) {
             // every row is later than every key of the block: no masks.  A chunk key takes the
             // weight of its distance m - n and the eager path's roundings; a cached key (only in
@@ -888,24 +941,6 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
                     }
                 }
             }
-        } else if (!tail && !diag && !new_chunk) {
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-#pragma unroll
-                for (int v4 = 0; v4 < 4; v4++) {
-                    const int r0 = 32 * c + 8 * v4 + 4 * half;
-                    const float4 w4 = *reinterpret_cast<const float4*>(w_lds + r0);
-                    const float ws[4] = {w4.x, w4.y, w4.z, w4.w};
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-#pragma unroll
-                        for (int ks = 0; ks < 2; ks++) {
-                            const float pe = __builtin_amdgcn_exp2f(sacc[c][ks][4 * v4 + e]);
-                            acc[ks] = fmaf(ws[e], pe, acc[ks]);
-                        }
-                    }
-                }
-            }
         } else {
 #pragma unroll
             for (int c = 0; c < 2; c++) {
@@ -932,6 +967,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
                 }
             }
         }
+        }  // special cases
         if (mt + kQT2 >= Q) {  // head finished: combine the two lane halves and store
             const int64_t h = kvh * p.G + g;
 #pragma unroll
@@ -945,7 +981,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     };
 
     // two steps per trip: while stage s is consumed the copy of the next step fills stage s^1
-    int g_cur = 0, mt_cur = m_first;          // step being consumed
+    int g_cur = g_first, mt_cur = m_first;    // step being consumed
     auto advance = [&](int& g, int& mt) {
         mt += kQT2;
         if (mt >= Q) {
@@ -953,7 +989,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
             g++;
         }
     };
-    if (n_steps > 0) issue(0, m_first, 0);
+    if (n_steps > 0) issue(g_first, m_first, 0);
     for (int step = 0; step < n_steps; step += 2) {
         int g_n = g_cur, mt_n = mt_cur;
         advance(g_n, mt_n);
@@ -973,7 +1009,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
         }
     }
     if (n_steps == 0) {  // no query can see these keys (only possible for padding blocks)
-        for (int g = 0; g < p.G; g++)
+        for (int g = g_first; g < g_first + g_cnt; g++)
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
                 const int64_t n = key_w + 32 * ks + col;
@@ -1068,7 +1104,8 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         cp.first_chunk_blk = (int)(cp.Nc / 256);
         cp.nbkv = (int)(mp.B * mp.KVH);
         cp.xcd_aware = cp.nbkv % 8 == 0;
-        const dim3 grid((unsigned)(cp.nkb * cp.nbkv));
+        cp.gsplit = G;  // one head per workgroup
+        const dim3 grid((unsigned)(cp.nkb * cp.nbkv * cp.gsplit));
         const int lds = 2 * kCsStage + (int)mp.Q * 4;
         CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(colsum_mfma_kernel<T>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
