@@ -869,10 +869,11 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
 // one workgroup per (b, h): 4 quarters of 128 threads walk every 4th tile, then merge through LDS
 template <typename T>
 __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
-    __shared__ float sh_m[512], sh_l[4], sh_o[4][kD];
+    __shared__ float sh_m[512], sh_l[16];
+    __shared__ float4 sh_o[16][32];
     const ckv_attn_args& a = p.a;
     const int64_t row = blockIdx.x;  // b * H + h
-    const int tid = threadIdx.x, d = tid & 127, qtr = tid >> 7;
+    const int tid = threadIdx.x, d4 = tid & 31, grp = tid >> 5;  // 16 groups of 32 threads, 4 dims per thread
     const float* ml = p.part_ml + row * p.tiles * 2;
     float M = -INFINITY;
     for (int t = tid; t < p.tiles; t += 512) M = fmaxf(M, ml[2 * t]);
@@ -883,23 +884,37 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
         __syncthreads();
     }
     M = sh_m[0];
-    float L = 0.f, o = 0.f;
-    for (int t = qtr; t < p.tiles; t += 4) {
+    // every tile's partial is written by the main kernel (zeros when the tile is hidden), so the
+    // loop needs no branch and its loads can all be in flight together
+    float L = 0.f;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4* po = reinterpret_cast<const float4*>(p.part_o + row * p.tiles * kD) + d4;
+#pragma unroll 4
+    for (int t = grp; t < p.tiles; t += 16) {
         const float m = ml[2 * t];
-        if (m == -INFINITY) continue;
-        const float sc = __builtin_amdgcn_exp2f(m - M);
+        const float sc = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - M);
+        const float4 v = po[(int64_t)t * (kD / 4)];
         L = fmaf(ml[2 * t + 1], sc, L);
-        o = fmaf(p.part_o[(row * p.tiles + t) * kD + d], sc, o);
+        o.x = fmaf(v.x, sc, o.x);
+        o.y = fmaf(v.y, sc, o.y);
+        o.z = fmaf(v.z, sc, o.z);
+        o.w = fmaf(v.w, sc, o.w);
     }
-    sh_o[qtr][d] = o;
-    if (d == 0) sh_l[qtr] = L;
+    sh_o[grp][d4] = o;
+    if (d4 == 0) sh_l[grp] = L;
     __syncthreads();
-    if (qtr != 0) return;
-    o = sh_o[0][d] + sh_o[1][d] + sh_o[2][d] + sh_o[3][d];
-    L = sh_l[0] + sh_l[1] + sh_l[2] + sh_l[3];
+    if (tid >= kD) return;
+    const int d = tid;
+    float od = 0.f;
+    L = 0.f;
+#pragma unroll
+    for (int g = 0; g < 16; g++) {
+        od += reinterpret_cast<const float*>(&sh_o[g][0])[d];
+        L += sh_l[g];
+    }
     const int64_t b = row / a.H, h = row % a.H;
     T* out = (T*)a.out + b * a.out_stride[0] + h * a.out_stride[1];
-    out[d * a.out_stride[3]] = Elem<T>::from_float(o / L);
+    out[d * a.out_stride[3]] = Elem<T>::from_float(od / L);
     if (d == 0) {
         const float l2 = M + __builtin_amdgcn_logf(L);
         p.lse2[row] = l2;
