@@ -237,8 +237,15 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
             const int64_t seg = st_l[i] < W ? st_l[i] : W;
             if (seg <= 0) break;
             const int64_t sx = sx_l[i];
-            for (int64_t j = tid; j < W; j += T) {
-                pos[((int64_t)i * W + j) * A.pos_stride[2]] = ((j + seg - sx) % seg) + ub - seg;
+            if (W < (1ll << 30)) {  // the usual case: 32-bit arithmetic, a 64-bit modulo per slot costs far more
+                const uint32_t seg32 = (uint32_t)seg, add32 = (uint32_t)(seg - sx);
+                for (int64_t j = tid; j < W; j += T) {
+                    pos[((int64_t)i * W + j) * A.pos_stride[2]] = (int64_t)(((uint32_t)j + add32) % seg32) + ub - seg;
+                }
+            } else {
+                for (int64_t j = tid; j < W; j += T) {
+                    pos[((int64_t)i * W + j) * A.pos_stride[2]] = ((j + seg - sx) % seg) + ub - seg;
+                }
             }
             ub -= W;
             if (ub <= 0) break;
@@ -518,7 +525,8 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
         p.k_sub = ksub;
         p.do_pos = (off + ksub == A.K) ? 1 : 0;
         // small calls still rewrite max_seq_len position ids per (n, h): keep enough lanes for that
-        const int T = ksub <= 256 ? 256 : 1024;
+        // few tokens: a small block plans them, unless the position pass has many slots to rewrite
+        const int T = (ksub <= 256 && A.max_seq_len < 8192) ? 256 : 1024;
         const size_t lds = plan_lds_bytes(ksub);
         if (lds > 48 * 1024) {
             CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(ckv_update_plan_kernel),
