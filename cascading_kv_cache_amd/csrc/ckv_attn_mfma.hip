@@ -5,14 +5,17 @@
 //                tiles Vt[tile][d][key'] (key' = the order the PV MFMA consumes), build one 64-bit
 //                visibility word per key tile.  cos/sin are computed once per key and reused for
 //                every (batch, kv-head) that shares the position row.
-//   stage_q      rotate Q.
-//   fwd          flash forward.  One workgroup = one kv head x 256 (head, position) rows, so the G
-//                query heads of a group share every K/V tile staged in LDS.  S^T = K Q^T keeps a
-//                query in one lane pair: the row max / sum need a single cross-half exchange and
-//                exp(S^T) is already laid out as the B operand of O^T += V^T P^T.
-//   colsum       exact score sums.  One workgroup = one kv head x 256 keys held in registers;
-//                the queries stream through LDS, P = exp(S - lse) with the final normaliser, and
-//                the weighted column sums stay inside a lane (S = Q K^T orientation).
+//   stage_q      rotate Q and fold the softmax scale (times log2 e) in.
+//   fwd          flash forward, software pipelined.  One workgroup = one kv head x 256 (head,
+//                position) rows, so the G query heads of a group share every K/V tile staged in
+//                LDS.  S^T = K Q^T keeps a query in one lane pair: the row max / sum need a single
+//                cross-half exchange and exp2(S^T) is already laid out as the B operand of
+//                O^T += V^T P^T.  The softmax of tile i runs beside the logits of tile i+1 and the
+//                P.V product of tile i-1.
+//   colsum       exact score sums.  One workgroup = one head x 256 keys held in registers; the
+//                queries stream through LDS, the accumulators start from minus the final
+//                normaliser so the matrix pipe returns log2 P, and the weighted column sums stay
+//                inside a lane (S = Q K^T orientation).
 #include "ckv_attn_internal.h"
 
 #include <type_traits>
