@@ -194,6 +194,8 @@ def lib():
         L.ckv_attn_dense.restype = C.c_int
         L.ckv_dense_workspace_bytes.argtypes = [I64, I64, I64, I64, I64, C.c_int32]
         L.ckv_dense_workspace_bytes.restype = I64
+        L.ckv_chunk_positions.argtypes = [C.c_void_p, I64, I64, C.c_void_p, I64, I64, C.c_void_p, C.c_void_p]
+        L.ckv_chunk_positions.restype = C.c_int
         L.ckv_profile_enable.argtypes = [C.c_int]
         L.ckv_profile_enable.restype = C.c_int
         L.ckv_profile_read.argtypes = [C.POINTER(C.c_double), C.POINTER(I64)]
@@ -209,8 +211,9 @@ def lib():
 STAGES = ("prep", "fwd", "scores", "finish", "decode", "decode_tail", "plan", "apply")
 
 
-def profile_enable(on: bool) -> bool:
-    return bool(lib().ckv_profile_enable(int(on)))
+def profile_enable(on) -> int:
+    """0 / False: off; 1 / True: every stage; 2: only the attention main kernels.  Returns the previous level."""
+    return int(lib().ckv_profile_enable(int(on)))
 
 
 def profile_read():

@@ -27,18 +27,29 @@ def default_inv_freq(head_dim: int, theta: float, device) -> torch.Tensor:
 def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_pos: bool = False) -> torch.Tensor:
     """Position ids of the incoming chunk (cascade_attention.py:119-150) without a host sync:
     0.. on the first call, otherwise one past the largest id among sinks and cache slots
-    (stale and masked entries included, as in the reference)."""
+    (stale and masked entries included, as in the reference).  One small kernel of the library."""
+    _require_device(cache.key_cache[layer_idx], "the cache")
     dev = cache.key_cache[layer_idx].device
-    ar = torch.arange(q_len, device=dev, dtype=torch.long)
-    if cache._seen_host[layer_idx] == 0:
-        return ar
-    if do_og_pos:
-        key_max = cache.og_pos[layer_idx].amax()
-    else:
-        key_max = cache.pos[layer_idx][0, 0].amax() + cache.pos_shift(layer_idx)
-    if cache.num_sink_tokens > 0:
-        key_max = torch.maximum(key_max, cache.sink_pos[layer_idx][0, 0].amax())
-    return ar + (key_max + 1)
+    out = torch.empty(q_len, device=dev, dtype=torch.long)
+    key_ptr, n_key, shift, sink_ptr, n_sink = None, 0, 0, None, 0
+    if cache._seen_host[layer_idx] != 0:
+        if do_og_pos:
+            og = cache.og_pos[layer_idx]
+            assert og.is_contiguous()
+            key_ptr, n_key = og.data_ptr(), og.numel()
+        else:
+            row = cache.pos[layer_idx][0, 0]
+            assert row.is_contiguous()
+            key_ptr, n_key, shift = row.data_ptr(), row.numel(), int(cache.pos_shift(layer_idx))
+        if cache.num_sink_tokens > 0:
+            srow = cache.sink_pos[layer_idx][0, 0]
+            assert srow.is_contiguous()
+            sink_ptr, n_sink = srow.data_ptr(), srow.numel()
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        _abi.check(_abi.lib().ckv_chunk_positions(key_ptr, n_key, shift, sink_ptr, n_sink, q_len, out.data_ptr(), stream),
+                   "ckv_chunk_positions")
+    return out
 
 
 def cascade_attention(query_states, key_states, value_states, cache: CascadingKVCache, layer_idx: int,

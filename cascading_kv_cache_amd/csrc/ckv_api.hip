@@ -1,6 +1,7 @@
 // Entry points of libckv that are not tied to one kernel family.
 #include "ckv_common.h"
 
+#include <cstdint>
 #include <vector>
 
 namespace ckv {
@@ -9,13 +10,17 @@ struct Span {
     int stage;
     hipEvent_t t0, t1;
 };
-bool g_prof_on = false;
+int g_prof_level = 0;  // 0 off, 1 every stage, 2 attention main kernels only
 std::vector<Span> g_spans;
 hipEvent_t g_open[CKV_STAGE_COUNT];
 }  // namespace
 
+static bool prof_wanted(int stage) {
+    return g_prof_level == 1 || (g_prof_level == 2 && (stage == CKV_STAGE_FWD || stage == CKV_STAGE_DECODE));
+}
+
 void prof_begin(int stage, hipStream_t stream) {
-    if (!g_prof_on) return;
+    if (!prof_wanted(stage)) return;
     hipEvent_t e;
     if (hipEventCreate(&e) != hipSuccess) return;
     (void)hipEventRecord(e, stream);
@@ -23,7 +28,7 @@ void prof_begin(int stage, hipStream_t stream) {
 }
 
 void prof_end(int stage, hipStream_t stream) {
-    if (!g_prof_on || !g_open[stage]) return;
+    if (!g_open[stage]) return;
     hipEvent_t e;
     if (hipEventCreate(&e) != hipSuccess) return;
     (void)hipEventRecord(e, stream);
@@ -33,8 +38,8 @@ void prof_end(int stage, hipStream_t stream) {
 }  // namespace ckv
 
 extern "C" int ckv_profile_enable(int on) {
-    const int prev = ckv::g_prof_on ? 1 : 0;
-    ckv::g_prof_on = on != 0;
+    const int prev = ckv::g_prof_level;
+    ckv::g_prof_level = on < 0 || on > 2 ? 1 : on;
     return prev;
 }
 
@@ -50,6 +55,50 @@ extern "C" int ckv_profile_read(double* ms, int64_t* launches) {
         (void)hipEventDestroy(s.t1);
     }
     ckv::g_spans.clear();
+    return CKV_OK;
+}
+
+namespace ckv {
+namespace {
+__global__ void __launch_bounds__(1024) chunk_positions_kernel(const int64_t* key_pos, int64_t n_key, int64_t key_shift,
+                                                               const int64_t* sink_pos, int64_t n_sink, int64_t q_len,
+                                                               int64_t* q_pos) {
+    __shared__ int64_t red[1024];
+    const int tid = threadIdx.x;
+    int64_t base = 0;
+    if (key_pos || sink_pos) {
+        int64_t m = INT64_MIN;
+        for (int64_t i = tid; i < n_key; i += 1024) {
+            const int64_t v = key_pos[i] + key_shift;
+            m = v > m ? v : m;
+        }
+        for (int64_t i = tid; i < n_sink; i += 1024) {
+            const int64_t v = sink_pos[i];
+            m = v > m ? v : m;
+        }
+        red[tid] = m;
+        __syncthreads();
+        for (int off = 512; off > 0; off >>= 1) {
+            if (tid < off) red[tid] = red[tid + off] > red[tid] ? red[tid + off] : red[tid];
+            __syncthreads();
+        }
+        base = red[0] + 1;
+    }
+    for (int64_t i = tid; i < q_len; i += 1024) q_pos[i] = base + i;
+}
+}  // namespace
+}  // namespace ckv
+
+extern "C" int ckv_chunk_positions(const int64_t* key_pos, int64_t n_key, int64_t key_shift, const int64_t* sink_pos,
+                                   int64_t n_sink, int64_t q_len, int64_t* q_pos, void* stream_) {
+    if (!q_pos) return CKV_ERR_NULL;
+    if (q_len <= 0 || n_key < 0 || n_sink < 0) return CKV_ERR_SHAPE;
+    if (n_key == 0) key_pos = nullptr;
+    if (n_sink == 0) sink_pos = nullptr;
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    hipLaunchKernelGGL(ckv::chunk_positions_kernel, dim3(1), dim3(1024), 0, stream, key_pos, key_pos ? n_key : 0, key_shift,
+                       sink_pos, sink_pos ? n_sink : 0, q_len, q_pos);
+    CKV_HIP_TRY(hipGetLastError());
     return CKV_OK;
 }
 

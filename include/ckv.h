@@ -221,6 +221,17 @@ int64_t ckv_dense_workspace_bytes(int64_t B, int64_t H, int64_t n_ctx, int64_t n
 int ckv_attn_dense(const ckv_dense_args* args, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Position ids of an incoming chunk (cascade_attention.py:114-150): q_pos[i] = i on the first call
+ * of a sequence (key_pos and sink_pos NULL), otherwise i + 1 + max(max(key_pos[0..n_key)) + key_shift,
+ * max(sink_pos[0..n_sink))) - stale and masked entries included, as in the reference.  One small
+ * kernel on `stream`, no host synchronisation (the reference reads the maxima back to the host).
+ * key_pos is the cache's position row (or its og_pos tensor with key_shift 0); either array may be
+ * NULL / empty.
+ * ---------------------------------------------------------------------------------------- */
+int ckv_chunk_positions(const int64_t* key_pos, int64_t n_key, int64_t key_shift, const int64_t* sink_pos,
+                        int64_t n_sink, int64_t q_len, int64_t* q_pos, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Stage timing (the reference's BENCHMARK=True switch, cascading_cache.py:986-1026, extended to
  * every kernel stage).  While enabled, each stage of ckv_attn / ckv_update is bracketed by HIP
  * events on the caller's stream; ckv_profile_read waits for them, ADDS the elapsed milliseconds
@@ -239,6 +250,8 @@ typedef enum ckv_stage {
     CKV_STAGE_COUNT = 8
 } ckv_stage;
 
+/* on: 0 = off, 1 = every stage, 2 = only the attention main kernels (CKV_STAGE_FWD, CKV_STAGE_DECODE):
+ * two event records per call instead of a dozen, for timing inside a throughput measurement */
 int ckv_profile_enable(int on);                       /* returns the previous setting */
 int ckv_profile_read(double* ms, int64_t* launches);  /* both arrays CKV_STAGE_COUNT long */
 

@@ -32,7 +32,7 @@ def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for must in ("ckv_update", "ckv_update_workspace_bytes", "ckv_attn", "ckv_attn_workspace_bytes", "ckv_attn_dense",
                  "ckv_dense_workspace_bytes", "ckv_strerror", "ckv_abi_version", "ckv_profile_enable",
-                 "ckv_profile_read"):
+                 "ckv_profile_read", "ckv_chunk_positions"):
         assert must in names
 
 
@@ -99,6 +99,8 @@ def test_attention_argument_validation_needs_no_gpu(lib):
     a.head_reduction = 0
     assert lib.ckv_attn(C.byref(a), None) == -1  # q / k_new / ... missing
     assert lib.ckv_attn_dense(None, None) == -1
+    assert lib.ckv_chunk_positions(None, 0, 0, None, 0, 4, None, None) == -1   # no output
+    assert lib.ckv_chunk_positions(None, 0, 0, None, 0, 0, 8, None) == -2      # empty chunk (checked before any launch)
     d = _abi.DenseArgs()
     d.dtype = _abi.CKV_F16
     d.B, d.H, d.n_ctx, d.n_kv, d.D = 1, 1, 16, 8, 64

@@ -215,6 +215,29 @@ def test_decode_streaming_many_items(H, KVH, dtype, fill):
             assert torch.equal(getattr(gpu, name)[0].cpu(), getattr(cpu, name)), f"step {step}: {name}"
 
 
+@pytest.mark.parametrize("do_og_pos", [False, True])
+def test_chunk_positions_kernel(do_og_pos):
+    """ckv_chunk_positions against the rule of cascade_attention.py:114-150: 0.. on the first call,
+    then one past the largest position id among sinks and slots (stale entries included)."""
+    from cascading_kv_cache_amd.cascade_attention import chunk_positions
+
+    B, KVH, D, NS, W, C = 2, 2, 32, 4, 16, 4
+    gpu, cpu = make_pair(B, KVH, D, NS, W, C, torch.float32)
+    gen = torch.Generator().manual_seed(3)
+    assert torch.equal(chunk_positions(gpu, 0, 7, do_og_pos).cpu(), torch.arange(7))
+    for n in (3, 9, 40, 1, 100):
+        k = torch.randn(B, KVH, n, D, generator=gen)
+        cpu.update(k, k.clone(), torch.rand(B, KVH, n, generator=gen))
+        push_state(gpu, cpu)
+        if do_og_pos:
+            key_max = cpu.og_pos.amax()
+        else:
+            shift = NS if int(cpu.seen_tokens) > NS else 0
+            key_max = cpu.pos[0, 0].amax() + shift
+        want = torch.arange(5) + max(int(key_max), int(cpu.sink_pos[0, 0].amax())) + 1
+        assert torch.equal(chunk_positions(gpu, 0, 5, do_og_pos).cpu(), want)
+
+
 def dense_reference(q, k, v, mask, sm_scale):
     n_ctx, n_kv = q.size(2), k.size(2)
     logits = torch.matmul(q.float(), k.float().transpose(2, 3)) * sm_scale

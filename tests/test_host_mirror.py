@@ -90,16 +90,12 @@ def test_acceptance_schedules_agree_with_the_oracle_tables():
             assert acceptance_periods(name, c) == oracle_periods(name, c), (name, c)
 
 
-def test_chunk_positions_follow_the_largest_id():
-    """cascade/models/cascade_attention.py:119-150."""
+def test_chunk_positions_need_the_device():
+    """cascade/models/cascade_attention.py:119-150 is one kernel of the library (checked against the rule on
+    the GPU, tests/test_gpu_attention.py): on host tensors it refuses, like every other entry point."""
     c = make()
-    assert chunk_positions(c, 0, 3).tolist() == [0, 1, 2]
-    c._seen_host[0] = 20
-    c.pos[0][0, 0, :] = torch.arange(16)
-    c.sink_pos[0][0, 0, :] = torch.tensor([0, 1])
-    assert chunk_positions(c, 0, 2).tolist() == [18, 19]  # 15 + sink shift 2 + 1
-    c.og_pos[0][1, 2, 5] = 99
-    assert chunk_positions(c, 0, 2, do_og_pos=True).tolist() == [100, 101]
+    with pytest.raises(_abi.CkvError):
+        chunk_positions(c, 0, 3)
 
 
 def test_no_cpu_fallback_anywhere():
