@@ -949,8 +949,8 @@ __device__ inline float reduce_group(const float* v, int n, int mode) {
 
 // one thread per (b, kvh, key): P of the G (or all H) heads, dtype rounding like the eager path
 // (cascade_attention.py:319-323 with a single query row), head reduction, EMA / new-token score
-template <typename T, int G>
-__global__ void decode_scores_kernel(DecodeParams p, float w_one, float beta_pow) {
+template <typename T, int G, bool HOMO>
+__global__ void __launch_bounds__(256) decode_scores_kernel(DecodeParams p, float w_one, float beta_pow) {
     const ckv_attn_args& a = p.a;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t per = a.S + 1;
@@ -958,9 +958,10 @@ __global__ void decode_scores_kernel(DecodeParams p, float w_one, float beta_pow
     const int64_t i = idx % per, kvh = (idx / per) % a.KVH, b = idx / (per * a.KVH);
     const int64_t n = a.num_sink + i;
     const bool is_new = i == a.S;
-    float vals[128];
+    // per kv head the G values stay in registers; only the all-heads reduction needs the long array
+    float vals[HOMO ? 128 : G];
     int cnt = 0;
-    const int64_t kv0 = a.homogeneous_heads ? 0 : kvh, kv1 = a.homogeneous_heads ? a.KVH : kvh + 1;
+    const int64_t kv0 = HOMO ? 0 : kvh, kv1 = HOMO ? a.KVH : kvh + 1;
     for (int64_t kv = kv0; kv < kv1; kv++) {
         const float* lg = p.logits + ((b * a.KVH + kv) * p.N + n) * G;
 #pragma unroll
@@ -970,7 +971,31 @@ __global__ void decode_scores_kernel(DecodeParams p, float w_one, float beta_pow
             vals[cnt++] = round_t<T>(__fmul_rn(pt, is_new ? round_t<T>(w_one) : w_one));
         }
     }
-    const float red = reduce_group<T, G>(vals, cnt, a.head_reduction);
+    float red;
+    if (HOMO) {
+        red = reduce_group<T, G>(vals, cnt, a.head_reduction);
+    } else if (a.head_reduction == CKV_REDUCE_MAX) {
+        red = vals[0];
+#pragma unroll
+        for (int g = 1; g < G; g++) red = fmaxf(red, vals[g]);
+    } else if (a.head_reduction == CKV_REDUCE_MEAN) {
+        red = 0.f;
+#pragma unroll
+        for (int g = 0; g < G; g++) red = __fadd_rn(red, vals[g]);
+        red = round_t<T>(red / (float)G);
+    } else {  // lower median: rank by counting, no indexed array
+        red = vals[0];
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            int below = 0, equal = 0;
+#pragma unroll
+            for (int h = 0; h < G; h++) {
+                below += vals[h] < vals[g];
+                equal += vals[h] == vals[g];
+            }
+            if (below <= (G - 1) / 2 && (G - 1) / 2 < below + equal) red = vals[g];
+        }
+    }
     if (is_new) {
         if (a.new_scores)
             *((T*)a.new_scores + b * a.new_scores_stride[0] + kvh * a.new_scores_stride[1]) = Elem<T>::from_float(red);
@@ -1036,8 +1061,12 @@ int run_decode(const DecodeParams& p, hipStream_t stream) {
             // built in the tensor dtype (cascade_attention.py:270-276)
             const float w_one = (float)(1.0 - a.beta);
             const int64_t items = a.B * a.KVH * (a.S + 1);
-            hipLaunchKernelGGL((decode_scores_kernel<T, G>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0, stream,
-                               p, w_one, (float)a.beta);
+            if (a.homogeneous_heads)
+                hipLaunchKernelGGL((decode_scores_kernel<T, G, true>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
+                                   stream, p, w_one, (float)a.beta);
+            else
+                hipLaunchKernelGGL((decode_scores_kernel<T, G, false>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
+                                   stream, p, w_one, (float)a.beta);
             CKV_HIP_TRY(hipGetLastError());
         }
     }

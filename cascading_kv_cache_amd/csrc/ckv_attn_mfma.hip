@@ -246,8 +246,8 @@ struct StageQParams {
 // thread = (position m, quarter of the rotation pairs); the cos/sin of the position are computed once
 // and reused for the batch x head rows of the block's share (blockIdx.y of gridDim.y)
 template <typename T>
-__global__ void __launch_bounds__(256) stage_q_kernel(StageQParams p) {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+__global__ void __launch_bounds__(64) stage_q_kernel(StageQParams p) {
+    const int64_t idx = (int64_t)blockIdx.x * 64 + threadIdx.x;
     const int64_t m = idx >> 2;
     const int quarter = idx & 3;
     if (m >= p.Q) return;
@@ -1066,11 +1066,12 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
                  mp.q_stride[1] % 8 == 0 && mp.q_stride[2] % 8 == 0;
         {
             // enough blocks to fill the chip; the rest of batch x heads is looped over inside, sharing cos/sin
-            const int64_t bx = (mp.Q * 4 + 255) / 256, nbh_q = mp.B * mp.H;
-            int64_t by = (1024 + bx - 1) / bx;
+            // one wavefront per block; about 2048 blocks, the rest of batch x heads looped over inside
+            const int64_t bx = (mp.Q * 4 + 63) / 64, nbh_q = mp.B * mp.H;
+            int64_t by = (2048 + bx - 1) / bx;
             if (by > nbh_q) by = nbh_q;
             if (by < 1) by = 1;
-            hipLaunchKernelGGL(stage_q_kernel<T>, dim3((unsigned)bx, (unsigned)by), dim3(256), 0, stream, sq);
+            hipLaunchKernelGGL(stage_q_kernel<T>, dim3((unsigned)bx, (unsigned)by), dim3(64), 0, stream, sq);
         }
         CKV_HIP_TRY(hipGetLastError());
     }
