@@ -245,7 +245,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU mode (every (batch, kv-head) unit is "
-              "independent; see DESIGN.md for how it would shard). Run with --gpus 1.", file=sys.stderr)
+              "independent, so it would shard by kv head with no exchange except a per-key score reduction). Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py needs a HIP device", file=sys.stderr)

@@ -89,7 +89,7 @@ def run_teacher_forced(B, H, KVH, D, NS, W, C, Q, chunks, dtype, seed, reduction
 
 
 def test_config1_float32_stream():
-    """BASELINE config 1: B=1, 32q/8kv heads, D=128, sink 4, window 512 in C=4, 4096 tokens in
+    """The float32 benchmark case: B=1, 32q/8kv heads, D=128, sink 4, window 512 in C=4, 4096 tokens in
     chunks of 256, theta 5e5, float32."""
     flips, compared = run_teacher_forced(1, 32, 8, 128, 4, 128, 4, 256, 16, torch.float32, seed=1)
     assert flips == 0, f"{flips} of {compared} slots differ in og_pos (eviction decisions flipped)"
