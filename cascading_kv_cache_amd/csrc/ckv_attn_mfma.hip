@@ -315,6 +315,7 @@ struct FwdParams {
     int64_t B, H, KVH, Q, N, Nc, n_pad;
     int G, QT;        // heads per kv head, positions per workgroup (G * QT <= 256)
     float scale_log2; // softmax scale * log2(e)
+    int n_qt, xcd_aware;  // query tiles per kv head; 1-D XCD-aware block order
 };
 
 __device__ inline const void* uniform_ptr(const void* p) {
@@ -375,9 +376,18 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, half = lane >> 5;
-    const int64_t bkv = blockIdx.y;
+    int bkv_i = blockIdx.y, qt_i = blockIdx.x;
+    // With 8 | B * KVH the grid is 1-D: workgroup ids go round the 8 XCDs, and all query tiles of a kv
+    // head are put on one XCD, so its K / V^T stream is fetched from HBM into one L2 instead of eight
+    // (same run time, a fifth of the HBM reads).
+    if (p.xcd_aware) {
+        const int id = blockIdx.x, jq = id >> 3;
+        bkv_i = (id & 7) + 8 * (jq / p.n_qt);
+        qt_i = jq % p.n_qt;
+    }
+    const int64_t bkv = bkv_i;
     const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
-    const int m0 = (int)blockIdx.x * p.QT;
+    const int m0 = qt_i * p.QT;
 
     int m_hi = m0 + p.QT - 1;
     if (m_hi > (int)p.Q - 1) m_hi = (int)p.Q - 1;
@@ -491,17 +501,27 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
             }
         }
     };
+    // One 64-bit word per lane says which keys of the tile its query row may see (visible slot and not
+    // later than the row); it is shifted once so that the bit of every element sits at a compile-time
+    // position.  Few live values: this path must not push the loop's registers into scratch.
     auto mask_tile = [&](int entry, f32x16(&s)[2]) {
         const int t = entry & 0x7fffffff;
-        const unsigned long long vis = vis_lds[t];
-        const int key0 = t * kBN;
+        unsigned long long allowed = vis_lds[t];
+        const int limit = row_m - (t * kBN - (int)p.Nc);  // last key index of the tile the row may see, if it is a chunk tile
+        if (t * kBN + kBN - 1 >= (int)p.Nc) {             // the tile holds chunk keys
+            const int first_chunk = (int)p.Nc - t * kBN;  // <= 0 when the whole tile is chunk
+            unsigned long long causal = limit >= 63 ? ~0ull : (limit < 0 ? 0ull : ((2ull << limit) - 1ull));
+            if (first_chunk > 0) causal |= (1ull << first_chunk) - 1ull;  // cached keys in front of the chunk: always allowed
+            allowed &= causal;
+        }
+        allowed >>= 4 * half;
+        const uint32_t lo = (uint32_t)allowed, hi = (uint32_t)(allowed >> 32);
 #pragma unroll
         for (int ks = 0; ks < 2; ks++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int kidx = 32 * ks + 8 * (v >> 2) + 4 * half + (v & 3);
-                const int nrel = key0 - (int)p.Nc + kidx;  // >= 0: key of the chunk
-                const bool ok = ((vis >> kidx) & 1ull) && (nrel < 0 || nrel <= row_m);
+                const int bit = 8 * (v >> 2) + (v & 3);  // key 32 ks + bit + 4 half
+                const bool ok = ((ks ? hi : lo) >> bit) & 1u;
                 s[ks][v] = ok ? s[ks][v] : -INFINITY;
             }
     };
@@ -675,25 +695,53 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     const int g_row = (wave * 32 + col) / p.QT;
     const int64_t row_h = kvh * p.G + g_row;
-    if (g_row < p.G && row_m < p.Q) {
-        const float inv = 1.f / l_tot;
+    const bool row_ok = g_row < p.G && row_m < p.Q;
+    const float inv = 1.f / l_tot;
+    const bool rows16 = p.out_stride[3] == 1 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0 && p.out_stride[0] % 8 == 0 &&
+                        p.out_stride[1] % 8 == 0 && p.out_stride[2] % 8 == 0;
+    if (rows16) {
+        // through LDS, so that a row leaves as 16-byte pieces of 16 neighbouring lanes (a lane's own
+        // 8-byte pieces would reach memory as partly filled 32-byte sectors)
+        constexpr int kRowPitch = 256 + 16;  // bytes; the pad spreads the banks
+        __syncthreads();                      // the tile stages are no longer read
+        unsigned char* ow = smem + wave * (32 * kRowPitch);
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+#pragma unroll
+            for (int v4 = 0; v4 < 4; v4++) {
+                uint2 w;
+                w.x = Mma<T>::pack2(oacc[dt][4 * v4] * inv, oacc[dt][4 * v4 + 1] * inv);
+                w.y = Mma<T>::pack2(oacc[dt][4 * v4 + 2] * inv, oacc[dt][4 * v4 + 3] * inv);
+                *reinterpret_cast<uint2*>(ow + col * kRowPitch + (32 * dt + 8 * v4 + 4 * half) * (int)sizeof(T)) = w;
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_wave_barrier();
+        // 4 rows per pass: lane = (row in the pass, 16-byte piece)
+#pragma unroll
+        for (int pass = 0; pass < 8; pass++) {
+            const int r = 4 * pass + (lane >> 4), piece = lane & 15;
+            const int rr = wave * 32 + r;
+            const int g_r = rr / p.QT, m_r = m0 + rr % p.QT;
+            if (g_r < p.G && m_r < p.Q) {
+                const uint4 v = *reinterpret_cast<const uint4*>(ow + r * kRowPitch + piece * 16);
+                T* dst = (T*)p.out + b * p.out_stride[0] + (kvh * p.G + g_r) * p.out_stride[1] + m_r * p.out_stride[2];
+                *reinterpret_cast<uint4*>(dst + piece * 8) = v;
+            }
+        }
+    } else if (row_ok) {
         T* orow = (T*)p.out + b * p.out_stride[0] + row_h * p.out_stride[1] + row_m * p.out_stride[2];
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) {
 #pragma unroll
             for (int v4 = 0; v4 < 4; v4++) {
                 const int d = 32 * dt + 8 * v4 + 4 * half;
-                if (p.out_stride[3] == 1) {
-                    uint2 w;
-                    w.x = Mma<T>::pack2(oacc[dt][4 * v4] * inv, oacc[dt][4 * v4 + 1] * inv);
-                    w.y = Mma<T>::pack2(oacc[dt][4 * v4 + 2] * inv, oacc[dt][4 * v4 + 3] * inv);
-                    *reinterpret_cast<uint2*>(orow + d) = w;
-                } else {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) orow[(d + e) * p.out_stride[3]] = Elem<T>::from_float(oacc[dt][4 * v4 + e] * inv);
-                }
+                for (int e = 0; e < 4; e++) orow[(d + e) * p.out_stride[3]] = Elem<T>::from_float(oacc[dt][4 * v4 + e] * inv);
             }
         }
+    }
+    if (row_ok) {
         if (half == 0) {
             const float l2 = m_run + __builtin_amdgcn_logf(l_tot);  // v_log_f32 is log2
             p.lse[(b * p.H + row_h) * p.Q + row_m] = l2 * 0.6931471805599453f;
@@ -1092,7 +1140,10 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         const int lds = pipe_lds_bytes(n_pad);
         CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fwd_pipe_kernel<T>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        hipLaunchKernelGGL(fwd_pipe_kernel<T>, grid, dim3(512), lds, stream, fp);
+        fp.n_qt = (int)grid.x;
+        fp.xcd_aware = grid.y % 8 == 0;
+        if (fp.xcd_aware) hipLaunchKernelGGL(fwd_pipe_kernel<T>, dim3(grid.x * grid.y), dim3(512), lds, stream, fp);
+        else hipLaunchKernelGGL(fwd_pipe_kernel<T>, grid, dim3(512), lds, stream, fp);
         CKV_HIP_TRY(hipGetLastError());
     }
     if (mp.colsum) {
