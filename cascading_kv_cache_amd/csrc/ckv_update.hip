@@ -125,12 +125,24 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
     __syncthreads();
     if (tid == 0 && n_sink_new > 0) *g_sinks = sinks0 + n_sink_new;
 
+    // 64-bit division per arrival is what this kernel would spend its time on: token indices, periods
+    // and the window fit 32 bits in every realistic call, and both divisors are usually powers of two
+    const bool small = seen + cap + S + NS < (1ll << 31) && W < (1ll << 31);
+    const bool w_pow2 = (W & (W - 1)) == 0;
+    auto mod_w = [&](int64_t x) -> int {  // x >= 0
+        if (w_pow2) return (int)(x & (W - 1));
+        if (small) return (int)((uint32_t)x % (uint32_t)W);
+        return (int)(x % W);
+    };
+
     int nA = cap - n_sink_new;
     int cur = 0;
     for (int i = 0; i < C && nA > 0; i++) {
         const int64_t l = (int64_t)i * W;
         const int stored0 = st_l[i], start0 = sx_l[i];
         const int64_t per = A.do_cache_every_n[i];
+        const bool per_small = small && per > 0 && per < (1ll << 31);
+        const bool per_pow2 = per > 0 && (per & (per - 1)) == 0;
         const int32_t* Asrc = a_src[cur];
         const int32_t* Atrig = a_trig[cur];
         const float* Ascore = a_score[cur];
@@ -143,7 +155,10 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
             bool f = false;
             if (a < nA) {
                 const int64_t gidx = seen + Atrig[a];  // 0-based global index of the triggering token
-                const bool acc = (A.eager_fill && gidx <= S + NS) || (((gidx - NS) % per) == 0);
+                const int64_t rel = gidx - NS;  // >= 0: sink tokens never arrive here
+                const bool on_period = per_pow2 ? (rel & (per - 1)) == 0
+                                                : (per_small ? ((uint32_t)rel % (uint32_t)per) == 0 : (rel % per) == 0);
+                const bool acc = (A.eager_fill && gidx <= S + NS) || on_period;
                 f = acc || (stored0 == 0 && a == 0);
             }
             int ex;
@@ -194,7 +209,7 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
                 int ns;
                 float nv;
                 if (mv < stored0 - 1) {     // an old ring entry nobody touched in this call
-                    ns = (int)l + (int)((start0 + (int64_t)mv) % W);
+                    ns = (int)l + mod_w(start0 + (int64_t)mv);
                     nv = load_as_float(A.cache_s, cs_base + (int64_t)ns * A.cache_s_stride[2], A.dtype);
                 } else {
                     ns = w_src[mv - stored0 + 1];
@@ -205,7 +220,7 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
                 Btrig[mv] = Atrig[a];
             }
             if (e >= E - (int)W) {  // not evicted again before the call ends
-                const int phys = (int)l + (int)(((int64_t)start0 + stored0 + e) % W);
+                const int phys = (int)l + mod_w((int64_t)start0 + stored0 + e);
                 emit_move(first, next_of, phys, w_src[e + 1]);
             }
         }
@@ -216,7 +231,7 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
         __syncthreads();
         if (tid == 0) {
             const int st_new = stored0 + E < (int)W ? stored0 + E : (int)W;
-            const int sx_new = (int)(((int64_t)start0 + n_ev) % W);
+            const int sx_new = mod_w((int64_t)start0 + n_ev);
             st_l[i] = st_new;
             sx_l[i] = sx_new;
             g_stored[i * A.tracker_stride[2]] = st_new;
