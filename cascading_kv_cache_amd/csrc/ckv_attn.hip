@@ -30,15 +30,15 @@ AttnWorkspace carve_attn(void* base, int64_t B, int64_t H, int64_t KVH, int64_t 
     const int64_t es = elem_bytes(dtype), N = NS + S + Q, n_pad = mfma_n_pad(N);
     Carver c(base);
     AttnWorkspace w;
-    w.qr = c.take((B * H * Q + 64) * D * es);  // 64 rows of slack for the MFMA column pass
+    w.qr = c.take((B * H * Q + kColSlack) * D * es);  // rows of slack for the MFMA column pass
     w.kr = c.take(B * KVH * n_pad * D * es);   // padded to whole key tiles for the MFMA family
     w.vc = c.take(B * KVH * n_pad * D * es);
     w.tile_vis = (unsigned long long*)c.take(n_pad / 64 * 8);
     w.kmasked = (uint8_t*)c.take(NS + S);
     w.lse = (float*)c.take(B * H * Q * 4);
-    w.lse2 = (float*)c.take((B * H * Q + 64) * 4);
+    w.lse2 = (float*)c.take((B * H * Q + kColSlack) * 4);
     w.colsum = (float*)c.take(B * H * N * 4);
-    w.w_ema = (float*)c.take((Q + 64) * 4);
+    w.w_ema = (float*)c.take((Q + kColSlack) * 4);
     w.w_new = (float*)c.take(Q * 4);
     w.bytes = c.off;
     return w;
@@ -183,7 +183,7 @@ extern "C" int64_t ckv_dense_workspace_bytes(int64_t B, int64_t H, int64_t n_ctx
     using ckv::align_up;
     if (ckv::dense_uses_mfma(dtype, D, H, n_ctx, n_kv))  // staged Q / K / V^T and the column pass's scratch
         return ckv::carve_attn(nullptr, B, H, H, n_ctx, D, 0, n_kv - n_ctx, dtype).bytes;
-    return align_up(B * H * n_ctx * 4, 256) + align_up(B * H * n_kv * 4, 256) + 2 * align_up((n_ctx + 64) * 4, 256);
+    return align_up(B * H * n_ctx * 4, 256) + align_up(B * H * n_kv * 4, 256) + 2 * align_up((n_ctx + ckv::kColSlack) * 4, 256);
 }
 
 extern "C" int ckv_attn_dense(const ckv_dense_args* args, void* stream_) {
@@ -243,7 +243,7 @@ extern "C" int ckv_attn_dense(const ckv_dense_args* args, void* stream_) {
     Carver c(a.workspace);
     float* lse = (float*)c.take(a.B * a.H * a.n_ctx * 4);
     float* colsum = (float*)c.take(a.B * a.H * a.n_kv * 4);
-    float* w_ema = (float*)c.take((a.n_ctx + 64) * 4);
+    float* w_ema = (float*)c.take((a.n_ctx + kColSlack) * 4);
     float* w_new = (float*)c.take(a.n_ctx * 4);
     int rc;
     if (a.scores) {

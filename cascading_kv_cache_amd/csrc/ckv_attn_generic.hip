@@ -18,7 +18,7 @@ __device__ inline float round_t(float v) {
 template <typename T>
 __global__ void weights_kernel(float* w_ema, float* w_new, int64_t Q, double beta) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= Q + 64) return;
+    if (i >= Q + kColSlack) return;
     if (i >= Q) {  // slack read (and multiplied by zero) by the MFMA column pass
         w_ema[i] = 0.f;
         return;
@@ -358,7 +358,7 @@ int launch_cast_scores(const float* colsum, void* scores, const int64_t* stride,
 }
 
 int launch_weights(float* w_ema, float* w_new, int64_t Q, double beta, int dtype, hipStream_t stream) {
-    const dim3 grid((unsigned)((Q + 64 + 255) / 256)), block(256);
+    const dim3 grid((unsigned)((Q + kColSlack + 255) / 256)), block(256);
     switch (dtype) {
         case CKV_F32: hipLaunchKernelGGL(weights_kernel<float>, grid, block, 0, stream, w_ema, w_new, Q, beta); break;
         case CKV_F16: hipLaunchKernelGGL(weights_kernel<__half>, grid, block, 0, stream, w_ema, w_new, Q, beta); break;

@@ -63,6 +63,10 @@ struct FinishProblem {
 };
 int launch_finish(const FinishProblem& p, hipStream_t stream);
 
+// rows of slack behind the staged queries, their normalisers and weights: the column pass reads whole
+// tiles of this many query rows
+constexpr int64_t kColSlack = 128;
+
 // ---- bf16/fp16 MFMA family (head_dim 128) ----
 struct MfmaSegment {
     const void* k;
@@ -88,7 +92,7 @@ struct MfmaProblem {
     void* out;
     int64_t out_stride[4];
     float* lse;            // (B, H, Q) natural log
-    float* lse2;           // (B*H*Q + 64) scratch: log2-domain copy for the column pass
+    float* lse2;           // (B*H*Q + kColSlack) scratch: minus the log2-domain normaliser, for the column pass
     float* colsum;         // (B, H, n) or null
     const float* w_ema;
     const float* w_new;

@@ -754,11 +754,11 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
 // score sums
 // ---------------------------------------------------------------------------------------------
 struct ColsumParams {
-    const void* qr;       // (B*H*Q + 64 rows of slack, D)
+    const void* qr;       // (B*H*Q + kColSlack rows, D)
     const void* kr;
     const unsigned long long* tile_vis;
-    const float* lse2;    // (B*H*Q + 64) minus the log2-domain row normalisers
-    const float* w_ema;   // (Q + 64), zero beyond Q
+    const float* lse2;    // (B*H*Q + kColSlack) minus the log2-domain row normalisers
+    const float* w_ema;   // (Q + kColSlack), zero beyond Q
     const float* w_new;   // (Q)
     float* colsum;        // (B*H, N)
     int64_t B, H, KVH, Q, N, Nc, n_pad;
@@ -768,8 +768,9 @@ struct ColsumParams {
     int nkb, first_chunk_blk, nbkv, xcd_aware, gsplit;  // block order and head split, see the kernel
 };
 
-constexpr int kQT2 = 64;                      // query rows per LDS tile of the column pass
-constexpr int kCsStage = 16384 + 256 + 256;   // Q tile + its lse2 + its weights
+constexpr int kQT2 = 128;                     // query rows per LDS tile of the column pass
+constexpr int kCsSub = kQT2 / 32;             // 32-row subtiles of a tile
+constexpr int kCsStage = kQT2 * 256 + 2 * kQT2 * 4;   // Q tile + its lse2 + its weights
 
 // One workgroup = one kv head x 256 keys (64 per wavefront, held in registers as the B operand of
 // S = Q K^T).  The (head, query-tile) sequence streams through a double-buffered LDS stage filled
@@ -848,12 +849,13 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     const int nmt = (Q - m_first + kQT2 - 1) / kQT2;  // query tiles per head
     const int n_steps = nmt * g_cnt;
 
-    // async copy assignments: the Q tile is 16 blocks of 1 KiB (4 per wavefront); wavefront 0 also
-    // brings the tile's 64 normalisers, wavefront 1 its 64 weights (16 lanes x 16 bytes each)
-    uint32_t q_src[4];
+    // async copy assignments: the Q tile is kQT2 / 4 blocks of 1 KiB (a quarter per wavefront); wavefront 0
+    // also brings the tile's normalisers, wavefront 1 its weights (kQT2 / 4 lanes x 16 bytes each)
+    constexpr int kQBlocks = kQT2 / 16;   // per wavefront
+    uint32_t q_src[kQBlocks];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int pos = (wave * 4 + j) * 64 + lane;
+    for (int j = 0; j < kQBlocks; j++) {
+        const int pos = (wave * kQBlocks + j) * 64 + lane;
         const int r = pos >> 4, c = (pos & 15) ^ (r & 15);
         q_src[j] = r * 256 + c * 16;
     }
@@ -868,10 +870,10 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
         const char* qt = (const char*)p.qr + row0 * (kD * (int64_t)sizeof(T));
         const uint32_t st = smem_addr + stage * kCsStage;
 #pragma unroll
-        for (int j = 0; j < 4; j++) async_copy16(qt, q_src[j], st + (wave * 4 + j) * 1024);
-        if (wave < 2 && lane < 16) {
+        for (int j = 0; j < kQBlocks; j++) async_copy16(qt, q_src[j], st + (wave * kQBlocks + j) * 1024);
+        if (wave < 2 && lane < kQT2 / 4) {
             const char* src = wave ? (const char*)(p.w_ema + mt) : (const char*)(p.lse2 + row0);
-            async_copy16(src, lane * 16, st + 16384 + wave * 256);
+            async_copy16(src, lane * 16, st + kQT2 * 256 + wave * (kQT2 * 4));
         }
     };
 
@@ -879,10 +881,13 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     auto tile_step = [&](auto stage_tag, int g, int mt) {
         constexpr int ST = decltype(stage_tag)::value;
         const unsigned char* q_lds = smem + ST * kCsStage;
-        const float* lse_lds = reinterpret_cast<const float*>(q_lds + 16384);
-        const float* w_lds = lse_lds + 64;
+        const float* lse_lds = reinterpret_cast<const float*>(q_lds + kQT2 * 256);
+        const float* w_lds = lse_lds + kQT2;
         const bool tail = mt + kQT2 > Q;                       // rows past the chunk end
         const bool diag = chunk_keys && mt <= last_nrel;       // tile may cross the diagonal
+        // Accumulators start from minus the row normaliser, so the matrix pipe hands back log2 P (the
+        // softmax scale is already on the staged queries).  Element (c, v) of a 32-row subtile c:
+        // query row mt + 32c + 8(v/4) + 4half + v%4, key column of this lane.
         auto row_init = [&](int c) {
             f32x16 init;
 #pragma unroll
@@ -895,130 +900,125 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
             }
             return init;
         };
+        auto load_weights = [&](int c, float(&ws)[16]) {
+#pragma unroll
+            for (int v4 = 0; v4 < 4; v4++) {
+                const float4 w4 = *reinterpret_cast<const float4*>(w_lds + 32 * c + 8 * v4 + 4 * half);
+                ws[4 * v4] = w4.x; ws[4 * v4 + 1] = w4.y; ws[4 * v4 + 2] = w4.z; ws[4 * v4 + 3] = w4.w;
+            }
+        };
         if (!tail && !diag && !new_chunk) {
-            // The common case, written in issue order: the logits of the second 32 rows go through
-            // the matrix pipe while the vector ALU turns the first 32 rows into weighted probabilities.
-            // Accumulators start from minus the row normaliser, so the matrix pipe hands back log2 P.
-            f32x16 s0[2], s1[2];
-            s0[0] = s0[1] = row_init(0);
-            uint4 a1[8];
+            // The common case, written in issue order: the logits of subtile c go through the matrix
+            // pipe while the vector ALU turns subtile c-1 into weighted probabilities.
+            f32x16 sq[2][2];  // [c & 1][ks]
+            sq[0][0] = sq[0][1] = row_init(0);
 #pragma unroll
             for (int kk = 0; kk < 8; kk++) {
                 const uint4 a = *reinterpret_cast<const uint4*>(q_lds + q_off[kk]);
-                s0[0] = Mma<T>::mma(a, kreg[0][kk], s0[0]);
-                s0[1] = Mma<T>::mma(a, kreg[1][kk], s0[1]);
+                sq[0][0] = Mma<T>::mma(a, kreg[0][kk], sq[0][0]);
+                sq[0][1] = Mma<T>::mma(a, kreg[1][kk], sq[0][1]);
             }
-            s1[0] = s1[1] = row_init(1);
 #pragma unroll
-            for (int kk = 0; kk < 8; kk++) a1[kk] = *reinterpret_cast<const uint4*>(q_lds + q_off[kk] + 8192);
-            float ws[16];
+            for (int c = 1; c < kCsSub; c++) {
+                sq[c & 1][0] = sq[c & 1][1] = row_init(c);
+                uint4 a1[8];
 #pragma unroll
-            for (int v4 = 0; v4 < 4; v4++) {
-                const float4 w4 = *reinterpret_cast<const float4*>(w_lds + 8 * v4 + 4 * half);
-                ws[4 * v4] = w4.x; ws[4 * v4 + 1] = w4.y; ws[4 * v4 + 2] = w4.z; ws[4 * v4 + 3] = w4.w;
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int slot = 0; slot < 16; slot++) {
-                const int kk = slot >> 1, ks = slot & 1;
-                s1[ks] = Mma<T>::mma(a1[kk], kreg[ks][kk], s1[ks]);
-#pragma unroll
-                for (int r = 0; r < 2; r++) {
-                    const int j = 2 * slot + r, ksv = j >> 4, v = j & 15;
-                    const float pe = __builtin_amdgcn_exp2f(s0[ksv][v]);
-                    acc[ksv] = fmaf(ws[v], pe, acc[ksv]);
-                }
+                for (int kk = 0; kk < 8; kk++) a1[kk] = *reinterpret_cast<const uint4*>(q_lds + q_off[kk] + c * 8192);
+                float ws[16];
+                load_weights(c - 1, ws);
                 __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int slot = 0; slot < 16; slot++) {
+                    const int kk = slot >> 1, ks = slot & 1;
+                    sq[c & 1][ks] = Mma<T>::mma(a1[kk], kreg[ks][kk], sq[c & 1][ks]);
+#pragma unroll
+                    for (int r = 0; r < 2; r++) {
+                        const int j = 2 * slot + r, ksv = j >> 4, v = j & 15;
+                        const float pe = __builtin_amdgcn_exp2f(sq[(c - 1) & 1][ksv][v]);
+                        acc[ksv] = fmaf(ws[v], pe, acc[ksv]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
+            {
+                float ws[16];
+                load_weights(kCsSub - 1, ws);
 #pragma unroll
-            for (int v4 = 0; v4 < 4; v4++) {
-                const float4 w4 = *reinterpret_cast<const float4*>(w_lds + 32 + 8 * v4 + 4 * half);
-                const float wv[4] = {w4.x, w4.y, w4.z, w4.w};
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
+                for (int v = 0; v < 16; v++) {
 #pragma unroll
                     for (int ks = 0; ks < 2; ks++) {
-                        const float pe = __builtin_amdgcn_exp2f(s1[ks][4 * v4 + e]);
-                        acc[ks] = fmaf(wv[e], pe, acc[ks]);
+                        const float pe = __builtin_amdgcn_exp2f(sq[(kCsSub - 1) & 1][ks][v]);
+                        acc[ks] = fmaf(ws[v], pe, acc[ks]);
                     }
                 }
             }
         } else {
-        // The accumulators start from minus the row normaliser, so the matrix pipe hands back
-        // log2 P directly (the softmax scale is already on the staged queries).
-        // Element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4.
-        f32x16 sacc[2][2];  // [c = query subtile][ks]
-#pragma unroll
-        for (int c = 0; c < 2; c++) sacc[c][0] = sacc[c][1] = row_init(c);
-#pragma unroll
-        for (int kk = 0; kk < 8; kk++) {
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-                const uint4 a = *reinterpret_cast<const uint4*>(q_lds + q_off[kk] + c * 8192);
-                sacc[c][0] = Mma<T>::mma(a, kreg[0][kk], sacc[c][0]);
-                sacc[c][1] = Mma<T>::mma(a, kreg[1][kk], sacc[c][1]);
-            }
-        }
-        // element (c, v): query row mt + 32c + 8(v/4) + 4half + v%4, key column of this lane
-        if (!tail && !diag && new_chunk) {
-            // every row is later than every key of the block: no masks.  A chunk key takes the
-            // weight of its distance m - n and the eager path's roundings; a cached key (only in
-            // the block that straddles the chunk start) takes the row's EMA weight unrounded.
-            const float* wb[2];
+            // special cases, one 32-row subtile at a time
+            const bool fast_new = !tail && !diag;   // new_chunk holds: every row is later than every key of the block
+            const float* wb[2] = {nullptr, nullptr};
             bool chunk_lane[2];
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
                 chunk_lane[ks] = nrel[ks] >= 0;
+                // a chunk key takes the weight of its distance m - n; a cached key (only in the block that
+                // straddles the chunk start) takes the row's EMA weight
                 wb[ks] = chunk_lane[ks] ? wnew_lds + (mt + 4 * half - nrel[ks]) : w_lds + 4 * half;
             }
+#pragma unroll 1
+            for (int c = 0; c < kCsSub; c++) {
+                f32x16 sacc[2];
+                sacc[0] = sacc[1] = row_init(c);
 #pragma unroll
-            for (int c = 0; c < 2; c++) {
+                for (int kk = 0; kk < 8; kk++) {
+                    const uint4 a = *reinterpret_cast<const uint4*>(q_lds + q_off[kk] + c * 8192);
+                    sacc[0] = Mma<T>::mma(a, kreg[0][kk], sacc[0]);
+                    sacc[1] = Mma<T>::mma(a, kreg[1][kk], sacc[1]);
+                }
+                if (fast_new) {
+                    // no masks; the eager path holds P and the products of chunk keys in the tensor dtype
 #pragma unroll
-                for (int v4 = 0; v4 < 4; v4++) {
-                    const int r0 = 32 * c + 8 * v4;
+                    for (int v4 = 0; v4 < 4; v4++) {
+                        const int r0 = 32 * c + 8 * v4;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
+                        for (int e = 0; e < 4; e++) {
+#pragma unroll
+                            for (int ks = 0; ks < 2; ks++) {
+                                const float pe = __builtin_amdgcn_exp2f(sacc[ks][4 * v4 + e]);
+                                const float w = wb[ks][r0 + e];
+                                if (pure_chunk) {
+                                    acc[ks] += Mma<T>::round1(Mma<T>::round1(pe) * w);
+                                } else {
+                                    const float prod = (chunk_lane[ks] ? Mma<T>::round1(pe) : pe) * w;
+                                    acc[ks] += chunk_lane[ks] ? Mma<T>::round1(prod) : prod;
+                                }
+                            }
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const int r = 32 * c + 8 * (v >> 2) + 4 * half + (v & 3);
+                        const int m = mt + r;
+                        const bool row_in = m < Q;
+                        const float we = w_lds[r];
 #pragma unroll
                         for (int ks = 0; ks < 2; ks++) {
-                            const float pe = __builtin_amdgcn_exp2f(sacc[c][ks][4 * v4 + e]);
-                            const float w = wb[ks][r0 + e];
-                            if (pure_chunk) {
+                            float pe = __builtin_amdgcn_exp2f(sacc[ks][v]);
+                            const bool is_chunk = nrel[ks] >= 0;
+                            const bool vis = row_in && (!is_chunk || m >= nrel[ks]);
+                            pe = vis ? pe : 0.f;
+                            if (is_chunk && p.new_mode) {
+                                // the eager path holds P and the products in the tensor dtype
+                                const float w = vis ? wnew_lds[m - nrel[ks]] : 0.f;
                                 acc[ks] += Mma<T>::round1(Mma<T>::round1(pe) * w);
                             } else {
-                                const float prod = (chunk_lane[ks] ? Mma<T>::round1(pe) : pe) * w;
-                                acc[ks] += chunk_lane[ks] ? Mma<T>::round1(prod) : prod;
+                                acc[ks] = fmaf(row_in ? we : 0.f, pe, acc[ks]);
                             }
                         }
                     }
                 }
             }
-        } else {
-#pragma unroll
-            for (int c = 0; c < 2; c++) {
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int r = 32 * c + 8 * (v >> 2) + 4 * half + (v & 3);
-                    const int m = mt + r;
-                    const bool row_in = m < Q;
-                    const float we = w_lds[r];
-#pragma unroll
-                    for (int ks = 0; ks < 2; ks++) {
-                        float pe = __builtin_amdgcn_exp2f(sacc[c][ks][v]);
-                        const bool is_chunk = nrel[ks] >= 0;
-                        const bool vis = row_in && (!is_chunk || m >= nrel[ks]);
-                        pe = vis ? pe : 0.f;
-                        if (is_chunk && p.new_mode) {
-                            // the eager path holds P and the products in the tensor dtype
-                            const float w = vis ? wnew_lds[m - nrel[ks]] : 0.f;
-                            acc[ks] += Mma<T>::round1(Mma<T>::round1(pe) * w);
-                        } else {
-                            acc[ks] = fmaf(row_in ? we : 0.f, pe, acc[ks]);
-                        }
-                    }
-                }
-            }
         }
-        }  // special cases
         if (mt + kQT2 >= Q) {  // head finished: combine the two lane halves and store
             const int64_t h = kvh * p.G + g;
 #pragma unroll
@@ -1175,7 +1175,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
 bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH, int64_t Q) {
     if (dtype != CKV_BF16 && dtype != CKV_F16) return false;
     if (D != kD) return false;
-    if (Q > 24576) return false;  // the column pass keeps a Q-long weight table in LDS
+    if (Q > 16384) return false;  // the column pass keeps a Q-long weight table in LDS beside its two stages
     const int64_t G = H / KVH;
     return G >= 1 && G <= kRows / 32;  // at least 32 positions per workgroup
 }
