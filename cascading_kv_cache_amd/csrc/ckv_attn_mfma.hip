@@ -92,8 +92,8 @@ struct StageParams {
     const float* inv_freq;
     float theta;
     int shared_pos;          // every (b, kvh) uses position row [0, 0]
-    void* kr;                // (B*KVH, n_pad, D)
-    void* vt;                // (B*KVH, n_pad/64, D, 64)
+    void* kr;                // (B*KVH, n_pad/64) K tile images, see k_image_off
+    void* vt;                // (B*KVH, n_pad/64) V^T tile images, see v_image_off
     unsigned long long* tile_vis;  // (n_pad/64,)
     int64_t B, KVH, n, n_pad;
 };
@@ -105,6 +105,16 @@ __device__ inline int find_segment(const StageParams& p, int64_t n, int64_t& loc
     local = n - p.seg[1].len;
     return 2;
 }
+
+// The staged K and V of one 64-key tile are 16 KiB images in exactly the order the forward kernel
+// keeps them in LDS, so a tile reaches LDS as a straight copy and the 64 lanes of an operand read
+// touch 1 KiB made of two contiguous halves (no bank conflicts, one base address per lane):
+//   K image:   16-byte piece c (elements 8c .. 8c+7) of key row r at  (c/2)*2048 + (c%2)*1024 + r*16
+//   V^T image: 16-byte piece c (key slots 8c .. 8c+7) of dim row d at (c/2)*4096 + (c%2)*2048 + d*16
+// Key slot 16s + 8h + 4a + e of a V^T row holds key 16s + 8a + 4h + e of the tile: the order in
+// which the logits leave the matrix pipe.
+__device__ __host__ inline int k_image_off(int r, int c) { return (c >> 1) * 2048 + (c & 1) * 1024 + r * 16; }
+__device__ __host__ inline int v_image_off(int d, int c) { return (c >> 1) * 4096 + (c & 1) * 2048 + d * 16; }
 
 // grid (n_pad/64, splits); 256 threads: thread = (key = tid/4, quarter = tid%4) owns rotation pairs
 // j = 16*quarter .. 16*quarter+15, i.e. elements [16q,16q+16) and [64+16q, 64+16q+16) of its row.
@@ -192,11 +202,11 @@ __global__ void __launch_bounds__(256) stage_keys_kernel(StageParams p) {
                 }
             }
         }
-        T* krow = (T*)p.kr + (bh * p.n_pad + n) * kD;
-        *reinterpret_cast<uint4*>(krow + 16 * quarter) = lo[0];
-        *reinterpret_cast<uint4*>(krow + 16 * quarter + 8) = lo[1];
-        *reinterpret_cast<uint4*>(krow + 64 + 16 * quarter) = hi[0];
-        *reinterpret_cast<uint4*>(krow + 64 + 16 * quarter + 8) = hi[1];
+        char* kimg = (char*)p.kr + (bh * (p.n_pad / kBN) + tile) * (int64_t)(kD * kBN * sizeof(T));
+        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 2 * quarter)) = lo[0];
+        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 2 * quarter + 1)) = lo[1];
+        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 8 + 2 * quarter)) = hi[0];
+        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 9 + 2 * quarter)) = hi[1];
 
         // V: through LDS into the transposed tile
         __syncthreads();
@@ -210,7 +220,7 @@ __global__ void __launch_bounds__(256) stage_keys_kernel(StageParams p) {
             }
         }
         __syncthreads();
-        T* vt = (T*)p.vt + (bh * (p.n_pad / kBN) + tile) * (int64_t)(kD * kBN);
+        char* vimg = (char*)p.vt + (bh * (p.n_pad / kBN) + tile) * (int64_t)(kD * kBN * sizeof(T));
         // thread -> (d = tid/2, half of the 64 slots): 32 slots = 4 x 16 bytes
         {
             const int d = tid >> 1, sh = (tid & 1) * 32;
@@ -222,10 +232,9 @@ __global__ void __launch_bounds__(256) stage_keys_kernel(StageParams p) {
                 const int s = slot >> 4, h = (slot >> 3) & 1, a = (slot >> 2) & 1, e = slot & 3;
                 tmp[sl] = v_lds[16 * s + 8 * a + 4 * h + e][d];
             }
-            uint4* dst = reinterpret_cast<uint4*>(vt + d * kBN + sh);
             const uint4* src = reinterpret_cast<const uint4*>(tmp);
 #pragma unroll
-            for (int i = 0; i < 4; i++) dst[i] = src[i];
+            for (int i = 0; i < 4; i++) *reinterpret_cast<uint4*>(vimg + v_image_off(d, sh / 8 + i)) = src[i];
         }
     }
 }
@@ -305,8 +314,8 @@ __global__ void __launch_bounds__(64) stage_q_kernel(StageQParams p) {
 // ---------------------------------------------------------------------------------------------
 struct FwdParams {
     const void* qr;   // (B*H, Q, D)
-    const void* kr;   // (B*KVH, n_pad, D)
-    const void* vt;   // (B*KVH, n_pad/64, D, 64)
+    const void* kr;   // (B*KVH, n_pad/64) K tile images
+    const void* vt;   // (B*KVH, n_pad/64) V^T tile images
     const unsigned long long* tile_vis;
     void* out;
     int64_t out_stride[4];
@@ -343,12 +352,10 @@ __device__ inline uint32_t lds_address(const void* p) {
 }
 
 
-// LDS tiles are unpadded (the async copy writes 1 KiB per wavefront contiguously); bank conflicts
-// are avoided by XOR-swizzling the 16-byte piece index with the row:
-//   K tile   piece c of key row r   lives at r*256 + ((c ^ (r & 15)) << 4)
-//   V^T tile piece c of dim row d   lives at d*128 + ((c ^ ((d >> 1) & 7)) << 4)
+// LDS tile of 256-byte rows taken from a row-major matrix (the query tile of the column pass): unpadded
+// (the async copy writes 1 KiB per wavefront contiguously); bank conflicts are avoided by XOR-swizzling
+// the 16-byte piece index with the row: piece c of row r lives at r*256 + ((c ^ (r & 15)) << 4)
 __device__ inline int k_lds_off(int r, int c) { return r * 256 + ((c ^ (r & 15)) << 4); }
-__device__ inline int v_lds_off(int d, int c) { return d * 128 + ((c ^ ((d >> 1) & 7)) << 4); }
 
 // max over the two lane halves (lane l and lane l ^ 32) without a trip through LDS
 __device__ inline float half_max(float x) {
@@ -359,14 +366,15 @@ __device__ inline float half_max(float x) {
 // Software-pipelined forward: eight wavefronts, 32 (head, position) rows each.  Iteration i runs
 // the softmax of tile i on the vector ALU while the matrix pipe adds the P.V product of tile i-1
 // and computes the logits of tile i+1; neither depends on the softmax in flight, so the two pipes
-// overlap inside one wavefront.  LDS: two K stages and three V^T stages.  Iteration i copies K
-// tile i+2 and V^T tile i+1, so everything an iteration reads was complete one barrier earlier
-// and its first operands can be fetched before the barrier.
+// overlap inside one wavefront.  LDS: three K stages and four V^T stages.  Iteration i copies K
+// tile i+3 and V^T tile i+2, which are first read in iteration i+2: the barrier between two
+// iterations waits only for the copies of the iteration before the last one (those of the last one
+// stay in flight across it), and the first operands of an iteration can be fetched before its barrier.
 constexpr int kPipeStage = 16384;
-constexpr int kPipeLds = 5 * kPipeStage;   // K0 K1 V0 V1 V2
-constexpr int kPipeSrc = 4 * 512 * 4;      // copy source offsets, 4 per lane
-// stages, copy offsets, one visibility word and one work-list entry per key tile, the list length
-inline int64_t pipe_lds_bytes(int64_t n_pad) { return kPipeLds + kPipeSrc + (n_pad / kBN) * 12 + 16; }
+constexpr int kKStages = 3, kVStages = 4;
+constexpr int kPipeLds = (kKStages + kVStages) * kPipeStage;   // K0 K1 K2 V0 V1 V2 V3
+// stages, one visibility word and one work-list entry per key tile, the list length
+inline int64_t pipe_lds_bytes(int64_t n_pad) { return kPipeLds + (n_pad / kBN) * 12 + 16; }
 constexpr int64_t kLdsLimit = 160 * 1024;
 
 template <typename T>
@@ -393,9 +401,8 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     if (m_hi > (int)p.Q - 1) m_hi = (int)p.Q - 1;
     const int n_tiles = (int)((p.Nc + m_hi) / kBN) + 1;
     const int tiles_cap = (int)(p.n_pad / kBN);
-    unsigned long long* vis_lds = reinterpret_cast<unsigned long long*>(smem + kPipeLds + kPipeSrc);
-    uint32_t* src_lds = reinterpret_cast<uint32_t*>(smem + kPipeLds);   // per-lane source offsets of the copies
-    int* list_lds = reinterpret_cast<int*>(smem + kPipeLds + kPipeSrc + 8 * tiles_cap);
+    unsigned long long* vis_lds = reinterpret_cast<unsigned long long*>(smem + kPipeLds);
+    int* list_lds = reinterpret_cast<int*>(smem + kPipeLds + 8 * tiles_cap);
     const uint32_t smem_addr = lds_address(smem);
 
     // ---- work list: tiles with at least one visible key; bit 31 marks tiles that need masking
@@ -440,40 +447,42 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
         for (int v = 0; v < 16; v++) oacc[dt][v] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;  // l_run: partial over this lane's keys; halves are added at the end
 
-    // ---- per-lane constants of the copies (source offsets) and of the operand reads (LDS offsets)
-    // (kept in LDS: a register spilled to scratch would make every reload wait for the copies in flight)
-#pragma unroll
-    for (int j = 0; j < kBlocksPerWave; j++) {
-        const int blk = wave * kBlocksPerWave + j;
-        const int pos = blk * 64 + lane;                     // piece position inside the LDS tile
-        const int kr_ = pos >> 4, kc = (pos & 15) ^ (kr_ & 15);
-        src_lds[(2 + j) * kThreads + tid] = kr_ * 256 + kc * 16;
-        const int vd = pos >> 3, vc = (pos & 7) ^ ((vd >> 1) & 7);
-        src_lds[j * kThreads + tid] = vd * 128 + vc * 16;
-    }
-    int k_off[8], v_off[4];  // key row `col` (+32 rows = +8192 B), dim row `col` (+32 rows = +4096 B)
-#pragma unroll
-    for (int kk = 0; kk < 8; kk++) k_off[kk] = k_lds_off(col, 2 * kk + half);
-#pragma unroll
-    for (int s = 0; s < 4; s++) v_off[s] = v_lds_off(col, 2 * s + half);
+    // ---- LDS byte offset of this lane's operand pieces inside the stage being read (pieces of later
+    // contraction steps / row blocks are at compile-time distances); moved from stage to stage in place.
+    // k_base: key row `col` of the K stage with the next logits' tile; v_base: dim row `col` of the V^T
+    // stage with the tile to multiply.
+    int k_base = k_image_off(col, half);
+    int v_base = v_image_off(col, half) + (kKStages + kVStages - 1) * kPipeStage;
+    int k_rd = 0, v_rd = kVStages - 1;  // the stages k_base / v_base point at
+    auto advance_k = [&]() {
+        k_base += k_rd == kKStages - 1 ? -(kKStages - 1) * kPipeStage : kPipeStage;
+        k_rd = k_rd == kKStages - 1 ? 0 : k_rd + 1;
+    };
+    auto advance_v = [&]() {
+        v_base += v_rd == kVStages - 1 ? -(kVStages - 1) * kPipeStage : kPipeStage;
+        v_rd = v_rd == kVStages - 1 ? 0 : v_rd + 1;
+    };
+    // K piece (kk, ks): contraction step kk of key rows 32ks ..; V^T piece (s, dt): step s of dim rows 32dt ..
+    auto k_piece = [&](int kk, int ks) { return *reinterpret_cast<const uint4*>(smem + k_base + kk * 2048 + ks * 512); };
+    auto v_piece = [&](int s_, int dt) { return *reinterpret_cast<const uint4*>(smem + v_base + s_ * 4096 + dt * 512); };
+    const uint32_t copy_off = lane * 16;  // a wavefront copies 1 KiB blocks of an image as they are
     const char* kbase = (const char*)uniform_ptr((const char*)p.kr + bkv * p.n_pad * kD * (int64_t)sizeof(T));
     const char* vbase = (const char*)uniform_ptr((const char*)p.vt + bkv * p.n_pad * kD * (int64_t)sizeof(T));
     constexpr int kTileBytes = kBN * kD * (int)sizeof(T);
 
-    // one 1 KiB block (j = 0, 1) of a tile into K stage `stage` (0, 1) / V^T stage `stage` (0..2)
-    auto copy_k = [&](int t, int stage, int j, uint32_t src) {
-        async_copy16(kbase + (int64_t)t * kTileBytes, src, smem_addr + stage * kPipeStage + (wave * kBlocksPerWave + j) * 1024);
+    // one 1 KiB block (j = 0, 1) of a tile into K stage `stage` / V^T stage `stage`
+    auto copy_k = [&](int t, int stage, int j) {
+        const int blk = (wave * kBlocksPerWave + j) * 1024;
+        async_copy16(kbase + (int64_t)t * kTileBytes + blk, copy_off, smem_addr + stage * kPipeStage + blk);
     };
-    auto copy_v = [&](int t, int stage, int j, uint32_t src) {
-        async_copy16(vbase + (int64_t)t * kTileBytes, src,
-                     smem_addr + (2 + stage) * kPipeStage + (wave * kBlocksPerWave + j) * 1024);
+    auto copy_v = [&](int t, int stage, int j) {
+        const int blk = (wave * kBlocksPerWave + j) * 1024;
+        async_copy16(vbase + (int64_t)t * kTileBytes + blk, copy_off, smem_addr + (kKStages + stage) * kPipeStage + blk);
     };
     auto work = [&](int j) { return __builtin_amdgcn_readfirstlane(list_lds[j < n_work ? j : n_work - 1]); };
 
-    // logits of the K tile in stage ST: s[ks][v] = key 32ks + 8(v/4) + 4half + v%4, query column col
-    auto qk = [&](auto stage_tag, f32x16(&s)[2]) {
-        constexpr int ST = decltype(stage_tag)::value;
-        const unsigned char* k_lds = smem + ST * kPipeStage;
+    // logits of the K tile k_base points at: s[ks][v] = key 32ks + 8(v/4) + 4half + v%4, query column col
+    auto qk = [&](f32x16(&s)[2]) {
 #pragma unroll
         for (int ks = 0; ks < 2; ks++)
 #pragma unroll
@@ -482,20 +491,18 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
         for (int kk = 0; kk < 8; kk++) {
 #pragma unroll
             for (int ks = 0; ks < 2; ks++) {
-                const uint4 a = *reinterpret_cast<const uint4*>(k_lds + k_off[kk] + ks * 8192);
-                s[ks] = Mma<T>::mma(a, qreg[kk], s[ks]);
+                s[ks] = Mma<T>::mma(k_piece(kk, ks), qreg[kk], s[ks]);
             }
         }
     };
     uint32_t pk[4][4];  // P^T of one tile as the B operands of the four P.V contraction steps
-    // O^T += V^T P^T with the V^T tile in stage `stage` (0..2)
-    auto pv = [&](int stage) {
-        const unsigned char* v_lds = smem + (2 + stage) * kPipeStage;
+    // O^T += V^T P^T with the V^T tile v_base points at
+    auto pv = [&]() {
 #pragma unroll
         for (int s = 0; s < 4; s++) {
 #pragma unroll
             for (int dt = 0; dt < 4; dt++) {
-                const uint4 a = *reinterpret_cast<const uint4*>(v_lds + v_off[s] + dt * 4096);
+                const uint4 a = v_piece(s, dt);
                 const uint4 bq = make_uint4(pk[s][0], pk[s][1], pk[s][2], pk[s][3]);
                 oacc[dt] = Mma<T>::mma(a, bq, oacc[dt]);
             }
@@ -537,34 +544,32 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     };
 
     // Iteration i, written in issue order: 32 slots, each one matrix instruction (slots 0..15: P.V of
-    // tile i-1 out of V^T stage v_rd, slots 16..31: logits of tile i+1 out of K stage ST), the LDS
-    // read of the operand kAhead slots ahead, and a slice of the softmax of tile i.  Scheduling
-    // barriers keep the slots as written, so matrix and vector instructions alternate inside the
-    // wavefront.  The probabilities of tile i overwrite those of tile i-1 piece by piece, each after
-    // its last use by the P.V product.  The copies (V^T tile t_v into stage v_wr, K tile t_k into
-    // the other K stage) go out one at a time, a quarter of the slots apart.
+    // tile i-1 out of the V^T stage at v_base, slots 16..31: logits of tile i+1 out of the K stage at
+    // k_base), the LDS read of the operand kAhead slots ahead, and a slice of the softmax of tile i.
+    // Scheduling barriers keep the slots as written, so matrix and vector instructions alternate
+    // inside the wavefront.  The probabilities of tile i overwrite those of tile i-1 piece by piece,
+    // each after its last use by the P.V product.  The copies (V^T tile t_v = i+2 into stage v_wr, K
+    // tile t_k = i+3 into stage k_wr, both last read in iteration i-1) go out one at a time, a quarter
+    // of the slots apart.
     // pre[]: on entry the operands of slots 0..kAhead-1, read before the barrier; on exit those
     // of the next iteration.
-    // fetch_idx / fetched: the work-list entry three tiles ahead is read from LDS in the middle of the
+    // fetch_idx / fetched: the work-list entry four tiles ahead is read from LDS in the middle of the
     // slots, so its latency is never waited for.
-    auto iteration = [&](auto stage_tag, auto with_pv, int entry, int t_v, int t_k, int v_rd, int v_wr, f32x16(&s_cur)[2],
-                         f32x16(&s_nxt)[2], uint4(&pre)[kAhead], int fetch_idx, int& fetched) {
-        constexpr int ST = decltype(stage_tag)::value;
+    auto iteration = [&](auto with_pv, int entry, int t_v, int t_k, f32x16(&s_cur)[2], f32x16(&s_nxt)[2],
+                         uint4(&pre)[kAhead], int fetch_idx, int& fetched) {
         constexpr bool kPV = decltype(with_pv)::value;
         constexpr int kSlots = kPV ? 32 : 16, kQk0 = kPV ? 16 : 0;
         constexpr int kCopyStep = kSlots / 4;
-        const unsigned char* k_lds = smem + ST * kPipeStage;
-        int v_addr[4];
-#pragma unroll
-        for (int s = 0; s < 4; s++) v_addr[s] = v_off[s] + (2 + v_rd) * kPipeStage;
+        const int v_wr = v_rd == 0 ? kVStages - 1 : v_rd - 1;   // (v_rd + 3) % 4
+        const int k_wr = k_rd == 0 ? kKStages - 1 : k_rd - 1;   // (k_rd + 2) % 3
         if (entry < 0) mask_tile(entry, s_cur);
         rescale();  // tile i-2 is in the accumulator; tile i-1, scaled for the newer maximum, is added below
         auto operand = [&](int k) -> uint4 {
             if (k >= kQk0) {
                 const int j = k - kQk0;  // K piece (kk, ks) = (j / 2, j % 2)
-                return *reinterpret_cast<const uint4*>(k_lds + k_off[j >> 1] + (j & 1) * 8192);
+                return k_piece(j >> 1, j & 1);
             }
-            return *reinterpret_cast<const uint4*>(smem + v_addr[k >> 2] + (k & 3) * 4096);  // V^T piece (s, dt)
+            return v_piece(k >> 2, k & 3);
         };
         uint4 ops[kSlots];
 #pragma unroll
@@ -576,19 +581,15 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
         constexpr int kExpFirst = kMaxSlots + 1;           // first slot with probabilities
         constexpr int kExpPer = kPV ? 1 : 2;               // pairs per slot
         float q0[kExpPer], q1[kExpPer];                    // exponentials of the previous slot, packed one slot later
-        // the source offset of a copy is read from LDS two slots before the copy, so that waiting
-        // for it does not also wait for the operand reads issued since
-        uint32_t src = src_lds[tid];
         int raw_entry = 0;
 #pragma unroll
         for (int k = 0; k < kSlots; k++) {
             if (k + kAhead < kSlots) ops[k + kAhead] = operand(k + kAhead);
             if (k % kCopyStep == 1) {
                 const int q = k / kCopyStep;               // 0, 1: V^T blocks; 2, 3: K blocks
-                if (q < 2) copy_v(t_v, v_wr, q, src);
-                else copy_k(t_k, 1 - ST, q - 2, src);
+                if (q < 2) copy_v(t_v, v_wr, q);
+                else copy_k(t_k, k_wr, q - 2);
             }
-            if (k % kCopyStep == kCopyStep - 1 && k + 2 < kSlots) src = src_lds[((k + 2) / kCopyStep) * kThreads + tid];
             if (k == 4) raw_entry = list_lds[fetch_idx];
             if (k >= kQk0) {
                 const int j = k - kQk0;
@@ -634,14 +635,12 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
         }
         l_run = l_run * alpha + (rs0 + rs1);
         fetched = __builtin_amdgcn_readfirstlane(raw_entry);
-        // first operands of the next iteration: V^T tile i, complete since the last barrier
-        {
-            const int v_next = v_rd == 2 ? 0 : v_rd + 1;
+        // on to the stages of tiles i and i+2; first operands of the next iteration: V^T tile i,
+        // complete since the last barrier
+        advance_v();
+        advance_k();
 #pragma unroll
-            for (int k = 0; k < kAhead; k++) {
-                pre[k] = *reinterpret_cast<const uint4*>(smem + v_off[k >> 2] + (2 + v_next) * kPipeStage + (k & 3) * 4096);
-            }
-        }
+        for (int k = 0; k < kAhead; k++) pre[k] = v_piece(k >> 2, k & 3);
         // keep the packed probabilities in this region (they are next read after the barrier)
 #pragma unroll
         for (int st = 0; st < 4; st++) asm volatile("" ::"v"(pk[st][0]), "v"(pk[st][1]), "v"(pk[st][2]), "v"(pk[st][3]));
@@ -649,45 +648,41 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
 
     f32x16 sA[2], sB[2];
     uint4 pre[kAhead];
-    using S0 = std::integral_constant<int, 0>;
-    using S1 = std::integral_constant<int, 1>;
     if (n_work > 0) {
 #pragma unroll
         for (int j = 0; j < kBlocksPerWave; j++) {
-            copy_k(work(0) & 0x7fffffff, 0, j, src_lds[(2 + j) * kThreads + tid]);
-            copy_k(work(1) & 0x7fffffff, 1, j, src_lds[(2 + j) * kThreads + tid]);
-            copy_v(work(0) & 0x7fffffff, 0, j, src_lds[j * kThreads + tid]);
+            copy_k(work(0) & 0x7fffffff, 0, j);
+            copy_k(work(1) & 0x7fffffff, 1, j);
+            copy_k(work(2) & 0x7fffffff, 2, j);
+            copy_v(work(0) & 0x7fffffff, 0, j);
+            copy_v(work(1) & 0x7fffffff, 1, j);
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
-        qk(S0{}, sA);
-        // iteration 0: nothing to multiply by V yet.  e0 / e1 / e2: work-list entries of tiles i, i+1, i+2
+        qk(sA);
+        advance_k();
+        // iteration 0: nothing to multiply by V yet.  e0 .. e3: work-list entries of tiles i .. i+3
         auto clamp_idx = [&](int j) { return j < n_work ? j : n_work - 1; };
-        int e0 = work(0), e1 = work(1), e2 = work(2), e3 = 0;
+        int e0 = work(0), e1 = work(1), e2 = work(2), e3 = work(3), e4 = 0;
         __syncthreads();                     // every wavefront is done with K stage 0
-        iteration(S1{}, std::false_type{}, e0, e1 & 0x7fffffff, e2 & 0x7fffffff, 2, 1, sA, sB, pre, clamp_idx(3), e3);
-        int v_rd = 0;                        // (i - 1) % 3
-        auto next3 = [](int x) { return x == 2 ? 0 : x + 1; };
+        iteration(std::false_type{}, e0, e2 & 0x7fffffff, e3 & 0x7fffffff, sA, sB, pre, clamp_idx(4), e4);
+        // all copies but the four of the iteration just finished have landed
+        constexpr int kWaitOlder = 0x0F74;   // vmcnt(4)
         for (int i = 1; i < n_work; i += 2) {
-            // odd iteration: K stage 0 is read, K stage 1 refilled
-            e0 = e1; e1 = e2; e2 = e3;
-            __builtin_amdgcn_s_waitcnt(0x0F70);
+            e0 = e1; e1 = e2; e2 = e3; e3 = e4;
+            __builtin_amdgcn_s_waitcnt(kWaitOlder);
             __syncthreads();
-            iteration(S0{}, std::true_type{}, e0, e1 & 0x7fffffff, e2 & 0x7fffffff, v_rd, next3(next3(v_rd)), sB, sA, pre,
-                      clamp_idx(i + 3), e3);
-            v_rd = next3(v_rd);
+            iteration(std::true_type{}, e0, e2 & 0x7fffffff, e3 & 0x7fffffff, sB, sA, pre, clamp_idx(i + 4), e4);
             if (i + 1 < n_work) {
-                e0 = e1; e1 = e2; e2 = e3;
-                __builtin_amdgcn_s_waitcnt(0x0F70);
+                e0 = e1; e1 = e2; e2 = e3; e3 = e4;
+                __builtin_amdgcn_s_waitcnt(kWaitOlder);
                 __syncthreads();
-                iteration(S1{}, std::true_type{}, e0, e1 & 0x7fffffff, e2 & 0x7fffffff, v_rd, next3(next3(v_rd)), sA, sB, pre,
-                          clamp_idx(i + 4), e3);
-                v_rd = next3(v_rd);
+                iteration(std::true_type{}, e0, e2 & 0x7fffffff, e3 & 0x7fffffff, sA, sB, pre, clamp_idx(i + 5), e4);
             }
         }
         // the P.V product of the last tile; the copies still in flight are repeats that nobody reads
         rescale();
-        pv(v_rd);
+        pv();
         __builtin_amdgcn_s_waitcnt(0x0F70);
     }
 
@@ -821,7 +816,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     const int64_t key_w = key_blk + wave * 64;            // first key of this wavefront
 
     uint4 kreg[2][8];
-    const T* kbase = (const T*)p.kr + bkv * p.n_pad * kD;
+    const char* kbase = (const char*)p.kr + bkv * p.n_pad * kD * (int64_t)sizeof(T);
     bool live[2];
     int nrel[2];
 #pragma unroll
@@ -829,7 +824,8 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
         const int64_t n = key_w + 32 * ks + col;
 #pragma unroll
         for (int kk = 0; kk < 8; kk++) {
-            kreg[ks][kk] = n < p.n_pad ? *reinterpret_cast<const uint4*>(kbase + n * kD + 16 * kk + 8 * half)
+            kreg[ks][kk] = n < p.n_pad ? *reinterpret_cast<const uint4*>(kbase + (n / kBN) * (int64_t)(kBN * kD * sizeof(T)) +
+                                                                         k_image_off((int)(n % kBN), 2 * kk + half))
                                        : make_uint4(0, 0, 0, 0);
         }
         live[ks] = n < p.N && ((p.tile_vis[n / kBN] >> (n % kBN)) & 1ull);
