@@ -574,16 +574,28 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
 // ---------------------------------------------------------------------------------------------
 // Streaming variant of the main kernel (16-bit caches, shared positions, G <= 4).
 //
-// The (key tile, batch x kv-head) items are dealt out in equal contiguous runs, one workgroup per
-// CU, so the launch has no tail.  K and V rows are read with fully coalesced 16-byte loads (1 KiB
-// per wavefront instruction) one item ahead into registers, then written to LDS, from where the
-// MFMA operand layout (K) and the dims-per-lane layout (V) are read back.  Each of the eight
-// wavefronts stages exactly the 16 key rows it consumes, so staging needs no workgroup barrier.
-// The partial results of an item are written out one iteration late, off the critical path.
+// The (64-key tile, batch x kv-head) items are dealt out in equal contiguous runs over as many
+// workgroups as the chip holds at once (two per CU), so the launch has no tail.  A workgroup is four
+// wavefronts; each stages 16 key rows of an item.  The rows travel global -> LDS as asynchronous
+// copies one item ahead (two LDS stages), swizzled on the way by the choice of each lane's source
+// piece, so no register holds data in flight and the loads of the next item overlap the arithmetic
+// of this one.  Per item: (1) every wavefront rotates its 16 K rows in registers (cos / sin of the
+// tile's positions stay in registers for all (b, kvh) of the tile) and gets their logits from the
+// matrix pipe; (2) after the item's only workgroup barrier every wavefront normalises all 64 logits
+// of each head (redundantly: 4 values per lane) and (3) multiplies P by a 32-dim slice of all 64 V
+// rows on the matrix pipe, so the tile's partial result is complete in registers and needs no
+// combination across wavefronts.  It is written out at the top of the next item, off the critical
+// path.
 // ---------------------------------------------------------------------------------------------
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-constexpr int kSK = 128;                       // keys per tile
-constexpr int kStreamStage = 2 * kSK * 256;    // K rows then V rows of one tile (16-bit, 256 B per row)
+constexpr int kStreamWaves = 8;                   // wavefronts per workgroup, 16 keys each
+constexpr int kSK = 16 * kStreamWaves;            // keys per tile
+constexpr int kStreamThreads = 64 * kStreamWaves;
+constexpr int kStreamWgPerCu = 8 / kStreamWaves;  // eight wavefronts per CU
+constexpr int kStreamDimBlocks = 8 / kStreamWaves;  // 16-dim blocks of the output a wavefront owns
+constexpr int kStreamStage = 2 * kSK * 256;       // K rows then V rows of one tile (16-bit, 256 B per row)
+// two stages | per wavefront two 1 KiB query blocks | two [4 heads][kSK keys] logit planes | per wavefront [4][kSK] probabilities
+constexpr int kStreamQ = 2 * kStreamStage, kStreamS = kStreamQ + kStreamWaves * 2048, kStreamP = kStreamS + 2 * 4 * kSK * 4;
+constexpr int kStreamLds = kStreamP + kStreamWaves * 4 * kSK * 2;
 
 // sum / max over the four 16-lane rows of a wavefront (lanes l, l^16, l^32, l^48)
 __device__ inline float rows4_sum(float x) {
@@ -598,29 +610,44 @@ __device__ inline float rows4_max(float x) {
     const auto q = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
     return fmaxf(__uint_as_float(q[0]), __uint_as_float(q[1]));
 }
+// all-reduce over lanes l, l+4, l+8, l+12 of every 16-lane row, then over the four rows: the 16 lanes with equal l % 4
+__device__ inline float mod4_max(float m) {
+    m = fmaxf(m, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(m), 0x124, 0xF, 0xF, true)));  // row_ror:4
+    m = fmaxf(m, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(m), 0x128, 0xF, 0xF, true)));  // row_ror:8
+    return rows4_max(m);
+}
+__device__ inline float mod4_sum(float l) {
+    l += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(l), 0x124, 0xF, 0xF, true));
+    l += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(l), 0x128, 0xF, 0xF, true));
+    return rows4_sum(l);
+}
 
-inline int stream_lds_bytes(int G) { return kStreamStage + (8 * G * kD + 8 * G * 2 + 8 * 16 * 8) * (int)sizeof(float); }
+// the byte offsets of the rows inside a (b, kvh) slab must fit the 32-bit lane offsets of the copies
+inline bool stream_offsets_fit(const ckv_attn_args& a) {
+    const int64_t lim = (int64_t)1 << 31, es = 2;
+    return a.S * a.cache_stride[2] * es + 256 < lim && a.num_sink * a.sink_stride[2] * es + 256 < lim;
+}
 
 template <typename T, int G>
-__global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
+__global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_kernel(DecodeParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
-    float* red_o = reinterpret_cast<float*>(smem + kStreamStage);  // [8 waves][G][128]
-    float* red_ml = red_o + 8 * G * kD;                                // [8][G][2]
-    float* s_lds = red_ml + 8 * G * 2;                                 // [8][16 keys][8] logits, then [16][4] probabilities
-    const uint32_t lds_base = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)smem;
+    const uint32_t lds_base = lds_address(smem);
     const ckv_attn_args& a = p.a;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int key16 = lane & 15, kq = lane >> 4;  // phase 1: MFMA column (key) and k-quarter
-    const int pkey = lane >> 2, pg = lane & 3;    // softmax: one (key, head) per lane
-    float* s_wave = s_lds + wave * 16 * 8;
+    const int key16 = lane & 15, kq = lane >> 4;  // logits: MFMA column (key) and k-quarter
+    const int pg = lane & 3, kgrp = lane >> 2;    // softmax: head and group of kKpl keys
+    constexpr int kKpl = kSK / 16, kDb = kStreamDimBlocks;
     const int64_t nbh = a.B * a.KVH, total = (int64_t)p.tiles * nbh;
     const int64_t item0 = total * blockIdx.x / gridDim.x, item1 = total * (blockIdx.x + 1) / gridDim.x;
     const int64_t NS = a.num_sink, S = a.S;
+    const int KVH = (int)a.KVH;
+    constexpr int kEs = (int)sizeof(T);
 
-    // LDS read offsets.  K row r keeps source piece c at slot c ^ (r & 15), which makes the 16-byte
-    // operand reads conflict free.  V row r keeps piece c at slot c ^ ((r & 7) << 1): the transposing
-    // reads below take 32 bytes from each of four rows, and this puts the rows on different banks.
+    // LDS offsets inside a stage.  K row r keeps source piece c at slot c ^ (r & 15), which makes the
+    // 16-byte operand reads conflict free.  V row r keeps piece c at slot c ^ ((r & 7) << 1): the
+    // transposing reads below take 32 bytes from each of four rows, and this puts the rows on
+    // different banks.
     int kaddr[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) kaddr[ks] = (wave * 16 + key16) * 256 + (((4 * ks + kq) ^ key16) << 4);
@@ -628,15 +655,20 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
     // ds_read_b64_tr_b16 hands lane i of a 16-lane group element [4e + i/4][i%4] (e = 0..3) of the
     // 16 x 4 matrix whose row r is the 8 bytes lane r points at.  With lane r of group q pointing at
     // dims 16 blk + 4 (r%4) .. +3 of key 4q + r/4, lane i receives dim 16 blk + i of keys 4q .. 4q+3:
-    // the A operand.
-    int vt_addr[8];
+    // the A operand.  This wavefront owns kDb blocks of 16 dims (blk = kDb wave ..); the keys of
+    // contraction step ks are 16 rows further per step.
+    int vt_addr[kDb];
     {
         const int r_l = lane & 15, key = 4 * (lane >> 4) + (r_l >> 2);
 #pragma unroll
-        for (int blk = 0; blk < 8; blk++) {
-            vt_addr[blk] = kSK * 256 + (wave * 16 + key) * 256 + 32 * (blk ^ (key & 7)) + 16 * ((r_l & 3) >> 1) + 8 * (r_l & 1);
+        for (int b2 = 0; b2 < kDb; b2++) {
+            vt_addr[b2] = kSK * 256 + key * 256 + 32 * ((kDb * wave + b2) ^ (key & 7)) + 16 * ((r_l & 3) >> 1) + 8 * (r_l & 1);
         }
     }
+    // query block of an item: head g at g * 256; lanes of idle MFMA rows read head 0 (their results are not used)
+    const int q_off = kStreamQ + wave * 2048 + (key16 < G ? key16 : 0) * 256 + kq * 16;
+    float* s_all = reinterpret_cast<float*>(smem + kStreamS);                                   // [2][4][kSK]
+    unsigned char* p_wave = smem + kStreamP + wave * (4 * kSK * 2);                             // [4][kSK] 16-bit
 
     for (int64_t item = item0; item < item1;) {
         const int64_t tile = item / nbh, bh0 = item % nbh;
@@ -662,11 +694,32 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
                     fast_sincos(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
                 }
         }
-        // bit k: key n_wave + k is visible (lanes 0..15 are the sixteen keys)
-        const uint32_t vis_keys = __builtin_amdgcn_readfirstlane((uint32_t)(__builtin_amdgcn_ballot_w64(vis1) & 0xffffull));
-        // rows loaded by this lane: block jb holds rows 4 jb .. 4 jb + 3 of the wavefront's 16, piece lane % 16
+        // Rows of hidden slots may hold anything (their probability is zero, but 0 * NaN is not), so
+        // they are zeroed on the way into the P.V product: masks of this lane's operand keys
+        // 16 ks + 4 kq .. + 3, two 16-bit values per word.
+        uint32_t m01[kKpl], m23[kKpl];
+#pragma unroll
+        for (int half = 0; half < kSK / 64; half++) {
+            const int64_t n = tile * kSK + 64 * half + lane;
+            bool v = false;
+            if (n < NS) v = a.sink_mask[n] == 0;
+            else if (n < NS + S) v = a.mask[n - NS] == 0;
+            else if (n < p.N) v = true;
+            const unsigned long long vis64 = __builtin_amdgcn_ballot_w64(v);
+#pragma unroll
+            for (int k4 = 0; k4 < 4; k4++) {
+                const int ks = 4 * half + k4;
+                const uint32_t vk = (uint32_t)(vis64 >> (16 * k4 + 4 * kq)) & 0xfu;
+                m01[ks] = ((vk & 1u) ? 0x0000ffffu : 0u) | ((vk & 2u) ? 0xffff0000u : 0u);
+                m23[ks] = ((vk & 4u) ? 0x0000ffffu : 0u) | ((vk & 8u) ? 0xffff0000u : 0u);
+            }
+        }
+        // Copies: block jb of a wavefront brings rows 4 jb .. 4 jb + 3 of its 16 (1 KiB: lane i lands at
+        // +16 i, i.e. row 4 jb + i / 16, slot i % 16, and fetches the source piece that belongs there).
+        // seg: 0 sink, 1 cache, 2 the new token (rows past the end repeat it and stay hidden).
         int seg_c[4];
-        int64_t off_c[4];  // element offset inside the (b, kvh) slab of the row's segment
+        uint32_t relk[4], relv[4];  // byte offsets inside the (b, kvh) slab of the row's segment
+        bool cache_only[4];         // every row of the block is a cache slot: one copy with the slab as base
 #pragma unroll
         for (int jb = 0; jb < 4; jb++) {
             const int r = 4 * jb + (lane >> 4);
@@ -674,85 +727,108 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
             int64_t row_off;
             if (n < NS) { seg_c[jb] = 0; row_off = n * a.sink_stride[2]; }
             else if (n < NS + S) { seg_c[jb] = 1; row_off = (n - NS) * a.cache_stride[2]; }
-            else { seg_c[jb] = 2; row_off = 0; }  // the new token; rows past the end repeat it and stay hidden
-            off_c[jb] = row_off + ((lane & 15) << 3);
+            else { seg_c[jb] = 2; row_off = 0; }
+            relk[jb] = (uint32_t)(row_off * kEs) + ((((uint32_t)lane & 15u) ^ ((uint32_t)r & 15u)) << 4);
+            relv[jb] = (uint32_t)(row_off * kEs) + ((((uint32_t)lane & 15u) ^ (((uint32_t)r & 7u) << 1)) << 4);
+            cache_only[jb] = __builtin_amdgcn_ballot_w64(seg_c[jb] == 1) == ~0ull;
         }
-        // rows of one item: eight 16-byte pieces per lane (four K, four V blocks of 1 KiB per wavefront),
-        // loaded one item ahead into registers and written to LDS at the top of the item's iteration
-        auto load_rows = [&](int b, int kvh, u32x4(&kr)[4], u32x4(&vr)[4]) {
-            const T* kseg[3] = {(const T*)a.sink_k + b * a.sink_stride[0] + kvh * a.sink_stride[1],
-                                (const T*)a.cache_k + b * a.cache_stride[0] + kvh * a.cache_stride[1],
-                                (const T*)a.k_new + b * a.kv_new_stride[0] + kvh * a.kv_new_stride[1]};
-            const T* vseg[3] = {(const T*)a.sink_v + b * a.sink_stride[0] + kvh * a.sink_stride[1],
-                                (const T*)a.cache_v + b * a.cache_stride[0] + kvh * a.cache_stride[1],
-                                (const T*)a.v_new + b * a.kv_new_stride[0] + kvh * a.kv_new_stride[1]};
+        // slab pointers of (b, kvh)
+        auto slabs = [&](int b, int kvh, const char* (&kb)[3], const char* (&vb)[3]) {
+            const int64_t o0 = ((int64_t)b * a.sink_stride[0] + (int64_t)kvh * a.sink_stride[1]) * kEs;
+            const int64_t o1 = ((int64_t)b * a.cache_stride[0] + (int64_t)kvh * a.cache_stride[1]) * kEs;
+            const int64_t o2 = ((int64_t)b * a.kv_new_stride[0] + (int64_t)kvh * a.kv_new_stride[1]) * kEs;
+            kb[0] = (const char*)a.sink_k + o0; vb[0] = (const char*)a.sink_v + o0;
+            kb[1] = (const char*)a.cache_k + o1; vb[1] = (const char*)a.cache_v + o1;
+            kb[2] = (const char*)a.k_new + o2; vb[2] = (const char*)a.v_new + o2;
+        };
+        // four copies, at least one per block whatever the segments (the waits below count on that)
+        auto copy_rows = [&](const char* (&base)[3], const uint32_t(&rel)[4], uint32_t dst) {
 #pragma unroll
             for (int jb = 0; jb < 4; jb++) {
-                const T* kb = seg_c[jb] == 0 ? kseg[0] : (seg_c[jb] == 1 ? kseg[1] : kseg[2]);
-                const T* vb = seg_c[jb] == 0 ? vseg[0] : (seg_c[jb] == 1 ? vseg[1] : vseg[2]);
-                kr[jb] = *reinterpret_cast<const u32x4*>(kb + off_c[jb]);
-                vr[jb] = *reinterpret_cast<const u32x4*>(vb + off_c[jb]);
-            }
-        };
-        // A operand: rotated queries of the group's heads (rows >= G are zero)
-        auto load_q = [&](int b, int kvh, uint4(&q)[4]) {
-            const T* qr = (const T*)p.qrot_t + (((int64_t)b * a.H) + kvh * G + key16) * kD;
+                if (cache_only[jb]) {
+                    async_copy16(base[1], rel[jb], dst + jb * 1024);
+                } else {
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++)
-                q[ks] = key16 < G ? *reinterpret_cast<const uint4*>(qr + 32 * ks + 8 * kq) : make_uint4(0, 0, 0, 0);
-        };
-
-        uint4 q_next[4];
-        u32x4 k_next[4], v_next[4];  // plain vectors: an aggregate copied to LDS would be kept in scratch
-        // (batch, kv head) of the item in hand and of the next one, stepped without divisions
-        const int KVH = (int)a.KVH;
-        int b = (int)(bh0 / KVH), kvh = (int)(bh0 % KVH);
-        load_q(b, kvh, q_next);
-        load_rows(b, kvh, k_next, v_next);
-        bool pending = false;
-        int pend_b = 0, pend_kvh = 0;
-        float pend_o = 0.f, pend_m = 0.f, pend_l = 0.f;
-        auto flush = [&]() {
-            if (!pending) return;
-            if (tid < G * kD) {
-                const int g = tid >> 7, d = tid & 127;
-                const int64_t row = ((int64_t)pend_b * a.H + pend_kvh * G + g) * p.tiles + tile;
-                p.part_o[row * kD + d] = pend_o;
-                if (d == 0) {
-                    p.part_ml[row * 2] = pend_m;
-                    p.part_ml[row * 2 + 1] = pend_l;
+                    for (int sgm = 0; sgm < 3; sgm++)
+                        if (seg_c[jb] == sgm) async_copy16(base[sgm], rel[jb], dst + jb * 1024);
                 }
             }
         };
-        for (int64_t bh = bh0; bh < bh1; bh++) {
-            // this wavefront's 16 rows go to LDS (it is their only reader, so no workgroup barrier);
-            // K piece c of row r lands in slot c ^ (r & 15)
+        // K rows and the query block of (b, kvh) into stage `st`: five copies
+        auto copy_kq = [&](int b, int kvh, int st) {
+            const char *kb[3], *vb[3];
+            slabs(b, kvh, kb, vb);
+            copy_rows(kb, relk, lds_base + st * kStreamStage + wave * 4096);
+            const char* qsrc = (const char*)p.qrot_t + ((int64_t)b * a.H + (int64_t)kvh * G) * (kD * kEs);
+            if ((lane >> 4) < G) async_copy16(qsrc, lane * 16, lds_base + kStreamQ + wave * 2048 + st * 1024);
+        };
+        // V rows: four copies
+        auto copy_v = [&](int b, int kvh, int st) {
+            const char *kb[3], *vb[3];
+            slabs(b, kvh, kb, vb);
+            copy_rows(vb, relv, lds_base + st * kStreamStage + kSK * 256 + wave * 4096);
+        };
+
+        int b = (int)(bh0 / KVH), kvh = (int)(bh0 % KVH);
+        // results of the previous item, stored at the top of the next one
+        bool pending = false;
+        int pend_b = 0, pend_kvh = 0;
+        f32x4 pend_acc[kDb];
+        float pend_m = 0.f, pend_l = 0.f, pend_sv[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int jb = 0; jb < 4; jb++) {
-                const int r = 4 * jb + (lane >> 4);
-                *reinterpret_cast<u32x4*>(smem + (wave * 16 + r) * 256 + (((lane & 15) ^ (r & 15)) << 4)) = k_next[jb];
-                *reinterpret_cast<u32x4*>(smem + kSK * 256 + (wave * 16 + r) * 256 + (((lane & 15) ^ ((r & 7) << 1)) << 4)) = v_next[jb];
+        for (int b2 = 0; b2 < kDb; b2++) pend_acc[b2] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // Stores share the counter of the copies and retire in order with them, so all stores of an item
+        // are issued together right after a wait: by the next wait that has to outlast them they are a
+        // whole item old.
+        auto flush = [&]() {
+            if (!pending) return;
+            if (kq == 0 && n_wave + key16 < p.N) {  // with G <= 4 only the lanes of kq == 0 hold logits
+                float* lg = p.logits + (((int64_t)pend_b * KVH + pend_kvh) * p.N + n_wave + key16) * G;
+                if constexpr (G == 4) {
+                    *reinterpret_cast<float4*>(lg) = make_float4(pend_sv[0], pend_sv[1], pend_sv[2], pend_sv[3]);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < G; v++) lg[v] = pend_sv[v];
+                }
             }
-            uint4 qop[4];
+            if (key16 < G) {
+                const int64_t row = ((int64_t)pend_b * a.H + pend_kvh * G + key16) * p.tiles + tile;
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) qop[ks] = q_next[ks];
+                for (int b2 = 0; b2 < kDb; b2++) {
+                    *reinterpret_cast<float4*>(p.part_o + row * kD + 16 * (kDb * wave + b2) + 4 * kq) =
+                        make_float4(pend_acc[b2][0], pend_acc[b2][1], pend_acc[b2][2], pend_acc[b2][3]);
+                }
+            }
+            if (wave == 0 && kgrp == 0 && pg < G) {
+                const int64_t row = ((int64_t)pend_b * a.H + pend_kvh * G + pg) * p.tiles + tile;
+                *reinterpret_cast<float2*>(p.part_ml + row * 2) = make_float2(pend_m, pend_l);
+            }
+        };
+
+        // The waits count copies only.  Loads retire in issue order, so "at most n operations
+        // outstanding" with n younger copies issued after the wanted ones means the wanted ones are done.
+        copy_kq(b, kvh, 0);
+        copy_v(b, kvh, 0);
+        int st = 0;
+        for (int64_t bh = bh0; bh < bh1; bh++) {
             int b_nx = b, kvh_nx = kvh;
-            if (bh + 1 < bh1) {  // the last item of a run loads itself again: cheaper than a branch around the loads
+            if (bh + 1 < bh1) {  // the last item of a run copies itself again: cheaper than a different path
                 kvh_nx = kvh + 1 == KVH ? 0 : kvh + 1;
                 b_nx = kvh + 1 == KVH ? b + 1 : b;
             }
-            load_q(b_nx, kvh_nx, q_next);
-            load_rows(b_nx, kvh_nx, k_next, v_next);
+            // K rows and queries of this item are in LDS (only its four V copies may still be in flight)
+            __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
             flush();
-            const unsigned char* st = smem;
-            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the rows are in LDS
-            __builtin_amdgcn_wave_barrier();
+            copy_kq(b_nx, kvh_nx, st ^ 1);
+            const unsigned char* stage = smem + st * kStreamStage;
 
-            // ---- phase 1: rotate K in registers, logits by MFMA, share them through LDS
+            // ---- rotate K in registers, logits by MFMA, shared through LDS
             {
-                uint4 kraw[4];
+                uint4 kraw[4], qop[4];
 #pragma unroll
-                for (int ks = 0; ks < 4; ks++) kraw[ks] = *reinterpret_cast<const uint4*>(st + kaddr[ks]);
+                for (int ks = 0; ks < 4; ks++) kraw[ks] = *reinterpret_cast<const uint4*>(stage + kaddr[ks]);
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) qop[ks] = *reinterpret_cast<const uint4*>(smem + q_off + st * 1024 + ks * 64);
                 uint4 kop[4];
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++) {
@@ -774,95 +850,90 @@ __global__ void __launch_bounds__(512) decode_stream_kernel(DecodeParams p) {
                 f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int ks = 0; ks < 4; ks++) sacc = Mma16<T>::mma(qop[ks], kop[ks], sacc);
-                // lane holds heads 4 kq + v of key key16
-                const int64_t n = n_wave + key16;
+                // lane holds heads 4 kq + v of key key16: with G <= 4 only the lanes of kq == 0 hold heads
 #pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    const int g = 4 * kq + v;
-                    if (g < G) {
-                        const float sv = vis1 ? sacc[v] * p.scale_log2 : -INFINITY;
-                        s_wave[key16 * 8 + g] = sv;
-                        if (n < p.N) p.logits[(((int64_t)b * KVH + kvh) * p.N + n) * G + g] = sv;
+                for (int v = 0; v < 4; v++) pend_sv[v] = vis1 ? sacc[v] * p.scale_log2 : -INFINITY;
+                if (kq == 0) {
+#pragma unroll
+                    for (int v = 0; v < G; v++) s_all[(st * 4 + v) * kSK + wave * 16 + key16] = pend_sv[v];
+                }
+            }
+            // this wavefront's V rows of the item have landed (younger: the five copies of the next item's K
+            // rows and queries and, after the first item, the stores of flush()) and its logits are
+            // in LDS
+            __builtin_amdgcn_s_waitcnt(0x0070 | (6 + kDb));  // vmcnt(5 copies + 1 + kDb stores), lgkmcnt(0)
+            __builtin_amdgcn_s_barrier();
+            // every wavefront is past the previous item: its V stage can be refilled
+            copy_v(b_nx, kvh_nx, st ^ 1);
+
+            // ---- softmax over the tile's keys, done by every wavefront: lane = (head, kKpl keys)
+            float m_t, l_t;
+            {
+                float x[kKpl];
+#pragma unroll
+                for (int e = 0; e < kKpl; e += 4) {
+                    float4 x4 = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+                    if (pg < G) x4 = *reinterpret_cast<const float4*>(s_all + (st * 4 + pg) * kSK + kKpl * kgrp + e);
+                    x[e] = x4.x; x[e + 1] = x4.y; x[e + 2] = x4.z; x[e + 3] = x4.w;
+                }
+                float mloc = x[0];
+#pragma unroll
+                for (int e = 1; e < kKpl; e++) mloc = fmaxf(mloc, x[e]);
+                const float m = mod4_max(mloc);
+                const float ms = m == -INFINITY ? 0.f : m;
+                float lloc = 0.f;
+#pragma unroll
+                for (int e = 0; e < kKpl; e += 4) {
+                    const float e0 = __builtin_amdgcn_exp2f(x[e] - ms), e1 = __builtin_amdgcn_exp2f(x[e + 1] - ms);
+                    const float e2 = __builtin_amdgcn_exp2f(x[e + 2] - ms), e3 = __builtin_amdgcn_exp2f(x[e + 3] - ms);
+                    lloc += (e0 + e1) + (e2 + e3);
+                    // probabilities in the tensor dtype, [head][kSK keys] (hidden keys and idle lanes: 0)
+                    *reinterpret_cast<uint2*>(p_wave + pg * (kSK * 2) + (kKpl * kgrp + e) * 2) =
+                        make_uint2(Mma16<T>::pack2(e0, e1), Mma16<T>::pack2(e2, e3));
+                }
+                m_t = m;
+                l_t = mod4_sum(lloc);
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+            __builtin_amdgcn_wave_barrier();
+            // ---- weighted V sum on the matrix pipe: this wavefront's dims over all keys of the tile.  Lane
+            //      16 q + g (g < G) ends up with dims 16 (kDb wave + b2) + 4 q .. + 3 of head g.
+            f32x4 acc[kDb];
+#pragma unroll
+            for (int b2 = 0; b2 < kDb; b2++) acc[b2] = f32x4{0.f, 0.f, 0.f, 0.f};
+            {
+                const uint32_t vbase = lds_base + st * kStreamStage;
+#pragma unroll
+                for (int ks = 0; ks < kKpl; ks++) {
+                    uint2 pb = make_uint2(0u, 0u);
+                    if (key16 < G) pb = *reinterpret_cast<const uint2*>(p_wave + key16 * (kSK * 2) + ks * 32 + kq * 8);
+#pragma unroll
+                    for (int b2 = 0; b2 < kDb; b2++) {
+                        const s16x4_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(vbase + vt_addr[b2] + ks * 4096));
+                        uint2 av = __builtin_bit_cast(uint2, va);
+                        av.x &= m01[ks];
+                        av.y &= m23[ks];
+                        acc[b2] = Mma16<T>::mma_k16(av, pb, acc[b2]);
                     }
                 }
             }
-            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront's LDS writes are done
-            __builtin_amdgcn_wave_barrier();
-            // ---- phase 2a: softmax of the wavefront's 16 keys, one (key, head) per lane
-            {
-                const float sv = pg < G ? s_wave[pkey * 8 + pg] : -INFINITY;
-                // all-reduce over the 16 keys of a head: lanes pg, pg + 4, ... of every 16-lane row, then the rows
-                float m = sv;
-                m = fmaxf(m, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(m), 0x124, 0xF, 0xF, true)));  // row_ror:4
-                m = fmaxf(m, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(m), 0x128, 0xF, 0xF, true)));  // row_ror:8
-                m = rows4_max(m);
-                const float pe = __builtin_amdgcn_exp2f(sv - (m == -INFINITY ? 0.f : m));  // hidden keys and idle lanes: 0
-                float l = pe;
-                l += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(l), 0x124, 0xF, 0xF, true));
-                l += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(l), 0x128, 0xF, 0xF, true));
-                l = rows4_sum(l);
-                __builtin_amdgcn_wave_barrier();      // every lane has read its logit
-                // probabilities in the tensor dtype, [head][16 keys] (hidden keys: 0)
-                reinterpret_cast<unsigned short*>(s_wave)[pg * 16 + pkey] = (unsigned short)Mma16<T>::pack2(pe, 0.f);
-                if (pkey == 0 && pg < G) {
-                    red_ml[(wave * G + pg) * 2] = m;
-                    red_ml[(wave * G + pg) * 2 + 1] = l;
-                }
-            }
-            __builtin_amdgcn_s_waitcnt(0xC07F);
-            __builtin_amdgcn_wave_barrier();
-            // ---- phase 2b: weighted V sum on the matrix pipe.  Lane 16 q + g (g < G) ends up with
-            //      dims 16 blk + 4 q .. + 3 of head g.  Rows of hidden slots may hold anything (their
-            //      probability is zero, but 0 * NaN is not), so they are zeroed on the way in.
-            {
-                const int g = lane & 15, q4 = lane >> 4;
-                uint2 pb = make_uint2(0u, 0u);
-                if (g < G) pb = *reinterpret_cast<const uint2*>(reinterpret_cast<const unsigned char*>(s_wave) + g * 32 + q4 * 8);
-                // this lane's operand pieces are keys 4 q4 .. 4 q4 + 3
-                const uint32_t vk = (vis_keys >> (4 * q4)) & 0xfu;
-                const uint32_t m01 = ((vk & 1u) ? 0x0000ffffu : 0u) | ((vk & 2u) ? 0xffff0000u : 0u);
-                const uint32_t m23 = ((vk & 4u) ? 0x0000ffffu : 0u) | ((vk & 8u) ? 0xffff0000u : 0u);
 #pragma unroll
-                for (int blk = 0; blk < 8; blk++) {
-                    const s16x4_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(lds_base + vt_addr[blk]));
-                    uint2 av = __builtin_bit_cast(uint2, va);
-                    av.x &= m01;
-                    av.y &= m23;
-                    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-                    const f32x4 acc = Mma16<T>::mma_k16(av, pb, zero);
-                    if (g < G)
-                        *reinterpret_cast<float4*>(red_o + (wave * G + g) * kD + 16 * blk + 4 * q4) =
-                            make_float4(acc[0], acc[1], acc[2], acc[3]);
-                }
-            }
-            __syncthreads();
-            // ---- combine the eight wavefronts; the result is stored at the top of the next iteration
-            if (tid < G * kD) {
-                const int g = tid >> 7, d = tid & 127;
-                float M = -INFINITY;
-#pragma unroll
-                for (int w = 0; w < 8; w++) M = fmaxf(M, red_ml[(w * G + g) * 2]);
-                float acc = 0.f, L = 0.f;
-#pragma unroll
-                for (int w = 0; w < 8; w++) {
-                    const float mw = red_ml[(w * G + g) * 2];
-                    const float sc = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - M);
-                    acc = fmaf(red_o[(w * G + g) * kD + d], sc, acc);
-                    L = fmaf(red_ml[(w * G + g) * 2 + 1], sc, L);
-                }
-                pend_o = acc;
-                pend_m = M;
-                pend_l = L;
-            }
+            for (int b2 = 0; b2 < kDb; b2++) pend_acc[b2] = acc[b2];
+            pend_m = m_t;
+            pend_l = l_t;
             pending = true;
             pend_b = b;
             pend_kvh = kvh;
             b = b_nx;
             kvh = kvh_nx;
-            __syncthreads();  // red_* may be overwritten
+            st ^= 1;
         }
         flush();
+        // the repeated copies of the last item must land, and every wavefront be done with the stages,
+        // before the next run of items refills them
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __builtin_amdgcn_s_barrier();
     }
 }
 
@@ -1007,8 +1078,12 @@ __global__ void __launch_bounds__(256) decode_scores_kernel(DecodeParams p, floa
 }
 
 template <typename T, int G>
-int run_decode(const DecodeParams& p, hipStream_t stream) {
+int run_decode(const DecodeParams& p_in, hipStream_t stream) {
+    DecodeParams p = p_in;
     const ckv_attn_args& a = p.a;
+    const bool use_stream =
+        !std::is_same<T, float>::value && G <= 4 && p.shared_pos && stream_offsets_fit(a) && !getenv("CKV_DECODE_OLD");
+    if (use_stream) p.tiles = (int)((p.N + kSK - 1) / kSK);  // the streaming kernel has its own tile size
     {
         StageScope sc(CKV_STAGE_PREP, stream);
         hipLaunchKernelGGL(decode_q_kernel<T>, dim3((unsigned)(a.B * a.H)), dim3(64), 0, stream, p);
@@ -1029,18 +1104,18 @@ int run_decode(const DecodeParams& p, hipStream_t stream) {
             }
             hipLaunchKernelGGL((decode_main_kernel<T, G>), dim3((unsigned)p.tiles, (unsigned)groups), dim3(256), lds,
                                stream, p);
-        } else if (G <= 4 && p.shared_pos && !getenv("CKV_DECODE_OLD")) {
-            // streaming kernel: one workgroup per CU, items dealt out evenly
+        } else if (use_stream) {
+            // streaming kernel: as many workgroups as run at once, items dealt out evenly
             if constexpr (G <= 4) {
-                const int lds_s = stream_lds_bytes(G);
+                const int lds_s = kStreamLds;
                 CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stream_kernel<T, G>),
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds_s));
                 int dev = 0, cus = 0;
                 CKV_HIP_TRY(hipGetDevice(&dev));
                 CKV_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-                int64_t wgs = cus > 0 ? cus : 256;
+                int64_t wgs = (cus > 0 ? cus : 256) * kStreamWgPerCu;
                 if (wgs > p.tiles * nbh) wgs = p.tiles * nbh;
-                hipLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(512), lds_s, stream, p);
+                hipLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads), lds_s, stream, p);
             }
         } else {
             if (lds > 48 * 1024) {
@@ -1106,8 +1181,10 @@ bool decode_supported(const ckv_attn_args& a) {
     return true;
 }
 
+constexpr int64_t kMinTile = kSK < kTK ? kSK : kTK;  // the partial results are sized for the smaller tile
+
 int64_t decode_workspace_bytes(int64_t B, int64_t H, int64_t KVH, int64_t num_sink, int64_t S) {
-    const int64_t N = num_sink + S + 1, tiles = (N + kTK - 1) / kTK, G = H / KVH;
+    const int64_t N = num_sink + S + 1, tiles = (N + kMinTile - 1) / kMinTile, G = H / KVH;
     return 2 * align_up(B * H * kD * 4, 256) + align_up(B * KVH * N * G * 4, 256) + align_up(B * H * tiles * 2 * 4, 256) +
            align_up(B * H * tiles * kD * 4, 256) + align_up(B * H * 4, 256);
 }
@@ -1122,8 +1199,9 @@ int launch_decode(const ckv_attn_args& a, hipStream_t stream) {
     p.qrot = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * kD * 4, 256);
     p.qrot_t = w; w += align_up(a.B * a.H * kD * 4, 256);
     p.logits = reinterpret_cast<float*>(w); w += align_up(a.B * a.KVH * p.N * G * 4, 256);
-    p.part_ml = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * p.tiles * 2 * 4, 256);
-    p.part_o = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * p.tiles * kD * 4, 256);
+    const int64_t tiles_max = (p.N + kMinTile - 1) / kMinTile;
+    p.part_ml = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * tiles_max * 2 * 4, 256);
+    p.part_o = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * tiles_max * kD * 4, 256);
     p.lse2 = reinterpret_cast<float*>(w);
     p.shared_pos = a.sink_pos_stride[0] == 0 && a.sink_pos_stride[1] == 0 && a.pos_stride[0] == 0 && a.pos_stride[1] == 0;
     p.scale_log2 = a.scale * 1.4426950408889634f;

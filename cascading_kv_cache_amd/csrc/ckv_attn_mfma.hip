@@ -327,31 +327,6 @@ struct FwdParams {
     int n_qt, xcd_aware;  // query tiles per kv head; 1-D XCD-aware block order
 };
 
-__device__ inline const void* uniform_ptr(const void* p) {
-    const uint64_t v = reinterpret_cast<uint64_t>(p);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo);
-}
-
-// Asynchronous global -> LDS copy of one 16-byte piece per lane (gfx950 global_load_lds_dwordx4):
-// the wavefront's 64 pieces land contiguously at LDS byte address `lds_wave_base` (uniform, goes
-// to M0), lane i at +16*i; the source is `sbase` (uniform, SGPR pair) + `voff` (per lane).
-// Inline assembly on purpose: the compiler keeps no scoreboard entry for the copy, so it cannot
-// force it to complete before unrelated LDS reads; completion is awaited explicitly with
-// s_waitcnt vmcnt(n) (copies retire in issue order).
-__device__ inline void async_copy16(const void* sbase, uint32_t voff, uint32_t lds_wave_base) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(__builtin_amdgcn_readfirstlane(lds_wave_base)), "v"(voff), "s"(uniform_ptr(sbase))
-                 : "memory");
-}
-
-__device__ inline uint32_t lds_address(const void* p) {
-    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)p;
-}
-
-
 // LDS tile of 256-byte rows taken from a row-major matrix (the query tile of the column pass): unpadded
 // (the async copy writes 1 KiB per wavefront contiguously); bank conflicts are avoided by XOR-swizzling
 // the 16-byte piece index with the row: piece c of row r lives at r*256 + ((c ^ (r & 15)) << 4)
