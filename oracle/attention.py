@@ -11,7 +11,8 @@ Follows the reference's eager path so that rounding happens at the same points:
 Pinned by tests/test_oracle_attention.py: dense masked softmax attention over the valid keys
 (the oracle of cascade/models/test.py:196-219), plain causal attention for an empty cache,
 "chunked with cache == dense single shot" when the stream fits one cascade
-(cascade/models/test.py:123-165), the closed forms of the score sums, and torch's own
+(cascade/models/test.py:123-165), dense attention with per-head positions for the original-position
+mode (cascade_attention.py:141-144, 161-164), the closed forms of the score sums, and torch's own
 mean/amax/median for the head reduction.  The bf16 rounding ORDER is not pinned by any
 reference test (parity unpinned for that aspect); it is fixed here by using the same torch ops.
 """
@@ -76,12 +77,13 @@ class OracleCascadeAttention:
     """One attention layer over an :class:`OracleCache` (projections excluded)."""
 
     def __init__(self, num_heads, num_kv_heads, head_dim, rope_theta=500000.0, head_reduction="mean",
-                 homogeneous_heads=False):
+                 homogeneous_heads=False, do_og_pos=False):
         self.num_heads, self.num_kv_heads, self.head_dim = num_heads, num_kv_heads, head_dim
         self.groups = num_heads // num_kv_heads
         self.rope_theta = rope_theta
         self.head_reduction = head_reduction
         self.homogeneous_heads = homogeneous_heads
+        self.do_og_pos = do_og_pos  # cached keys rotated per (batch, head) at their original token index
         self.last_q_size = None
         self.query_pos = None
         self.causal_mask = None
@@ -97,11 +99,13 @@ class OracleCascadeAttention:
         q_len = query_states.size(2)
         first_it = int(cache.seen_tokens) == 0  # cascade_attention.py:114
 
-        sink_k, sink_v, sink_pos, sink_mask, k_states, v_states, key_pos, key_mask, _og = cache.get_vals()
+        sink_k, sink_v, sink_pos, sink_mask, k_states, v_states, key_pos, key_mask, og_pos = cache.get_vals()
 
         max_pos = 0
         if first_it:  # cascade_attention.py:120-123
             self.query_pos = torch.arange(0, q_len, dtype=torch.long).view(1, -1)
+        elif self.do_og_pos:  # cascade_attention.py:141-144
+            max_pos = torch.cat((sink_pos.amax().view(1), og_pos.amax().view(1)), dim=-1).amax() + 1
         else:  # cascade_attention.py:145-148
             max_pos = torch.cat((sink_pos.amax().view(1), key_pos.amax().view(1)), dim=-1).amax() + 1
         query_pos = self.query_pos[:, :q_len] + max_pos  # cascade_attention.py:150
@@ -110,7 +114,11 @@ class OracleCascadeAttention:
         query_states = self.rope(query_states, query_pos)
         key_states_pos = self.rope(key_states, query_pos)
         sink_k = self.rope(sink_k, sink_pos)
-        k_states = self.rope(k_states, key_pos)
+        if self.do_og_pos:  # cascade_attention.py:161-164
+            b, h, s, d = k_states.size()
+            k_states = self.rope(k_states.view(b * h, 1, s, d), og_pos.view(b * h, -1)).view(b, h, s, d)
+        else:
+            k_states = self.rope(k_states, key_pos)
 
         g = self.groups
         key_states_pos = repeat_kv(key_states_pos, g)

@@ -54,12 +54,12 @@ def assert_scores_close(got, want, dtype, what):
 
 
 def run_teacher_forced(B, H, KVH, D, NS, W, C, Q, chunks, dtype, seed, reduction="mean", homogeneous=False,
-                       eager=True, theta=5e5, std=1.0, q_last=None):
+                       eager=True, theta=5e5, std=1.0, q_last=None, do_og_pos=False):
     from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
 
     gpu, cpu = make_pair(B, KVH, D, NS, W, C, dtype, eager=eager, reduction=reduction)
     layer = OracleCascadeAttention(H, KVH, D, rope_theta=theta, head_reduction=reduction,
-                                   homogeneous_heads=homogeneous)
+                                   homogeneous_heads=homogeneous, do_og_pos=do_og_pos)
     inv_freq = default_inv_freq(D, theta, "cuda:0")
     gen = torch.Generator().manual_seed(seed)
     flips = 0
@@ -71,7 +71,7 @@ def run_teacher_forced(B, H, KVH, D, NS, W, C, Q, chunks, dtype, seed, reduction
         v = (torch.randn(B, KVH, qn, D, generator=gen) * std).to(dtype)
         push_state(gpu, cpu)
         out_g, new_g = cascade_attention(q.cuda(), k.cuda(), v.cuda(), gpu, 0, inv_freq, head_reduction=reduction,
-                                         homogeneous_heads=homogeneous, update_cache=False)
+                                         homogeneous_heads=homogeneous, update_cache=False, do_og_pos=do_og_pos)
         gpu.update(k.cuda(), v.cuda(), 0, score_states=new_g)
         out_c = layer.forward(q, k, v, cpu)
         torch.cuda.synchronize()
@@ -213,6 +213,23 @@ def test_decode_streaming_many_items(H, KVH, dtype, fill):
         assert_scores_close(new_g, layer.last_new_scores[:, :KVH], dtype, f"step {step} new-token scores")
         for name in META:
             assert torch.equal(getattr(gpu, name)[0].cpu(), getattr(cpu, name)), f"step {step}: {name}"
+
+
+@pytest.mark.parametrize("dtype,D,H,KVH,Q,q_last", [
+    (torch.float32, 32, 4, 2, 10, 3),       # fp32-math kernels
+    (torch.bfloat16, 128, 8, 2, 64, 17),    # matrix-core prefill, key positions per (batch, kv head)
+    (torch.float16, 128, 4, 4, 40, None),
+    (torch.bfloat16, 128, 8, 2, 1, None),   # single-token steps, positions per (batch, kv head)
+    (torch.float16, 128, 7, 1, 1, None),
+])
+def test_original_position_mode(dtype, D, H, KVH, Q, q_last):
+    """cascade_attention.py:141-144, 161-164 (do_og_pos): cached keys are rotated per (batch, head) at the index
+    of the token a slot holds; without eager fill the heads soon keep different tokens."""
+    chunks = 40 if Q == 1 else 8
+    flips, compared = run_teacher_forced(2, H, KVH, D, 4, 16, 2, Q, chunks, dtype, seed=21, eager=False, std=0.7,
+                                         q_last=q_last, do_og_pos=True)
+    if dtype == torch.float32:
+        assert flips == 0, f"{flips} of {compared} slots differ in og_pos"
 
 
 @pytest.mark.parametrize("do_og_pos", [False, True])

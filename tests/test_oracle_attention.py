@@ -90,6 +90,35 @@ def test_every_chunk_matches_dense_attention_over_valid_keys(C, eager):
         assert torch.allclose(out.double(), ref, atol=2e-5), f"chunk {step}"
 
 
+def test_original_position_mode_matches_dense_attention_with_per_head_positions():
+    """cascade_attention.py:141-144, 161-164 (do_og_pos): cached keys are rotated per (batch, head) at the
+    1-based index of the token each slot holds, sinks at their slot number, the chunk one past the
+    largest index in the cache.  Scores differ per head, so the heads keep different tokens."""
+    g = torch.Generator().manual_seed(7)
+    B, H, KVH, D, NS, W, C, Q, theta = 2, 4, 2, 8, 2, 4, 2, 3, 10000.0
+    cache = OracleCache(window_length=W, num_sink_tokens=NS, max_batch_size=B, heads=KVH, dim=D, max_seq_len=W * C,
+                        dtype=torch.float32, eager_fill=False)
+    attn = OracleCascadeAttention(H, KVH, D, rope_theta=theta, do_og_pos=True)
+    differed = False
+    for step in range(14):
+        q, k, v = rand_chunk(g, B, H, KVH, Q, D)
+        sink_k, sink_v, sink_pos, sink_mask, ck, cv, _key_pos, key_mask, og_pos = cache.get_vals()
+        sv, cvalid = ~sink_mask[0, 0], ~key_mask[0, 0]
+        differed = differed or not torch.equal(og_pos[0, 0, cvalid], og_pos[0, 1, cvalid])
+        q_pos = torch.arange(Q) + (0 if step == 0 else max(int(sink_pos.max()), int(og_pos.max())) + 1)
+        keys = torch.cat((rope_complex(sink_k[:, :, sv], sink_pos[0, sv], theta),
+                          rope_complex(ck[:, :, cvalid], og_pos[:, :, cvalid], theta),
+                          rope_complex(k, q_pos, theta)), dim=2).repeat_interleave(H // KVH, dim=1)
+        vals = torch.cat((sink_v[:, :, sv], cv[:, :, cvalid], v), dim=2).double().repeat_interleave(H // KVH, dim=1)
+        n_prev = keys.size(2) - Q
+        logits = rope_complex(q, q_pos, theta) @ keys.transpose(-1, -2) / math.sqrt(D)
+        logits[..., n_prev:] = logits[..., n_prev:].masked_fill(torch.ones(Q, Q, dtype=torch.bool).triu(1), float("-inf"))
+        ref = torch.softmax(logits, dim=-1) @ vals
+        out = attn.forward(q, k, v, cache)
+        assert torch.allclose(out.double(), ref, atol=2e-5), f"chunk {step}"
+    assert differed, "the stream never made two heads keep different tokens: the per-head positions were not exercised"
+
+
 def test_chunked_with_cache_equals_dense_single_shot():
     """cascade/models/test.py:123-165: while the whole stream fits (C == 1), chunked attention
     through the cache equals ordinary causal attention with ordinary positions."""
