@@ -116,19 +116,19 @@ __device__ inline int find_segment(const StageParams& p, int64_t n, int64_t& loc
 __device__ __host__ inline int k_image_off(int r, int c) { return (c >> 1) * 2048 + (c & 1) * 1024 + r * 16; }
 __device__ __host__ inline int v_image_off(int d, int c) { return (c >> 1) * 4096 + (c & 1) * 2048 + d * 16; }
 
-// grid (n_pad/64, splits); 256 threads: thread = (key = tid/4, quarter = tid%4) owns rotation pairs
-// j = 16*quarter .. 16*quarter+15, i.e. elements [16q,16q+16) and [64+16q, 64+16q+16) of its row.
+// One block of 256 threads stages key tile `tile_i` for the (b, kvh) units split_i, split_i + n_split, ...:
+// thread = (key = tid/4, quarter = tid%4) owns rotation pairs j = 16*quarter .. 16*quarter+15, i.e.
+// elements [16q,16q+16) and [64+16q, 64+16q+16) of its row.
 template <typename T>
-__global__ void __launch_bounds__(256) stage_keys_kernel(StageParams p) {
-    __shared__ T v_lds[kBN][kD + 2];
+__device__ inline void stage_keys_block(const StageParams& p, int tile_i, int split_i, int n_split, T (*v_lds)[kD + 2]) {
     const int tid = threadIdx.x;
     const int key = tid >> 2, quarter = tid & 3;
-    const int64_t tile = blockIdx.x;
+    const int64_t tile = tile_i;
     const int64_t n = tile * kBN + key;
     int64_t local = 0;
     const int sidx = n < p.n ? find_segment(p, n, local) : -1;
 
-    if (blockIdx.y == 0 && tid < kBN) {  // visibility word of this tile
+    if (split_i == 0 && tid < kBN) {  // visibility word of this tile
         const int64_t nn = tile * kBN + tid;
         bool vis = nn < p.n;
         if (vis) {
@@ -152,7 +152,7 @@ __global__ void __launch_bounds__(256) stage_keys_kernel(StageParams p) {
         }
     }
     const int64_t nbh = p.B * p.KVH;
-    for (int64_t bh = blockIdx.y; bh < nbh; bh += gridDim.y) {
+    for (int64_t bh = split_i; bh < nbh; bh += n_split) {
         const int64_t b = bh / p.KVH, kvh = bh % p.KVH;
         uint4 lo[2], hi[2], vlo[2], vhi[2];
         lo[0] = lo[1] = hi[0] = hi[1] = vlo[0] = vlo[1] = vhi[0] = vhi[1] = make_uint4(0, 0, 0, 0);
@@ -253,10 +253,11 @@ struct StageQParams {
 };
 
 // thread = (position m, quarter of the rotation pairs); the cos/sin of the position are computed once
-// and reused for the batch x head rows of the block's share (blockIdx.y of gridDim.y)
+// and reused for the batch x head rows share_i, share_i + n_share, ...; a block of 256 threads covers
+// positions 64 blk .. 64 blk + 63
 template <typename T>
-__global__ void __launch_bounds__(64) stage_q_kernel(StageQParams p) {
-    const int64_t idx = (int64_t)blockIdx.x * 64 + threadIdx.x;
+__device__ inline void stage_q_block(const StageQParams& p, int blk, int share_i, int n_share) {
+    const int64_t idx = (int64_t)blk * 256 + threadIdx.x;
     const int64_t m = idx >> 2;
     const int quarter = idx & 3;
     if (m >= p.Q) return;
@@ -271,7 +272,7 @@ __global__ void __launch_bounds__(64) stage_q_kernel(StageQParams p) {
         }
     }
     const int64_t nbh = p.rows / p.Q;
-    for (int64_t bh = blockIdx.y; bh < nbh; bh += gridDim.y) {
+    for (int64_t bh = share_i; bh < nbh; bh += n_share) {
         const int64_t b = bh / p.H, h = bh % p.H;
         const T* src = (const T*)p.q + b * p.stride[0] + h * p.stride[1] + m * p.stride[2];
         T lo[16], hi[16];
@@ -306,6 +307,24 @@ __global__ void __launch_bounds__(64) stage_q_kernel(StageQParams p) {
         *reinterpret_cast<uint4*>(dst + 16 * quarter + 8) = reinterpret_cast<uint4*>(lo)[1];
         *reinterpret_cast<uint4*>(dst + 64 + 16 * quarter) = reinterpret_cast<uint4*>(hi)[0];
         *reinterpret_cast<uint4*>(dst + 64 + 16 * quarter + 8) = reinterpret_cast<uint4*>(hi)[1];
+    }
+}
+
+// One launch stages queries and keys: the two are independent, and side by side the shorter one costs
+// nothing.  1-D grid: the query blocks (q_bx x q_by) first, then the key blocks (k_bx x k_by).
+struct StageGrid {
+    int q_bx, q_by, k_bx, k_by;
+};
+template <typename T>
+__global__ void __launch_bounds__(256) stage_kernel(StageParams sp, StageQParams sq, StageGrid g) {
+    __shared__ T v_lds[kBN][kD + 2];
+    const int nq = g.q_bx * g.q_by;
+    int id = blockIdx.x;
+    if (id < nq) {
+        stage_q_block<T>(sq, id % g.q_bx, id / g.q_bx, g.q_by);
+    } else {
+        id -= nq;
+        stage_keys_block<T>(sp, id % g.k_bx, id / g.k_bx, g.k_by, v_lds);
     }
 }
 
@@ -1068,9 +1087,6 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         const int64_t nbh = mp.B * mp.KVH;
         int64_t splits = mp.shared_pos ? (nbh < 4 ? nbh : 4) : nbh;
         if (splits > 65535) splits = 65535;
-        hipLaunchKernelGGL(stage_keys_kernel<T>, dim3((unsigned)(n_pad / kBN), (unsigned)splits), dim3(256), 0, stream,
-                           sp);
-        CKV_HIP_TRY(hipGetLastError());
         StageQParams sq;
         sq.q = mp.q;
         for (int j = 0; j < 4; j++) sq.stride[j] = mp.q_stride[j];
@@ -1084,13 +1100,17 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         sq.vec = mp.q_stride[3] == 1 && reinterpret_cast<uintptr_t>(mp.q) % 16 == 0 && mp.q_stride[0] % 8 == 0 &&
                  mp.q_stride[1] % 8 == 0 && mp.q_stride[2] % 8 == 0;
         {
-            // enough blocks to fill the chip; the rest of batch x heads is looped over inside, sharing cos/sin
-            // one wavefront per block; about 2048 blocks, the rest of batch x heads looped over inside
-            const int64_t bx = (mp.Q * 4 + 63) / 64, nbh_q = mp.B * mp.H;
-            int64_t by = (2048 + bx - 1) / bx;
+            // about 1024 query blocks (64 positions each); the rest of batch x heads is looped over inside,
+            // sharing cos/sin
+            const int64_t bx = (mp.Q + 63) / 64, nbh_q = mp.B * mp.H;
+            int64_t by = (1024 + bx - 1) / bx;
             if (by > nbh_q) by = nbh_q;
             if (by < 1) by = 1;
-            hipLaunchKernelGGL(stage_q_kernel<T>, dim3((unsigned)bx, (unsigned)by), dim3(64), 0, stream, sq);
+            StageGrid g;
+            g.q_bx = (int)bx; g.q_by = (int)by; g.k_bx = (int)(n_pad / kBN); g.k_by = (int)splits;
+            const int64_t blocks = bx * by + (n_pad / kBN) * splits;
+            if (blocks > 0x7fffffff) return CKV_ERR_UNSUPPORTED;
+            hipLaunchKernelGGL(stage_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, sp, sq, g);
         }
         CKV_HIP_TRY(hipGetLastError());
     }
