@@ -595,7 +595,8 @@ constexpr int kStreamDimBlocks = 8 / kStreamWaves;  // 16-dim blocks of the outp
 constexpr int kStreamStage = 2 * kSK * 256;       // K rows then V rows of one tile (16-bit, 256 B per row)
 // two stages | per wavefront two 1 KiB query blocks | two [4 heads][kSK keys] logit planes | per wavefront [4][kSK] probabilities
 constexpr int kStreamQ = 2 * kStreamStage, kStreamS = kStreamQ + kStreamWaves * 2048, kStreamP = kStreamS + 2 * 4 * kSK * 4;
-constexpr int kStreamLds = kStreamP + kStreamWaves * 4 * kSK * 2;
+constexpr int kStreamPPitch = kSK * 2 + 32;        // bytes per head row of the probabilities: the pad puts the four heads on different banks
+constexpr int kStreamLds = kStreamP + kStreamWaves * 4 * kStreamPPitch;
 
 // sum / max over the four 16-lane rows of a wavefront (lanes l, l^16, l^32, l^48)
 __device__ inline float rows4_sum(float x) {
@@ -665,10 +666,12 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
             vt_addr[b2] = kSK * 256 + key * 256 + 32 * ((kDb * wave + b2) ^ (key & 7)) + 16 * ((r_l & 3) >> 1) + 8 * (r_l & 1);
         }
     }
-    // query block of an item: head g at g * 256; lanes of idle MFMA rows read head 0 (their results are not used)
-    const int q_off = kStreamQ + wave * 2048 + (key16 < G ? key16 : 0) * 256 + kq * 16;
+    // query block of an item: head g at g * 256, its 16-byte piece c in slot c ^ g (the heads' rows would
+    // otherwise sit on the same banks); lanes of idle MFMA rows read head 0 (their results are not used)
+    const int q_row = key16 < G ? key16 : 0;
+    const int q_off = kStreamQ + wave * 2048 + q_row * 256 + ((kq ^ q_row) << 4);
     float* s_all = reinterpret_cast<float*>(smem + kStreamS);                                   // [2][4][kSK]
-    unsigned char* p_wave = smem + kStreamP + wave * (4 * kSK * 2);                             // [4][kSK] 16-bit
+    unsigned char* p_wave = smem + kStreamP + wave * (4 * kStreamPPitch);                       // [4][kSK] 16-bit, padded rows
 
     for (int64_t item = item0; item < item1;) {
         const int64_t tile = item / nbh, bh0 = item % nbh;
@@ -760,7 +763,10 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
             slabs(b, kvh, kb, vb);
             copy_rows(kb, relk, lds_base + st * kStreamStage + wave * 4096);
             const char* qsrc = (const char*)p.qrot_t + ((int64_t)b * a.H + (int64_t)kvh * G) * (kD * kEs);
-            if ((lane >> 4) < G) async_copy16(qsrc, lane * 16, lds_base + kStreamQ + wave * 2048 + st * 1024);
+            // lane i fills slot i % 16 of head i / 16 with the piece that belongs there
+            if ((lane >> 4) < G)
+                async_copy16(qsrc, (lane >> 4) * 256 + (((lane & 15) ^ (lane >> 4)) << 4),
+                             lds_base + kStreamQ + wave * 2048 + st * 1024);
         };
         // V rows: four copies
         auto copy_v = [&](int b, int kvh, int st) {
@@ -888,7 +894,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                     const float e2 = __builtin_amdgcn_exp2f(x[e + 2] - ms), e3 = __builtin_amdgcn_exp2f(x[e + 3] - ms);
                     lloc += (e0 + e1) + (e2 + e3);
                     // probabilities in the tensor dtype, [head][kSK keys] (hidden keys and idle lanes: 0)
-                    *reinterpret_cast<uint2*>(p_wave + pg * (kSK * 2) + (kKpl * kgrp + e) * 2) =
+                    *reinterpret_cast<uint2*>(p_wave + pg * kStreamPPitch + (kKpl * kgrp + e) * 2) =
                         make_uint2(Mma16<T>::pack2(e0, e1), Mma16<T>::pack2(e2, e3));
                 }
                 m_t = m;
@@ -906,7 +912,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
 #pragma unroll
                 for (int ks = 0; ks < kKpl; ks++) {
                     uint2 pb = make_uint2(0u, 0u);
-                    if (key16 < G) pb = *reinterpret_cast<const uint2*>(p_wave + key16 * (kSK * 2) + ks * 32 + kq * 8);
+                    if (key16 < G) pb = *reinterpret_cast<const uint2*>(p_wave + key16 * kStreamPPitch + ks * 32 + kq * 8);
 #pragma unroll
                     for (int b2 = 0; b2 < kDb; b2++) {
                         const s16x4_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
