@@ -52,6 +52,10 @@ struct Mma<__hip_bfloat16> {
         const uint32_t u = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
         return __uint_as_float(u << 16);
     }
+    // acc + both halves of a packed pair (one v_dot2c with a pair of ones)
+    __device__ static float sum2(uint32_t w, float acc) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), __builtin_bit_cast(bf16x2, 0x3f803f80u), acc, false);
+    }
 };
 template <>
 struct Mma<__half> {
@@ -64,6 +68,9 @@ struct Mma<__half> {
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
     }
     __device__ static float round1(float v) { return (float)(_Float16)v; }
+    __device__ static float sum2(uint32_t w, float acc) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), __builtin_bit_cast(f16x2, 0x3c003c00u), acc, false);
+    }
 };
 
 // position of key `k` (0..63) of a tile inside a V^T row: the PV contraction step s covers keys
@@ -439,7 +446,13 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
         for (int v = 0; v < 16; v++) oacc[dt][v] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;  // l_run: partial over this lane's keys; halves are added at the end
+    // m_ref: the reference the row's logits and sums are relative to; m_run: running maximum relative to it
+    // (-inf until the row has seen a key); l_run: partial over this lane's keys, halves are added at the end
+    float m_ref = 0.f, m_run = -INFINITY, l_run = 0.f;
+    f32x16 cinit;  // -m_ref in every element: what the matrix pipe starts a tile's logits from
+#pragma unroll
+    for (int v = 0; v < 16; v++) cinit[v] = 0.f;
+    constexpr float kShiftAt = 10.f;  // probabilities stay below 2^10 between two moves of the reference
 
     // ---- LDS byte offset of this lane's operand pieces inside the stage being read (pieces of later
     // contraction steps / row blocks are at compile-time distances); moved from stage to stage in place.
@@ -478,9 +491,7 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     // logits of the K tile k_base points at: s[ks][v] = key 32ks + 8(v/4) + 4half + v%4, query column col
     auto qk = [&](f32x16(&s)[2]) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) s[ks][v] = 0.f;
+        for (int ks = 0; ks < 2; ks++) s[ks] = cinit;
 #pragma unroll
         for (int kk = 0; kk < 8; kk++) {
 #pragma unroll
@@ -557,38 +568,45 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
         const int v_wr = v_rd == 0 ? kVStages - 1 : v_rd - 1;   // (v_rd + 3) % 4
         const int k_wr = k_rd == 0 ? kKStages - 1 : k_rd - 1;   // (k_rd + 2) % 3
         if (entry < 0) mask_tile(entry, s_cur);
-        rescale();  // tile i-2 is in the accumulator; tile i-1, scaled for the newer maximum, is added below
+        rescale();  // tile i-2 is in the accumulator; tile i-1, scaled for the newer reference, is added below
         auto operand = [&](int k) -> uint4 {
             if (k >= kQk0) {
-                const int j = k - kQk0;  // K piece (kk, ks) = (j / 2, j % 2)
-                return k_piece(j >> 1, j & 1);
+                const int j = k - kQk0;  // K piece (kk, ks) = (j % 8, j / 8): one 32-key block after the other
+                return k_piece(j & 7, j >> 3);
             }
             return v_piece(k >> 2, k & 3);
         };
         uint4 ops[kSlots];
+        if (kPV) {
 #pragma unroll
-        for (int k = 0; k < kAhead; k++) ops[k] = kPV ? pre[k] : operand(k);
+            for (int k = 0; k < kAhead; k++) ops[k] = pre[k];
+        }
         float mx[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-        float m_use = 0.f, rs0 = 0.f, rs1 = 0.f;
+        float shift = 0.f, rs = 0.f;
+        // Softmax schedule.  With P.V: slots 0..7 running maxima (the last one also reduces them), then one
+        // pair of probabilities per slot: the first 32-key block of the tile is consumed by slot 15 and the
+        // second by slot 23, just before the matrix pipe starts to overwrite them with the next tile's
+        // logits (slots 16..23 and 24..31), so one set of logit registers serves both tiles.
         constexpr int kMaxSlots = kPV ? 8 : 4;             // slots with running maxima
         constexpr int kMaxPer = 32 / kMaxSlots;            // logits per such slot
-        constexpr int kExpFirst = kMaxSlots + 1;           // first slot with probabilities
+        constexpr int kExpFirst = kMaxSlots;               // first slot with probabilities
         constexpr int kExpPer = kPV ? 1 : 2;               // pairs per slot
         float q0[kExpPer], q1[kExpPer];                    // exponentials of the previous slot, packed one slot later
         int raw_entry = 0;
-#pragma unroll
-        for (int k = 0; k < kSlots; k++) {
-            if (k + kAhead < kSlots) ops[k + kAhead] = operand(k + kAhead);
+        bool moved = true;                                 // some row of the wavefront takes a new reference
+        auto slot = [&](int k) {
+            if (kPV && k + kAhead < kSlots) ops[k + kAhead] = operand(k + kAhead);
             if (k % kCopyStep == 1) {
                 const int q = k / kCopyStep;               // 0, 1: V^T blocks; 2, 3: K blocks
                 if (q < 2) copy_v(t_v, v_wr, q);
                 else copy_k(t_k, k_wr, q - 2);
             }
             if (k == 4) raw_entry = list_lds[fetch_idx];
-            if (k >= kQk0) {
+            if (!kPV) {
+                // the first iteration of a workgroup: the next tile's logits follow the slots (below)
+            } else if (k >= kQk0) {
                 const int j = k - kQk0;
-                const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                s_nxt[j & 1] = Mma<T>::mma(ops[k], qreg[j >> 1], j < 2 ? zero : s_nxt[j & 1]);
+                s_nxt[j >> 3] = Mma<T>::mma(ops[k], qreg[j & 7], (j & 7) == 0 ? cinit : s_nxt[j >> 3]);
             } else {
                 const int st = k >> 2, dt = k & 3;
                 const uint4 bq = make_uint4(pk[st][0], pk[st][1], pk[st][2], pk[st][3]);
@@ -600,35 +618,59 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
                     const int idx = k * kMaxPer + e;
                     mx[e & 3] = fmaxf(mx[e & 3], s_cur[idx >> 4][idx & 15]);
                 }
-            } else if (k == kMaxSlots) {
-                float m = fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3]));
-                m = half_max(m) * p.scale_log2;  // scale > 0 commutes with max
-                const float m_new = fmaxf(m_run, m);
-                m_use = m_new == -INFINITY ? 0.f : m_new;
-                alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-                m_run = m_new;
+                if (k == kMaxSlots - 1) {
+                    // The logits are relative to the row's reference m_ref (it rides on the accumulator
+                    // initialisation of the matrix pipe), m_run is the running maximum relative to it.
+                    // The reference moves only when the maximum has outgrown it by kShiftAt, or with the
+                    // first visible key of a row; until then a probability is a bare exponential.
+                    float m = fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3]));
+                    m = half_max(m);
+                    const float m_new = fmaxf(m_run, m);
+                    const bool first = m_run == -INFINITY && m != -INFINITY;
+                    const bool sh = first || m_new > kShiftAt;
+                    moved = __builtin_amdgcn_ballot_w64(sh) != 0ull;
+                    shift = sh ? m_new : 0.f;
+                    alpha = sh ? (first ? 0.f : __builtin_amdgcn_exp2f(-shift)) : 1.f;
+                    m_run = m_new - shift;
+                    m_ref += shift;
+                }
             } else {
 #pragma unroll
                 for (int r = 0; r < kExpPer; r++) {
                     const int prev = (k - 1 - kExpFirst) * kExpPer + r;  // pair computed one slot ago
                     if (prev >= 0 && prev < 16) {
                         const int ks = prev >> 3, v = 2 * (prev & 7);
-                        rs0 += q0[r];
-                        rs1 += q1[r];
-                        pk[2 * ks + (v >> 3)][(v & 7) >> 1] = Mma<T>::pack2(q0[r], q1[r]);
+                        const uint32_t w = Mma<T>::pack2(q0[r], q1[r]);
+                        rs = Mma<T>::sum2(w, rs);              // the row sum takes the rounded values the product uses
+                        pk[2 * ks + (v >> 3)][(v & 7) >> 1] = w;
                     }
                     const int pair = (k - kExpFirst) * kExpPer + r;      // (ks, v) = (pair / 8, 2 * (pair % 8))
                     if (pair < 16) {
                         const int ks = pair >> 3, v = 2 * (pair & 7);
-                        q0[r] = __builtin_amdgcn_exp2f(fmaf(s_cur[ks][v], p.scale_log2, -m_use));
-                        q1[r] = __builtin_amdgcn_exp2f(fmaf(s_cur[ks][v + 1], p.scale_log2, -m_use));
+                        q0[r] = __builtin_amdgcn_exp2f(s_cur[ks][v]);
+                        q1[r] = __builtin_amdgcn_exp2f(s_cur[ks][v + 1]);
                     }
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
+        };
+#pragma unroll
+        for (int k = 0; k < kMaxSlots; k++) slot(k);
+        if (moved) {
+            // rare after the first tiles: this tile's logits come down to the new reference here, the later
+            // ones through the accumulator initialisation
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) s_cur[ks][v] -= shift;
+#pragma unroll
+            for (int v = 0; v < 16; v++) cinit[v] = -m_ref;
         }
-        l_run = l_run * alpha + (rs0 + rs1);
+#pragma unroll
+        for (int k = kMaxSlots; k < kSlots; k++) slot(k);
+        l_run = l_run * alpha + rs;
         fetched = __builtin_amdgcn_readfirstlane(raw_entry);
+        if (!kPV) qk(s_nxt);  // once per workgroup, not interleaved: the logits of tile 1
         // on to the stages of tiles i and i+2; first operands of the next iteration: V^T tile i,
         // complete since the last barrier
         advance_v();
@@ -732,7 +774,7 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     }
     if (row_ok) {
         if (half == 0) {
-            const float l2 = m_run + __builtin_amdgcn_logf(l_tot);  // v_log_f32 is log2
+            const float l2 = m_ref + __builtin_amdgcn_logf(l_tot);  // v_log_f32 is log2
             p.lse[(b * p.H + row_h) * p.Q + row_m] = l2 * 0.6931471805599453f;
             p.lse2[(b * p.H + row_h) * p.Q + row_m] = -l2;
         }
