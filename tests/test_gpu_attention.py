@@ -132,6 +132,34 @@ def test_mfma_prefill_head128(H, KVH, Q, W, C, NS, eager, dtype):
     print(f"{flips}/{compared} slots chose a different token")
 
 
+@pytest.mark.parametrize("dtype,std", [(torch.bfloat16, 0.05), (torch.bfloat16, 1.0), (torch.bfloat16, 3.0),
+                                       (torch.float16, 2.5), (torch.bfloat16, 6.0)])
+def test_mfma_prefill_wide_range_of_logits(dtype, std):
+    """With every value row equal to one the output is one whatever the logits are: the sums of a row
+    and its weighted values must stay relative to the same reference while that reference moves.  Logits
+    of tens of units make the running maximum of a row outgrow its reference again and again along the
+    keys (the oracle is no yardstick there: its 16-bit rotation moves such logits by whole units)."""
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
+    from cascading_kv_cache_amd.cascading_cache import CascadingKVCache
+
+    B, H, KVH, D, NS, W, C, Q = 1, 8, 2, 128, 8, 128, 4, 96
+    cache = CascadingKVCache(window_length=W, num_sink_tokens=NS, max_batch_size=B, heads=KVH, dim=D,
+                             max_seq_len=W * C, device="cuda:0", dtype=dtype, layers=1, verbose=False)
+    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    gen = torch.Generator().manual_seed(31)
+    for c in range(9):
+        q = (torch.randn(B, H, Q, D, generator=gen) * std).to(dtype).cuda()
+        k = (torch.randn(B, KVH, Q, D, generator=gen) * std).to(dtype).cuda()
+        # keys that grow along the chunk: later tiles hold the larger logits
+        k = k * torch.linspace(0.25, 1.0, Q, device="cuda:0").to(dtype).view(1, 1, Q, 1)
+        v = torch.ones(B, KVH, Q, D, dtype=dtype, device="cuda:0")
+        out, new_scores = cascade_attention(q, k, v, cache, 0, inv_freq)
+        torch.cuda.synchronize()
+        err = (out.float() - 1.0).abs().max().item()
+        assert err <= 1e-2, f"chunk {c}: rows of probabilities sum to 1 +- {err:.3e}"
+        assert torch.isfinite(new_scores.float()).all() and torch.isfinite(cache.score_cache[0].float()).all()
+
+
 @pytest.mark.parametrize("H,KVH,W,C,NS,eager,dtype", [
     (8, 2, 64, 4, 8, True, torch.bfloat16),      # G = 4
     (14, 2, 32, 4, 4, False, torch.bfloat16),    # G = 7
