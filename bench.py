@@ -219,12 +219,13 @@ def run_cpu_baseline(cache, pool, dtype):
     q_s = 64
     q, k, v = (t[:, :, :q_s].cpu().contiguous() for t in pool[0])
     layer.query_pos = torch.arange(q_s).view(1, -1)
+    layer.forward(q, k, v, o)  # untimed: first-touch of the cache copy and thread start-up
     t0 = time.perf_counter()
     reps = 0
-    while True:
+    while True:  # a bounded sample: about ten seconds of CPU work
         layer.forward(q, k, v, o)
         reps += 1
-        if time.perf_counter() - t0 > 10.0 or reps >= 8:
+        if time.perf_counter() - t0 > 10.0 or reps >= 256:
             break
     dt = time.perf_counter() - t0
     return dict(value=cfg["B"] * q_s * reps / dt, unit="tokens/s", cores=threads, kind="port",
