@@ -86,3 +86,58 @@ def test_full_size_properties(cfg):
 
     # 4. the score EMA after the call does not depend on V at all
     assert torch.equal(half[0]["score_cache"], snapshot(cache)[0]["score_cache"])
+
+
+def _rope64(x, pos, theta=5e5):
+    """Textbook rotary embedding in float64 with complex numbers: pairs (x[d], x[d + D/2])."""
+    D = x.size(-1)
+    xd = x.double()
+    z = torch.complex(xd[..., : D // 2], xd[..., D // 2:])
+    freq = theta ** (-torch.arange(0, D, 2, dtype=torch.float64) / D)
+    ang = pos.double()[..., None] * freq
+    z = z * torch.polar(torch.ones_like(ang), ang)
+    return torch.cat((z.real, z.imag), dim=-1)
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(B=2, H=32, KVH=8, D=128, NS=64, S=16384, C=8, Q=2048, fill=10),
+    dict(B=16, H=32, KVH=8, D=128, NS=64, S=32768, C=4, Q=1, fill=17),     # decode with the cache full
+])
+def test_full_size_sampled_rows_against_dense_attention(cfg):
+    """At the benchmark sizes the whole oracle takes minutes, a few rows of it do not: for sampled
+    (batch, head, query) rows, softmax(q K^T / sqrt(D)) V over exactly the visible keys in float64, with
+    complex-number RoPE at the cache's position ids, against the library's output (2e-2 abs, bf16)."""
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, chunk_positions, default_inv_freq
+
+    dtype = torch.bfloat16
+    B, H, KVH, D, Q, NS = cfg["B"], cfg["H"], cfg["KVH"], cfg["D"], cfg["Q"], cfg["NS"]
+    G = H // KVH
+    cache = make_cache(B, KVH, D, NS, cfg["S"], cfg["C"], dtype)
+    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    gen = torch.Generator().manual_seed(9)
+    for _ in range(cfg["fill"]):
+        cascade_attention(*chunk(B, H, KVH, 2048, D, gen, dtype), cache, 0, inv_freq)
+    q, k, v = chunk(B, H, KVH, Q, D, gen, dtype)
+    # what the call will see: the state before it
+    vals = [t.clone() for t in cache.get_vals(0)]
+    sink_k, sink_v, sink_pos, sink_mask, ck, cv, key_pos, key_mask, _ = vals
+    q_pos = chunk_positions(cache, 0, Q).cpu().view(-1)
+    out, _ = cascade_attention(q, k, v, cache, 0, inv_freq, update_cache=False)
+    torch.cuda.synchronize()
+    sv, cvalid = (~sink_mask[0, 0]).cpu(), (~key_mask[0, 0]).cpu()
+    assert int(cvalid.sum()) == cfg["S"], "the cache should be full at this point"
+    sink_pos, key_pos = sink_pos[0].cpu(), key_pos[0].cpu()
+    rows = [(0, 0, 0), (B - 1, H - 1, Q - 1), (B // 2, 5, Q // 2), (0, 17, min(Q - 1, 63)), (B - 1, 30, min(Q - 1, 64)),
+            (0, 9, max(0, Q - 700))]
+    worst = 0.0
+    for b, h, m in rows:
+        kvh = h // G
+        keys = torch.cat((_rope64(sink_k[b, kvh].cpu()[sv], sink_pos[sv]),
+                          _rope64(ck[b, kvh].cpu()[cvalid], key_pos[cvalid]),
+                          _rope64(k[b, kvh, : m + 1].cpu(), q_pos[: m + 1])), dim=0)
+        valv = torch.cat((sink_v[b, kvh].cpu()[sv], cv[b, kvh].cpu()[cvalid], v[b, kvh, : m + 1].cpu()), dim=0).double()
+        qr = _rope64(q[b, h, m].cpu(), q_pos[m])
+        p = torch.softmax(keys @ qr / (D ** 0.5), dim=0)
+        want = p @ valv
+        worst = max(worst, (out[b, h, m].double().cpu() - want).abs().max().item())
+    assert worst <= 2e-2, f"sampled rows differ from dense attention by {worst:.3e}"
