@@ -946,7 +946,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
 // one workgroup per (b, h): 4 quarters of 128 threads walk every 4th tile, then merge through LDS
 template <typename T>
 __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
-    __shared__ float sh_m[512], sh_l[16];
+    __shared__ float sh_m[8], sh_l[16];
     __shared__ float4 sh_o[16][32];
     const ckv_attn_args& a = p.a;
     const int64_t row = blockIdx.x;  // b * H + h
@@ -954,28 +954,38 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
     const float* ml = p.part_ml + row * p.tiles * 2;
     float M = -INFINITY;
     for (int t = tid; t < p.tiles; t += 512) M = fmaxf(M, ml[2 * t]);
-    sh_m[tid] = M;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
+    if ((tid & 63) == 0) sh_m[tid >> 6] = M;
     __syncthreads();
-    for (int off = 256; off > 0; off >>= 1) {
-        if (tid < off) sh_m[tid] = fmaxf(sh_m[tid], sh_m[tid + off]);
-        __syncthreads();
-    }
-    M = sh_m[0];
+    M = sh_m[tid & 7];
+#pragma unroll
+    for (int off = 4; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
     // every tile's partial is written by the main kernel (zeros when the tile is hidden), so the
-    // loop needs no branch and its loads can all be in flight together
+    // loop needs no branch; the loads of eight tiles are in flight together
     float L = 0.f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     const float4* po = reinterpret_cast<const float4*>(p.part_o + row * p.tiles * kD) + d4;
-#pragma unroll 4
-    for (int t = grp; t < p.tiles; t += 16) {
-        const float m = ml[2 * t];
-        const float sc = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - M);
-        const float4 v = po[(int64_t)t * (kD / 4)];
-        L = fmaf(ml[2 * t + 1], sc, L);
-        o.x = fmaf(v.x, sc, o.x);
-        o.y = fmaf(v.y, sc, o.y);
-        o.z = fmaf(v.z, sc, o.z);
-        o.w = fmaf(v.w, sc, o.w);
+    constexpr int kBatch = 8;
+    for (int t0 = grp; t0 < p.tiles; t0 += 16 * kBatch) {
+        float4 v[kBatch];
+        float2 w[kBatch];
+#pragma unroll
+        for (int u = 0; u < kBatch; u++) {
+            const int t = t0 + 16 * u;
+            const bool ok = t < p.tiles;
+            v[u] = ok ? po[(int64_t)t * (kD / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
+            w[u] = ok ? *reinterpret_cast<const float2*>(ml + 2 * t) : make_float2(-INFINITY, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < kBatch; u++) {
+            const float sc = w[u].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w[u].x - M);
+            L = fmaf(w[u].y, sc, L);
+            o.x = fmaf(v[u].x, sc, o.x);
+            o.y = fmaf(v[u].y, sc, o.y);
+            o.z = fmaf(v[u].z, sc, o.z);
+            o.w = fmaf(v[u].w, sc, o.w);
+        }
     }
     sh_o[grp][d4] = o;
     if (d4 == 0) sh_l[grp] = L;
