@@ -1,0 +1,69 @@
+"""The generation loop of the reference (cascade_attention.py:452-538: prompt in strides, then one token at
+a time) over a small multi-layer decoder: every layer owns one layer of a CascadingKVCache.  The CPU side
+is the same decoder with the oracle's attention and one OracleCache per layer."""
+import pytest
+import torch
+
+from oracle.attention import OracleCascadeAttention
+from oracle.update import OracleCache
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_logits(model, oracles, caches, ids):
+    cfg = model.cfg
+    B, q = ids.shape
+    x = model.embed_tokens(ids)
+    for layer, attn_o, cache in zip(model.layers, oracles, caches):
+        h = layer.input_layernorm(x)
+        qs, ks, vs = layer.self_attn.qkv(h, (B, q, cfg.num_heads, cfg.head_dim), (B, q, cfg.num_kv_heads, cfg.head_dim))
+        a = attn_o.forward(qs, ks, vs, cache)
+        x = x + layer.self_attn.o_proj(a.transpose(1, 2).reshape(B, q, -1))
+        x = x + layer.mlp(layer.post_attention_layernorm(x))
+    return model.lm_head(model.norm(x[:, -1:]))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_small_decoder_prefill_and_greedy_steps_against_the_oracle(dtype):
+    from cascading_kv_cache_amd.decoder import PRESETS, CascadeDecoder
+
+    cfg = PRESETS["tiny"]
+    gpu = CascadeDecoder(cfg, dtype=dtype, device="cuda:0", seed=3)
+    cpu = CascadeDecoder(cfg, dtype=dtype, device="cpu", seed=3)
+    for (n1, p1), (n2, p2) in zip(gpu.named_parameters(), cpu.named_parameters()):
+        assert n1 == n2 and torch.equal(p1.cpu(), p2), n1
+    B, NS, W, C = 2, 4, 64, 2      # the stream below stays inside the window: no eviction, so no score ties decide
+    cache = gpu.new_cache(W * C, C, batch=B, num_sink_tokens=NS)
+    caches = [OracleCache(window_length=W, num_sink_tokens=NS, max_batch_size=B, heads=cfg.num_kv_heads,
+                          dim=cfg.head_dim, max_seq_len=W * C, dtype=dtype) for _ in range(cfg.num_layers)]
+    oracles = [OracleCascadeAttention(cfg.num_heads, cfg.num_kv_heads, cfg.head_dim, rope_theta=cfg.rope_theta,
+                                      head_reduction=cfg.head_reduction) for _ in range(cfg.num_layers)]
+    ids = torch.randint(0, cfg.vocab_size, (B, 70), generator=torch.Generator().manual_seed(4))
+    with torch.no_grad():
+        steps = [ids[:, 0:32], ids[:, 32:64], ids[:, 64:70]] + [ids[:, i:i + 1] for i in range(5)]
+        for n, chunk in enumerate(steps):
+            lg = gpu(chunk.cuda(), cache).float().cpu()
+            lc = oracle_logits(cpu, oracles, caches, chunk).float()
+            scale = lc.abs().max().item()
+            err = (lg - lc).abs().max().item()
+            assert err <= 3e-2 * scale + 1e-3, f"step {n}: logits differ by {err:.3e} (scale {scale:.3e})"
+    seen = cache.seen_tokens_by_layer.cpu().tolist()
+    assert seen == [75] * cfg.num_layers, seen
+    for i, oc in enumerate(caches):
+        for name in ("mask", "sink_mask", "pos", "sink_pos", "stored_tokens", "start_indices", "stored_sinks", "og_pos"):
+            assert torch.equal(getattr(cache, name)[i].cpu(), getattr(oc, name)), f"layer {i}: {name}"
+
+
+def test_generate_streams_past_the_window():
+    from cascading_kv_cache_amd.decoder import PRESETS, CascadeDecoder, generate
+
+    cfg = PRESETS["tiny"]
+    model = CascadeDecoder(cfg, dtype=torch.bfloat16, device="cuda:0", seed=5)
+    cache = model.new_cache(128, 4, batch=2, num_sink_tokens=4)
+    ids = torch.randint(0, cfg.vocab_size, (2, 500), generator=torch.Generator().manual_seed(6)).cuda()
+    out = generate(model, ids, cache, stride=96, max_new_tokens=12)
+    assert out.shape == (2, 512) and torch.equal(out[:, :500], ids)
+    assert int(out.min()) >= 0 and int(out.max()) < cfg.vocab_size
+    # 500 prompt tokens + 11 fed-back tokens went through every layer (the last new token is never fed back)
+    assert cache.seen_tokens_by_layer.cpu().tolist() == [511] * cfg.num_layers
+    assert not bool(cache.mask[0].any()) and not bool(cache.mask[cfg.num_layers - 1].any())  # every slot holds a token
