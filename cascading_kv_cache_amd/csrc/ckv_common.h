@@ -100,7 +100,8 @@ __device__ inline const void* uniform_ptr(const void* p) {
 // to M0), lane i at +16*i; the source is `sbase` (uniform, SGPR pair) + `voff` (per lane).
 // Inline assembly on purpose: the compiler keeps no scoreboard entry for the copy, so it cannot
 // force it to complete before unrelated LDS reads; completion is awaited explicitly with
-// s_waitcnt vmcnt(n) (copies retire in issue order).
+// s_waitcnt vmcnt(n) (copies retire in issue order).  M0 is written without being declared: the compiler
+// reserves it and loads it itself right before each of its own instructions that read it.
 __device__ inline void async_copy16(const void* sbase, uint32_t voff, uint32_t lds_wave_base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
