@@ -60,48 +60,29 @@ extern "C" int ckv_profile_read(double* ms, int64_t* launches) {
 
 namespace ckv {
 namespace {
-__device__ inline int64_t wave_max_i64(int64_t m) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const int64_t o = __shfl_xor(m, off);
-        m = o > m ? o : m;
-    }
-    return m;
-}
-
-// One workgroup: the largest position id in the cache (all slots, as the reference's amax) plus one, then
-// an arange from there.  All loads of a thread are issued before the first is used (one memory round
-// trip for 32 768 ids), and the reduction is a wavefront shuffle plus 16 values through LDS.
 __global__ void __launch_bounds__(1024) chunk_positions_kernel(const int64_t* key_pos, int64_t n_key, int64_t key_shift,
                                                                const int64_t* sink_pos, int64_t n_sink, int64_t q_len,
                                                                int64_t* q_pos) {
-    __shared__ int64_t red[16];
+    __shared__ int64_t red[1024];
     const int tid = threadIdx.x;
     int64_t base = 0;
     if (key_pos || sink_pos) {
         int64_t m = INT64_MIN;
-        constexpr int kBatch = 16;
-        for (int64_t i0 = 0; i0 < n_key; i0 += 1024 * kBatch) {
-            int64_t v[kBatch];
-#pragma unroll
-            for (int u = 0; u < kBatch; u++) {
-                const int64_t i = i0 + (int64_t)u * 1024 + tid;
-                v[u] = i < n_key ? key_pos[i] : INT64_MIN;
-            }
-#pragma unroll
-            for (int u = 0; u < kBatch; u++) m = v[u] > m ? v[u] : m;
+        for (int64_t i = tid; i < n_key; i += 1024) {
+            const int64_t v = key_pos[i] + key_shift;
+            m = v > m ? v : m;
         }
-        if (m != INT64_MIN) m += key_shift;
         for (int64_t i = tid; i < n_sink; i += 1024) {
             const int64_t v = sink_pos[i];
             m = v > m ? v : m;
         }
-        m = wave_max_i64(m);
-        if ((tid & 63) == 0) red[tid >> 6] = m;
+        red[tid] = m;
         __syncthreads();
-        m = red[tid & 15];
-        m = wave_max_i64(m);
-        base = m + 1;
+        for (int off = 512; off > 0; off >>= 1) {
+            if (tid < off) red[tid] = red[tid + off] > red[tid] ? red[tid + off] : red[tid];
+            __syncthreads();
+        }
+        base = red[0] + 1;
     }
     for (int64_t i = tid; i < q_len; i += 1024) q_pos[i] = base + i;
 }
