@@ -12,6 +12,7 @@
 //                 new token's own score (cascade_attention.py:315-330 with q_len == 1).
 #include "ckv_attn_internal.h"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace ckv {
@@ -70,6 +71,8 @@ struct DecodeParams {
     float* qrot;       // (B, H, 128) rotated, pre-scaled queries
     void* qrot_t;      // (B, H, 128) rotated queries in the tensor dtype (MFMA operand)
     float* logits;     // (B, KVH, N, G) log2-domain logits, -inf for hidden keys
+    void* probs;       // streaming kernel instead: (B, H, Np) fp16, 2^(logit - maximum of the key's tile), same memory
+    int64_t Np;        // row pitch of probs: the keys rounded up to whole tiles
     float* part_ml;    // (B, H, tiles, 2)
     float* part_o;     // (B, H, tiles, 128)
     float* lse2;       // (B, H)
@@ -629,6 +632,9 @@ inline bool stream_offsets_fit(const ckv_attn_args& a) {
     return a.S * a.cache_stride[2] * es + 256 < lim && a.num_sink * a.sink_stride[2] * es + 256 < lim;
 }
 
+constexpr int kStreamProbWave = 1;  // the wavefront that stores the tile's probabilities (wavefront 0 stores maximum and sum)
+static_assert(kSK / 16 == 8, "a lane's probabilities of a tile are stored as one 16-byte piece");
+
 template <typename T, int G>
 __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_kernel(DecodeParams p) {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -779,31 +785,26 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
         // results of the previous item, stored at the top of the next one
         bool pending = false;
         int pend_b = 0, pend_kvh = 0;
-        f32x4 pend_acc[kDb];
-        float pend_m = 0.f, pend_l = 0.f, pend_sv[4] = {0.f, 0.f, 0.f, 0.f};
+        uint2 pend_o[kDb];  // the tile's weighted V average (sum / l) of this lane's four dims, in the tensor dtype
+        float pend_m = 0.f, pend_l = 0.f;
+        uint4 pend_e = make_uint4(0u, 0u, 0u, 0u);  // the storing wavefront's probabilities: head pg, keys kKpl kgrp ..
 #pragma unroll
-        for (int b2 = 0; b2 < kDb; b2++) pend_acc[b2] = f32x4{0.f, 0.f, 0.f, 0.f};
-        // Stores share the counter of the copies and retire in order with them, so all stores of an item
-        // are issued together right after a wait: by the next wait that has to outlast them they are a
-        // whole item old.
+        for (int b2 = 0; b2 < kDb; b2++) pend_o[b2] = make_uint2(0u, 0u);
+        // Stores share the counter of the copies and retire in order with them.  All stores of an item are
+        // issued together, right after the copies of the next item's K rows; every wavefront issues kDb
+        // of them (two wavefronts one more each), and none before the first item of a run has results.
         auto flush = [&]() {
             if (!pending) return;
-            if (kq == 0 && n_wave + key16 < p.N) {  // with G <= 4 only the lanes of kq == 0 hold logits
-                float* lg = p.logits + (((int64_t)pend_b * KVH + pend_kvh) * p.N + n_wave + key16) * G;
-                if constexpr (G == 4) {
-                    *reinterpret_cast<float4*>(lg) = make_float4(pend_sv[0], pend_sv[1], pend_sv[2], pend_sv[3]);
-                } else {
-#pragma unroll
-                    for (int v = 0; v < G; v++) lg[v] = pend_sv[v];
-                }
+            if (wave == kStreamProbWave && pg < G) {  // every wavefront holds all of them: one stores, 16 bytes a lane
+                _Float16* pr = reinterpret_cast<_Float16*>(p.probs) +
+                               (((int64_t)pend_b * KVH + pend_kvh) * G + pg) * p.Np + tile * kSK + kKpl * kgrp;
+                *reinterpret_cast<uint4*>(pr) = pend_e;
             }
             if (key16 < G) {
                 const int64_t row = ((int64_t)pend_b * a.H + pend_kvh * G + key16) * p.tiles + tile;
 #pragma unroll
-                for (int b2 = 0; b2 < kDb; b2++) {
-                    *reinterpret_cast<float4*>(p.part_o + row * kD + 16 * (kDb * wave + b2) + 4 * kq) =
-                        make_float4(pend_acc[b2][0], pend_acc[b2][1], pend_acc[b2][2], pend_acc[b2][3]);
-                }
+                for (int b2 = 0; b2 < kDb; b2++)
+                    *reinterpret_cast<uint2*>(reinterpret_cast<T*>(p.part_o) + row * kD + 16 * (kDb * wave + b2) + 4 * kq) = pend_o[b2];
             }
             if (wave == 0 && kgrp == 0 && pg < G) {
                 const int64_t row = ((int64_t)pend_b * a.H + pend_kvh * G + pg) * p.tiles + tile;
@@ -811,21 +812,49 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
             }
         };
 
-        // The waits count copies only.  Loads retire in issue order, so "at most n operations
-        // outstanding" with n younger copies issued after the wanted ones means the wanted ones are done.
+        // Loads and stores retire in issue order, so "at most n operations outstanding" with n younger
+        // ones issued after the wanted copies means the wanted ones are done.  Per item the order is
+        // K rows and queries of the next item (5), stores of the previous one (kDb, once there is one),
+        // V rows of the next item (4).
         copy_kq(b, kvh, 0);
         copy_v(b, kvh, 0);
         int st = 0;
+        // stores this wavefront issued in the latest flush(): kDb partial averages, the probabilities
+        // from one wavefront, maximum and sum from another
+        const int my_stores = kDb + (wave == kStreamProbWave ? 1 : 0) + (wave == 0 ? 1 : 0);
+        int stored = 0;
+        auto wait_copies = [&](int younger, bool lds_too) {  // vmcnt(younger) [, lgkmcnt(0)]: the count is an immediate
+            if (lds_too) {
+                switch (younger) {
+                    case 5: __builtin_amdgcn_s_waitcnt(0x0075); break;
+                    case 6: __builtin_amdgcn_s_waitcnt(0x0076); break;
+                    case 7: __builtin_amdgcn_s_waitcnt(0x0077); break;
+                    case 8: __builtin_amdgcn_s_waitcnt(0x0078); break;
+                    default: __builtin_amdgcn_s_waitcnt(0x0070); break;
+                }
+            } else {
+                switch (younger) {
+                    case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+                    case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
+                    case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+                    case 7: __builtin_amdgcn_s_waitcnt(0x0F77); break;
+                    default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+                }
+            }
+        };
+        static_assert(kDb <= 2, "wait_copies covers up to kDb + 2 stores");
         for (int64_t bh = bh0; bh < bh1; bh++) {
             int b_nx = b, kvh_nx = kvh;
             if (bh + 1 < bh1) {  // the last item of a run copies itself again: cheaper than a different path
                 kvh_nx = kvh + 1 == KVH ? 0 : kvh + 1;
                 b_nx = kvh + 1 == KVH ? b + 1 : b;
             }
-            // K rows and queries of this item are in LDS (only its four V copies may still be in flight)
-            __builtin_amdgcn_s_waitcnt(0x0F74);  // vmcnt(4)
-            flush();
+            // K rows and queries of this item are in LDS: younger are the stores issued after them and the
+            // four V copies of this item
+            wait_copies(4 + stored, false);
             copy_kq(b_nx, kvh_nx, st ^ 1);
+            stored = pending ? my_stores : 0;
+            flush();
             const unsigned char* stage = smem + st * kStreamStage;
 
             // ---- rotate K in registers, logits by MFMA, shared through LDS
@@ -857,23 +886,22 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
 #pragma unroll
                 for (int ks = 0; ks < 4; ks++) sacc = Mma16<T>::mma(qop[ks], kop[ks], sacc);
                 // lane holds heads 4 kq + v of key key16: with G <= 4 only the lanes of kq == 0 hold heads
-#pragma unroll
-                for (int v = 0; v < 4; v++) pend_sv[v] = vis1 ? sacc[v] * p.scale_log2 : -INFINITY;
                 if (kq == 0) {
 #pragma unroll
-                    for (int v = 0; v < G; v++) s_all[(st * 4 + v) * kSK + wave * 16 + key16] = pend_sv[v];
+                    for (int v = 0; v < G; v++)
+                        s_all[(st * 4 + v) * kSK + wave * 16 + key16] = vis1 ? sacc[v] * p.scale_log2 : -INFINITY;
                 }
             }
             // this wavefront's V rows of the item have landed (younger: the five copies of the next item's K
-            // rows and queries and, after the first item, the stores of flush()) and its logits are
-            // in LDS
-            __builtin_amdgcn_s_waitcnt(0x0070 | (6 + kDb));  // vmcnt(5 copies + 1 + kDb stores), lgkmcnt(0)
+            // rows and queries and the stores of flush()) and its logits are in LDS
+            wait_copies(5 + stored, true);
             __builtin_amdgcn_s_barrier();
             // every wavefront is past the previous item: its V stage can be refilled
             copy_v(b_nx, kvh_nx, st ^ 1);
 
             // ---- softmax over the tile's keys, done by every wavefront: lane = (head, kKpl keys)
             float m_t, l_t;
+            uint4 e_half = make_uint4(0u, 0u, 0u, 0u);
             {
                 float x[kKpl];
 #pragma unroll
@@ -894,8 +922,14 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                     const float e2 = __builtin_amdgcn_exp2f(x[e + 2] - ms), e3 = __builtin_amdgcn_exp2f(x[e + 3] - ms);
                     lloc += (e0 + e1) + (e2 + e3);
                     // probabilities in the tensor dtype, [head][kSK keys] (hidden keys and idle lanes: 0)
-                    *reinterpret_cast<uint2*>(p_wave + pg * kStreamPPitch + (kKpl * kgrp + e) * 2) =
-                        make_uint2(Mma16<T>::pack2(e0, e1), Mma16<T>::pack2(e2, e3));
+                    const uint2 pk = make_uint2(Mma16<T>::pack2(e0, e1), Mma16<T>::pack2(e2, e3));
+                    *reinterpret_cast<uint2*>(p_wave + pg * kStreamPPitch + (kKpl * kgrp + e) * 2) = pk;
+                    // the copy that goes to memory for the score kernel is fp16 whatever the tensor dtype
+                    uint2 hk = pk;
+                    if constexpr (!std::is_same<T, __half>::value) {
+                        if (wave == kStreamProbWave) hk = make_uint2(Mma16<__half>::pack2(e0, e1), Mma16<__half>::pack2(e2, e3));
+                    }
+                    if (e == 0) { e_half.x = hk.x; e_half.y = hk.y; } else { e_half.z = hk.x; e_half.w = hk.y; }
                 }
                 m_t = m;
                 l_t = mod4_sum(lloc);
@@ -924,10 +958,17 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                     }
                 }
             }
+            {
+                // lanes 16 q + g hold head g, and g == pg there: l_t is that head's sum (0: the tile is hidden)
+                const float inv_l = l_t > 0.f ? 1.0f / l_t : 0.f;
 #pragma unroll
-            for (int b2 = 0; b2 < kDb; b2++) pend_acc[b2] = acc[b2];
+                for (int b2 = 0; b2 < kDb; b2++)
+                    pend_o[b2] = make_uint2(Mma16<T>::pack2(acc[b2][0] * inv_l, acc[b2][1] * inv_l),
+                                            Mma16<T>::pack2(acc[b2][2] * inv_l, acc[b2][3] * inv_l));
+            }
             pend_m = m_t;
             pend_l = l_t;
+            pend_e = e_half;
             pending = true;
             pend_b = b;
             pend_kvh = kvh;
@@ -944,7 +985,8 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
 }
 
 // one workgroup per (b, h): 4 quarters of 128 threads walk every 4th tile, then merge through LDS
-template <typename T>
+// AVG: the partials are per-tile averages in the tensor dtype (the streaming kernel) instead of fp32 sums
+template <typename T, bool AVG>
 __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
     __shared__ float sh_m[8], sh_l[16];
     __shared__ float4 sh_o[16][32];
@@ -966,6 +1008,7 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
     float L = 0.f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     const float4* po = reinterpret_cast<const float4*>(p.part_o + row * p.tiles * kD) + d4;
+    const uint2* po16 = reinterpret_cast<const uint2*>(reinterpret_cast<const T*>(p.part_o) + row * p.tiles * kD) + d4;
     constexpr int kBatch = 8;
     for (int t0 = grp; t0 < p.tiles; t0 += 16 * kBatch) {
         float4 v[kBatch];
@@ -974,13 +1017,23 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
         for (int u = 0; u < kBatch; u++) {
             const int t = t0 + 16 * u;
             const bool ok = t < p.tiles;
-            v[u] = ok ? po[(int64_t)t * (kD / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
+            if constexpr (AVG) {
+                const uint2 r = ok ? po16[(int64_t)t * (kD / 4)] : make_uint2(0u, 0u);
+                v[u] = make_float4(Mma16<T>::lo(r.x), Mma16<T>::hi(r.x), Mma16<T>::lo(r.y), Mma16<T>::hi(r.y));
+            } else {
+                v[u] = ok ? po[(int64_t)t * (kD / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
             w[u] = ok ? *reinterpret_cast<const float2*>(ml + 2 * t) : make_float2(-INFINITY, 0.f);
         }
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
-            const float sc = w[u].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w[u].x - M);
-            L = fmaf(w[u].y, sc, L);
+            float sc = w[u].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w[u].x - M);
+            if constexpr (AVG) {
+                sc *= w[u].y;
+                L += sc;
+            } else {
+                L = fmaf(w[u].y, sc, L);
+            }
             o.x = fmaf(v[u].x, sc, o.x);
             o.y = fmaf(v[u].y, sc, o.y);
             o.z = fmaf(v[u].z, sc, o.z);
@@ -1036,7 +1089,7 @@ __device__ inline float reduce_group(const float* v, int n, int mode) {
 
 // one thread per (b, kvh, key): P of the G (or all H) heads, dtype rounding like the eager path
 // (cascade_attention.py:319-323 with a single query row), head reduction, EMA / new-token score
-template <typename T, int G, bool HOMO>
+template <typename T, int G, bool HOMO, bool PROBS>
 __global__ void __launch_bounds__(256) decode_scores_kernel(DecodeParams p, float w_one, float beta_pow) {
     const ckv_attn_args& a = p.a;
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1053,7 +1106,15 @@ __global__ void __launch_bounds__(256) decode_scores_kernel(DecodeParams p, floa
         const float* lg = p.logits + ((b * a.KVH + kv) * p.N + n) * G;
 #pragma unroll
         for (int g = 0; g < G; g++) {
-            const float pt = round_t<T>(__builtin_amdgcn_exp2f(lg[g] - p.lse2[b * a.H + kv * G + g]));
+            const int64_t row = b * a.H + kv * G + g;
+            float pt;
+            if constexpr (PROBS) {  // 2^(logit - tile maximum) from the streaming kernel, and that maximum
+                const float e = (float)reinterpret_cast<const _Float16*>(p.probs)[row * p.Np + n];
+                const float m = p.part_ml[(row * p.tiles + n / kSK) * 2];
+                pt = e == 0.f ? 0.f : round_t<T>(e * __builtin_amdgcn_exp2f(m - p.lse2[row]));
+            } else {
+                pt = round_t<T>(__builtin_amdgcn_exp2f(lg[g] - p.lse2[row]));
+            }
             // cached slots: fp32 product, cast; the new token: product in the tensor dtype
             vals[cnt++] = round_t<T>(__fmul_rn(pt, is_new ? round_t<T>(w_one) : w_one));
         }
@@ -1093,6 +1154,91 @@ __global__ void __launch_bounds__(256) decode_scores_kernel(DecodeParams p, floa
     }
 }
 
+// The same after the streaming kernel, per kv head: one thread per (b, kvh, 8 consecutive keys), which are one
+// 16-byte piece of each head's fp16 probabilities and share the tile maximum.
+template <typename T, int G>
+__global__ void __launch_bounds__(256) decode_scores_probs_kernel(DecodeParams p, float w_one, float beta_pow) {
+    const ckv_attn_args& a = p.a;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t per = p.Np / 8;
+    if (idx >= a.B * a.KVH * per) return;
+    const int64_t n0 = (idx % per) * 8, kvh = (idx / per) % a.KVH, b = idx / (per * a.KVH);
+    if (n0 + 8 <= a.num_sink || n0 >= p.N) return;  // sinks keep no score; padding
+    float pr[G][8];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const int64_t row = b * a.H + kvh * G + g;
+        const uint4 raw = *reinterpret_cast<const uint4*>(reinterpret_cast<const _Float16*>(p.probs) + row * p.Np + n0);
+        const float c = __builtin_amdgcn_exp2f(p.part_ml[(row * p.tiles + n0 / kSK) * 2] - p.lse2[row]);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float e = (float)__builtin_bit_cast(f16x2_t, w[k >> 1])[k & 1];
+            pr[g][k] = e == 0.f ? 0.f : round_t<T>(e * c);
+        }
+    }
+    const float w_new = round_t<T>(w_one);
+    float red[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const bool is_new = n0 + k == p.N - 1;
+        float vals[G];
+        // cached slots: fp32 product, cast; the new token: product in the tensor dtype
+#pragma unroll
+        for (int g = 0; g < G; g++) vals[g] = round_t<T>(__fmul_rn(pr[g][k], is_new ? w_new : w_one));
+        float r;
+        if (a.head_reduction == CKV_REDUCE_MAX) {
+            r = vals[0];
+#pragma unroll
+            for (int g = 1; g < G; g++) r = fmaxf(r, vals[g]);
+        } else if (a.head_reduction == CKV_REDUCE_MEAN) {
+            r = 0.f;
+#pragma unroll
+            for (int g = 0; g < G; g++) r = __fadd_rn(r, vals[g]);
+            r = round_t<T>(r / (float)G);
+        } else {  // lower median: rank by counting
+            r = vals[0];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                int below = 0, equal = 0;
+#pragma unroll
+                for (int h = 0; h < G; h++) {
+                    below += vals[h] < vals[g];
+                    equal += vals[h] == vals[g];
+                }
+                if (below <= (G - 1) / 2 && (G - 1) / 2 < below + equal) r = vals[g];
+            }
+        }
+        red[k] = r;
+    }
+    const int64_t i0 = n0 - a.num_sink;
+    T* cs = a.cache_s ? (T*)a.cache_s + b * a.cache_s_stride[0] + kvh * a.cache_s_stride[1] : nullptr;
+    if (cs && i0 >= 0 && i0 + 8 <= a.S && a.cache_s_stride[2] == 1 && (reinterpret_cast<uintptr_t>(cs + i0) & 15) == 0) {
+        uint4 old = *reinterpret_cast<const uint4*>(cs + i0);
+        T* o = reinterpret_cast<T*>(&old);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float decayed = round_t<T>(__fmul_rn(beta_pow, Elem<T>::to_float(o[k])));
+            o[k] = Elem<T>::from_float(__fadd_rn(decayed, red[k]));
+        }
+        *reinterpret_cast<uint4*>(cs + i0) = old;
+        return;
+    }
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const int64_t i = i0 + k;
+        if (i < 0 || i > a.S) continue;
+        if (i == a.S) {
+            if (a.new_scores)
+                *((T*)a.new_scores + b * a.new_scores_stride[0] + kvh * a.new_scores_stride[1]) = Elem<T>::from_float(red[k]);
+        } else if (cs) {
+            T* c1 = cs + i * a.cache_s_stride[2];
+            const float decayed = round_t<T>(__fmul_rn(beta_pow, Elem<T>::to_float(*c1)));
+            *c1 = Elem<T>::from_float(__fadd_rn(decayed, red[k]));
+        }
+    }
+}
+
 template <typename T, int G>
 int run_decode(const DecodeParams& p_in, hipStream_t stream) {
     DecodeParams p = p_in;
@@ -1100,6 +1246,7 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
     const bool use_stream =
         !std::is_same<T, float>::value && G <= 4 && p.shared_pos && stream_offsets_fit(a) && !getenv("CKV_DECODE_OLD");
     if (use_stream) p.tiles = (int)((p.N + kSK - 1) / kSK);  // the streaming kernel has its own tile size
+    p.Np = (int64_t)p.tiles * kSK;
     {
         StageScope sc(CKV_STAGE_PREP, stream);
         hipLaunchKernelGGL(decode_q_kernel<T>, dim3((unsigned)(a.B * a.H)), dim3(64), 0, stream, p);
@@ -1145,19 +1292,34 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
     }
     {
         StageScope sc(CKV_STAGE_DECODE_TAIL, stream);
-        hipLaunchKernelGGL(decode_tail_kernel<T>, dim3((unsigned)(a.B * a.H)), dim3(512), 0, stream, p);
+        bool launched = false;
+        if constexpr (G <= 4 && !std::is_same<T, float>::value) {
+            if (use_stream) {
+                hipLaunchKernelGGL((decode_tail_kernel<T, true>), dim3((unsigned)(a.B * a.H)), dim3(512), 0, stream, p);
+                launched = true;
+            }
+        }
+        if (!launched) hipLaunchKernelGGL((decode_tail_kernel<T, false>), dim3((unsigned)(a.B * a.H)), dim3(512), 0, stream, p);
         CKV_HIP_TRY(hipGetLastError());
         if (a.cache_s || a.new_scores) {
             // w_ema[0] == w_new[0] == (1 - beta) for a single query row; the new token's weight is
             // built in the tensor dtype (cascade_attention.py:270-276)
             const float w_one = (float)(1.0 - a.beta);
             const int64_t items = a.B * a.KVH * (a.S + 1);
-            if (a.homogeneous_heads)
-                hipLaunchKernelGGL((decode_scores_kernel<T, G, true>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
-                                   stream, p, w_one, (float)a.beta);
+            const dim3 grid((unsigned)((items + 255) / 256));
+            if (a.homogeneous_heads && use_stream)
+                hipLaunchKernelGGL((decode_scores_kernel<T, G, true, true>), grid, dim3(256), 0, stream, p, w_one, (float)a.beta);
+            else if (a.homogeneous_heads)
+                hipLaunchKernelGGL((decode_scores_kernel<T, G, true, false>), grid, dim3(256), 0, stream, p, w_one, (float)a.beta);
+            else if (use_stream) {
+                if constexpr (G <= 4 && !std::is_same<T, float>::value) {
+                    const int64_t groups8 = a.B * a.KVH * (p.Np / 8);
+                    hipLaunchKernelGGL((decode_scores_probs_kernel<T, G>), dim3((unsigned)((groups8 + 255) / 256)), dim3(256), 0,
+                                       stream, p, w_one, (float)a.beta);
+                }
+            }
             else
-                hipLaunchKernelGGL((decode_scores_kernel<T, G, false>), dim3((unsigned)((items + 255) / 256)), dim3(256), 0,
-                                   stream, p, w_one, (float)a.beta);
+                hipLaunchKernelGGL((decode_scores_kernel<T, G, false, false>), grid, dim3(256), 0, stream, p, w_one, (float)a.beta);
             CKV_HIP_TRY(hipGetLastError());
         }
     }
@@ -1199,9 +1361,15 @@ bool decode_supported(const ckv_attn_args& a) {
 
 constexpr int64_t kMinTile = kSK < kTK ? kSK : kTK;  // the partial results are sized for the smaller tile
 
+// fp32 logits per (head, key), or the streaming kernel's fp16 probabilities with rows padded to whole tiles
+inline int64_t logits_area_bytes(int64_t B, int64_t H, int64_t N) {
+    const int64_t padded = (N + kSK - 1) / kSK * kSK;
+    return align_up(std::max(B * H * N * 4, B * H * padded * 2), 256);
+}
+
 int64_t decode_workspace_bytes(int64_t B, int64_t H, int64_t KVH, int64_t num_sink, int64_t S) {
-    const int64_t N = num_sink + S + 1, tiles = (N + kMinTile - 1) / kMinTile, G = H / KVH;
-    return 2 * align_up(B * H * kD * 4, 256) + align_up(B * KVH * N * G * 4, 256) + align_up(B * H * tiles * 2 * 4, 256) +
+    const int64_t N = num_sink + S + 1, tiles = (N + kMinTile - 1) / kMinTile;
+    return 2 * align_up(B * H * kD * 4, 256) + logits_area_bytes(B, H, N) + align_up(B * H * tiles * 2 * 4, 256) +
            align_up(B * H * tiles * kD * 4, 256) + align_up(B * H * 4, 256);
 }
 
@@ -1214,7 +1382,9 @@ int launch_decode(const ckv_attn_args& a, hipStream_t stream) {
     char* w = reinterpret_cast<char*>(a.workspace);
     p.qrot = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * kD * 4, 256);
     p.qrot_t = w; w += align_up(a.B * a.H * kD * 4, 256);
-    p.logits = reinterpret_cast<float*>(w); w += align_up(a.B * a.KVH * p.N * G * 4, 256);
+    p.logits = reinterpret_cast<float*>(w);
+    p.probs = w;
+    w += logits_area_bytes(a.B, a.H, p.N);
     const int64_t tiles_max = (p.N + kMinTile - 1) / kMinTile;
     p.part_ml = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * tiles_max * 2 * 4, 256);
     p.part_o = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * tiles_max * kD * 4, 256);
