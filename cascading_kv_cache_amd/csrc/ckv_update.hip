@@ -35,6 +35,7 @@ struct UpdateParams {
     int32_t do_pos;        // run the position pass (last launch of a call only)
     int32_t* first;        // [N*H][K]
     int32_t* next_of;      // [N*H][S]
+    int32_t* pos_flag;     // [N*H]: the call put a token into the cascades, so the position ids change
 };
 
 // exclusive prefix sum of one flag per thread over the whole workgroup; returns the block total
@@ -242,29 +243,56 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
     }
     __syncthreads();
 
-    // ---- position pass (cascading_cache.py:728-774, 129-142): only when the last token of the
-    //      call went to the cascades
-    if (p.do_pos && cap > n_sink_new) {
-        int64_t ub = 0;
-        for (int i = 0; i < C; i++) ub += st_l[i];
-        int64_t* pos = A.pos + n * A.pos_stride[0] + h * A.pos_stride[1];
-        for (int i = 0; i < C; i++) {
-            const int64_t seg = st_l[i] < W ? st_l[i] : W;
-            if (seg <= 0) break;
-            const int64_t sx = sx_l[i];
-            if (W < (1ll << 30)) {  // the usual case: 32-bit arithmetic, a 64-bit modulo per slot costs far more
-                const uint32_t seg32 = (uint32_t)seg, add32 = (uint32_t)(seg - sx);
-                for (int64_t j = tid; j < W; j += T) {
-                    pos[((int64_t)i * W + j) * A.pos_stride[2]] = (int64_t)(((uint32_t)j + add32) % seg32) + ub - seg;
-                }
-            } else {
-                for (int64_t j = tid; j < W; j += T) {
-                    pos[((int64_t)i * W + j) * A.pos_stride[2]] = ((j + seg - sx) % seg) + ub - seg;
-                }
-            }
-            ub -= W;
-            if (ub <= 0) break;
+    // the position ids change only when the last token of the call went to the cascades
+    if (p.do_pos && tid == 0) p.pos_flag[bh] = cap > n_sink_new ? 1 : 0;
+}
+
+// Position pass (cascading_cache.py:728-774, 129-142) after the plan kernel has updated the trackers:
+// slot j of cascade i gets ((j + seg - start) mod seg) + ub - seg, where seg is the number of stored
+// tokens and ub the ids still to hand out (all stored tokens, less a window per earlier cascade).
+// Grid: (chunks of kPosChunk slots over all cascades, N*H), so the whole chip writes.
+constexpr int kPosChunk = 2048;
+
+__global__ void __launch_bounds__(256) ckv_update_positions_kernel(UpdateParams p) {
+    const ckv_update_args& A = p.a;
+    const int64_t bh = blockIdx.y;
+    if (!p.pos_flag[bh]) return;
+    const int64_t n = bh / A.H, h = bh % A.H;
+    const int C = A.cascades;
+    const int W = (int)A.window_size;
+    const int per_c = (W + kPosChunk - 1) / kPosChunk;
+    const int i = (int)blockIdx.x / per_c, j0 = ((int)blockIdx.x % per_c) * kPosChunk;
+    const int64_t* g_stored = A.stored_tokens + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+    const int64_t* g_start = A.start_indices + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+    int64_t ub = 0;
+    for (int c = 0; c < C; c++) ub += g_stored[c * A.tracker_stride[2]];
+    // cascade i is written only if every earlier one holds tokens and ids are left
+    for (int c = 0; c < i; c++) {
+        if (g_stored[c * A.tracker_stride[2]] <= 0) return;
+        ub -= W;
+        if (ub <= 0) return;
+    }
+    const int64_t st = g_stored[i * A.tracker_stride[2]];
+    const uint32_t seg = (uint32_t)(st < W ? st : W);
+    if (seg == 0) return;
+    const uint32_t add = seg - (uint32_t)g_start[i * A.tracker_stride[2]];  // start < seg or start == 0
+    const int64_t base = ub - seg;
+    auto id_of = [&](int j) -> int64_t {
+        uint32_t x = (uint32_t)j + add;
+        if (x >= seg) x -= seg;
+        if (x >= seg) x %= seg;  // slots past the stored tokens of a cascade that is not full
+        return (int64_t)x + base;
+    };
+    int64_t* pos = A.pos + n * A.pos_stride[0] + h * A.pos_stride[1] + (int64_t)i * W * A.pos_stride[2];
+    const int tid = threadIdx.x;
+    if (A.pos_stride[2] == 1 && (reinterpret_cast<uintptr_t>(pos) & 15u) == 0 && (W & 1) == 0) {
+#pragma unroll
+        for (int it = 0; it < kPosChunk / 512; it++) {
+            const int j = j0 + it * 512 + 2 * tid;
+            if (j < W) *reinterpret_cast<longlong2*>(pos + j) = make_longlong2(id_of(j), id_of(j + 1));
         }
+    } else {
+        for (int j = j0 + tid; j < j0 + kPosChunk && j < W; j += 256) pos[(int64_t)j * A.pos_stride[2]] = id_of(j);
     }
 }
 
@@ -483,7 +511,8 @@ extern "C" int64_t ckv_update_workspace_bytes(int64_t N, int64_t H, int64_t K, i
                                               int32_t cascades) {
     (void)cascades;
     if (N <= 0 || H <= 0 || K < 0 || max_seq_len <= 0) return 0;
-    return ckv::align_up(N * H * (K + max_seq_len) * (int64_t)sizeof(int32_t), 256) + 256;
+    return ckv::align_up(N * H * (K + max_seq_len) * (int64_t)sizeof(int32_t), 256) +
+           ckv::align_up(N * H * (int64_t)sizeof(int32_t), 256) + 256;
 }
 
 extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
@@ -533,15 +562,15 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
     p.a = A;
     p.first = reinterpret_cast<int32_t*>(A.workspace);
     p.next_of = p.first + A.N * A.H * A.K;
+    p.pos_flag = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(A.workspace) +
+                                            align_up(A.N * A.H * (A.K + A.max_seq_len) * (int64_t)sizeof(int32_t), 256));
 
     for (int64_t off = 0; off < A.K; off += qmax) {
         const int ksub = (int)((A.K - off < qmax) ? (A.K - off) : qmax);
         p.token_offset = off;
         p.k_sub = ksub;
         p.do_pos = (off + ksub == A.K) ? 1 : 0;
-        // small calls still rewrite max_seq_len position ids per (n, h): keep enough lanes for that
-        // few tokens: a small block plans them, unless the position pass has many slots to rewrite
-        const int T = (ksub <= 256 && A.max_seq_len < 8192) ? 256 : 1024;
+        const int T = ksub <= 256 ? 256 : 1024;  // few tokens: a small block plans them
         const size_t lds = plan_lds_bytes(ksub);
         if (lds > 48 * 1024) {
             CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(ckv_update_plan_kernel),
@@ -550,6 +579,11 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
         {
             StageScope sc(CKV_STAGE_PLAN, stream);
             hipLaunchKernelGGL(ckv_update_plan_kernel, dim3((unsigned)(A.N * A.H)), dim3(T), lds, stream, p);
+            if (p.do_pos) {
+                const int64_t per_c = (A.window_size + kPosChunk - 1) / kPosChunk;
+                hipLaunchKernelGGL(ckv_update_positions_kernel, dim3((unsigned)(per_c * A.cascades), (unsigned)(A.N * A.H)),
+                                   dim3(256), 0, stream, p);
+            }
         }
         CKV_HIP_TRY(hipGetLastError());
         StageScope sc_apply(CKV_STAGE_APPLY, stream);
