@@ -71,8 +71,14 @@ struct DecodeParams {
     float* qrot;       // (B, H, 128) rotated, pre-scaled queries
     void* qrot_t;      // (B, H, 128) rotated queries in the tensor dtype (MFMA operand)
     float* logits;     // (B, KVH, N, G) log2-domain logits, -inf for hidden keys
-    void* probs;       // streaming kernel instead: (B, H, Np) fp16, 2^(logit - maximum of the key's tile), same memory
-    int64_t Np;        // row pitch of probs: the keys rounded up to whole tiles
+    // The streaming kernel instead (same memory): one chunk per (tile, b, kvh) item, G rows of kSK fp16
+    // values 2^(logit - maximum of the head's logits in the tile), then G rows of 128 per-tile weighted V
+    // averages in the tensor dtype.  Chunks are laid out by time: chunk (i, w) is the i-th item of
+    // workgroup w, and the chunks of equal i sit side by side, so that what the workgroups store at about
+    // the same time is one stretch of memory.
+    unsigned char* chunks;
+    int64_t Np;        // the keys rounded up to whole tiles of the streaming kernel
+    int stream_wgs;    // workgroups of the streaming kernel
     float* part_ml;    // (B, H, tiles, 2)
     float* part_o;     // (B, H, tiles, 128)
     float* lse2;       // (B, H)
@@ -81,6 +87,20 @@ struct DecodeParams {
     int shared_pos;
     float scale_log2;
 };
+
+// Items (tile-major: item = tile * B * KVH + b * KVH + kvh) are dealt out in equal contiguous runs:
+// workgroup w takes [total * w / wgs, total * (w + 1) / wgs).  Chunk index of an item.
+__device__ inline int64_t stream_chunk_of(int64_t item, int64_t total, int64_t wgs) {
+    int64_t w, first;
+    if ((total + 1) * wgs < ((int64_t)1 << 32)) {  // 32-bit division: a fraction of the cost
+        w = (int64_t)(((uint32_t)(item + 1) * (uint32_t)wgs - 1u) / (uint32_t)total);
+        first = (int64_t)((uint32_t)total * (uint32_t)w / (uint32_t)wgs);
+    } else {
+        w = ((item + 1) * wgs - 1) / total;
+        first = total * w / wgs;
+    }
+    return (item - first) * wgs + w;
+}
 
 template <typename T>
 __global__ void decode_q_kernel(DecodeParams p) {
@@ -632,6 +652,7 @@ inline bool stream_offsets_fit(const ckv_attn_args& a) {
     return a.S * a.cache_stride[2] * es + 256 < lim && a.num_sink * a.sink_stride[2] * es + 256 < lim;
 }
 
+constexpr int kStreamMaxWgs = 1024;  // the result chunks are sized for at most this many workgroups
 constexpr int kStreamProbWave = 1;  // the wavefront that stores the tile's probabilities (wavefront 0 stores maximum and sum)
 static_assert(kSK / 16 == 8, "a lane's probabilities of a tile are stored as one 16-byte piece");
 
@@ -795,16 +816,14 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
         // of them (two wavefronts one more each), and none before the first item of a run has results.
         auto flush = [&]() {
             if (!pending) return;
-            if (wave == kStreamProbWave && pg < G) {  // every wavefront holds all of them: one stores, 16 bytes a lane
-                _Float16* pr = reinterpret_cast<_Float16*>(p.probs) +
-                               (((int64_t)pend_b * KVH + pend_kvh) * G + pg) * p.Np + tile * kSK + kKpl * kgrp;
-                *reinterpret_cast<uint4*>(pr) = pend_e;
-            }
+            const int64_t pend_item = tile * nbh + (int64_t)pend_b * KVH + pend_kvh;
+            unsigned char* chunk = p.chunks + ((pend_item - item0) * gridDim.x + blockIdx.x) * (G * (kSK + kD) * 2);
+            if (wave == kStreamProbWave && pg < G)  // every wavefront holds all of them: one stores, 16 bytes a lane
+                *reinterpret_cast<uint4*>(chunk + (pg * kSK + kKpl * kgrp) * 2) = pend_e;
             if (key16 < G) {
-                const int64_t row = ((int64_t)pend_b * a.H + pend_kvh * G + key16) * p.tiles + tile;
 #pragma unroll
                 for (int b2 = 0; b2 < kDb; b2++)
-                    *reinterpret_cast<uint2*>(reinterpret_cast<T*>(p.part_o) + row * kD + 16 * (kDb * wave + b2) + 4 * kq) = pend_o[b2];
+                    *reinterpret_cast<uint2*>(chunk + (G * kSK + key16 * kD + 16 * (kDb * wave + b2) + 4 * kq) * 2) = pend_o[b2];
             }
             if (wave == 0 && kgrp == 0 && pg < G) {
                 const int64_t row = ((int64_t)pend_b * a.H + pend_kvh * G + pg) * p.tiles + tile;
@@ -1008,7 +1027,12 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
     float L = 0.f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     const float4* po = reinterpret_cast<const float4*>(p.part_o + row * p.tiles * kD) + d4;
-    const uint2* po16 = reinterpret_cast<const uint2*>(reinterpret_cast<const T*>(p.part_o) + row * p.tiles * kD) + d4;
+    // streaming kernel: the row's averages sit in the chunks of the items (tile, b, kvh)
+    const int64_t nbh_s = a.B * a.KVH, total_s = (int64_t)p.tiles * nbh_s;
+    const int G_s = (int)(a.H / a.KVH);
+    const int64_t bh_s = (row / a.H) * a.KVH + (row % a.H) / G_s;
+    const int64_t chunk_bytes = (int64_t)G_s * (kSK + kD) * 2;
+    const int64_t in_chunk = ((int64_t)G_s * kSK + (row % a.H) % G_s * kD) * 2 + d4 * 8;
     constexpr int kBatch = 8;
     for (int t0 = grp; t0 < p.tiles; t0 += 16 * kBatch) {
         float4 v[kBatch];
@@ -1018,7 +1042,10 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
             const int t = t0 + 16 * u;
             const bool ok = t < p.tiles;
             if constexpr (AVG) {
-                const uint2 r = ok ? po16[(int64_t)t * (kD / 4)] : make_uint2(0u, 0u);
+                uint2 r = make_uint2(0u, 0u);
+                if (ok)
+                    r = *reinterpret_cast<const uint2*>(
+                        p.chunks + stream_chunk_of((int64_t)t * nbh_s + bh_s, total_s, p.stream_wgs) * chunk_bytes + in_chunk);
                 v[u] = make_float4(Mma16<T>::lo(r.x), Mma16<T>::hi(r.x), Mma16<T>::lo(r.y), Mma16<T>::hi(r.y));
             } else {
                 v[u] = ok ? po[(int64_t)t * (kD / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -1109,7 +1136,8 @@ __global__ void __launch_bounds__(256) decode_scores_kernel(DecodeParams p, floa
             const int64_t row = b * a.H + kv * G + g;
             float pt;
             if constexpr (PROBS) {  // 2^(logit - tile maximum) from the streaming kernel, and that maximum
-                const float e = (float)reinterpret_cast<const _Float16*>(p.probs)[row * p.Np + n];
+                const int64_t ck = stream_chunk_of((n / kSK) * (a.B * a.KVH) + b * a.KVH + kv, p.tiles * (a.B * a.KVH), p.stream_wgs);
+                const float e = (float)reinterpret_cast<const _Float16*>(p.chunks + ck * (G * (kSK + kD) * 2))[g * kSK + n % kSK];
                 const float m = p.part_ml[(row * p.tiles + n / kSK) * 2];
                 pt = e == 0.f ? 0.f : round_t<T>(e * __builtin_amdgcn_exp2f(m - p.lse2[row]));
             } else {
@@ -1165,10 +1193,13 @@ __global__ void __launch_bounds__(256) decode_scores_probs_kernel(DecodeParams p
     const int64_t n0 = (idx % per) * 8, kvh = (idx / per) % a.KVH, b = idx / (per * a.KVH);
     if (n0 + 8 <= a.num_sink || n0 >= p.N) return;  // sinks keep no score; padding
     float pr[G][8];
+    const unsigned char* chunk =
+        p.chunks + stream_chunk_of((n0 / kSK) * (a.B * a.KVH) + b * a.KVH + kvh, p.tiles * (a.B * a.KVH), p.stream_wgs) *
+                       (G * (kSK + kD) * 2);
 #pragma unroll
     for (int g = 0; g < G; g++) {
         const int64_t row = b * a.H + kvh * G + g;
-        const uint4 raw = *reinterpret_cast<const uint4*>(reinterpret_cast<const _Float16*>(p.probs) + row * p.Np + n0);
+        const uint4 raw = *reinterpret_cast<const uint4*>(chunk + (g * kSK + n0 % kSK) * 2);
         const float c = __builtin_amdgcn_exp2f(p.part_ml[(row * p.tiles + n0 / kSK) * 2] - p.lse2[row]);
         const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -1277,7 +1308,9 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
                 CKV_HIP_TRY(hipGetDevice(&dev));
                 CKV_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
                 int64_t wgs = (cus > 0 ? cus : 256) * kStreamWgPerCu;
+                if (wgs > kStreamMaxWgs) wgs = kStreamMaxWgs;
                 if (wgs > p.tiles * nbh) wgs = p.tiles * nbh;
+                p.stream_wgs = (int)wgs;
                 hipLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads), lds_s, stream, p);
             }
         } else {
@@ -1361,15 +1394,17 @@ bool decode_supported(const ckv_attn_args& a) {
 
 constexpr int64_t kMinTile = kSK < kTK ? kSK : kTK;  // the partial results are sized for the smaller tile
 
-// fp32 logits per (head, key), or the streaming kernel's fp16 probabilities with rows padded to whole tiles
-inline int64_t logits_area_bytes(int64_t B, int64_t H, int64_t N) {
-    const int64_t padded = (N + kSK - 1) / kSK * kSK;
-    return align_up(std::max(B * H * N * 4, B * H * padded * 2), 256);
+// fp32 logits per (head, key), or the streaming kernel's result chunks: (kSK + 128) 16-bit values per head and
+// item, for up to one item per workgroup more than there are items (runs differ by one in length)
+inline int64_t logits_area_bytes(int64_t B, int64_t H, int64_t KVH, int64_t N) {
+    const int64_t tiles = (N + kSK - 1) / kSK, items = tiles * B * KVH, G = H / KVH;
+    const int64_t chunks = items + std::min<int64_t>(items, kStreamMaxWgs);
+    return align_up(std::max(B * H * N * 4, chunks * G * (kSK + kD) * 2), 256);
 }
 
 int64_t decode_workspace_bytes(int64_t B, int64_t H, int64_t KVH, int64_t num_sink, int64_t S) {
     const int64_t N = num_sink + S + 1, tiles = (N + kMinTile - 1) / kMinTile;
-    return 2 * align_up(B * H * kD * 4, 256) + logits_area_bytes(B, H, N) + align_up(B * H * tiles * 2 * 4, 256) +
+    return 2 * align_up(B * H * kD * 4, 256) + logits_area_bytes(B, H, KVH, N) + align_up(B * H * tiles * 2 * 4, 256) +
            align_up(B * H * tiles * kD * 4, 256) + align_up(B * H * 4, 256);
 }
 
@@ -1383,8 +1418,9 @@ int launch_decode(const ckv_attn_args& a, hipStream_t stream) {
     p.qrot = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * kD * 4, 256);
     p.qrot_t = w; w += align_up(a.B * a.H * kD * 4, 256);
     p.logits = reinterpret_cast<float*>(w);
-    p.probs = w;
-    w += logits_area_bytes(a.B, a.H, p.N);
+    p.chunks = reinterpret_cast<unsigned char*>(w);
+    p.stream_wgs = 0;
+    w += logits_area_bytes(a.B, a.H, a.KVH, p.N);
     const int64_t tiles_max = (p.N + kMinTile - 1) / kMinTile;
     p.part_ml = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * tiles_max * 2 * 4, 256);
     p.part_o = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * tiles_max * kD * 4, 256);
