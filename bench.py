@@ -30,7 +30,7 @@ PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the dominant kernels on the bench workloads, measured with rocprofv3 --pmc
 # FETCH_SIZE and WRITE_SIZE (one pass each), each scaled by the reading for a 512 MiB device copy in the
 # same run (profiles/hbm_traffic_bench_kernels.md).  Counters cannot be read inside this process.
-TRAFFIC_BYTES = {"fwd_pipe_kernel": 0.220e9, "decode_stream_kernel": 2.330e9}
+TRAFFIC_BYTES = {"fwd_pipe_kernel": 0.220e9, "decode_stream_kernel": 2.256e9}
 
 PREFILL = dict(B=2, H=32, KVH=8, D=128, NS=64, S=16384, C=8, Q=2048, theta=5e5, seed=2)
 DECODE = dict(B=16, H=32, KVH=8, D=128, NS=64, S=32768, C=4, Q=1, theta=5e5, seed=3)

@@ -79,7 +79,7 @@ struct DecodeParams {
     unsigned char* chunks;
     int64_t Np;        // the keys rounded up to whole tiles of the streaming kernel
     int stream_wgs;    // workgroups of the streaming kernel
-    float* part_ml;    // (B, H, tiles, 2)
+    float* part_ml;    // (B, H, tiles, 2); after the streaming kernel (chunk, G, 2)
     float* part_o;     // (B, H, tiles, 128)
     float* lse2;       // (B, H)
     int64_t N;         // num_sink + S + 1
@@ -817,7 +817,8 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
         auto flush = [&]() {
             if (!pending) return;
             const int64_t pend_item = tile * nbh + (int64_t)pend_b * KVH + pend_kvh;
-            unsigned char* chunk = p.chunks + ((pend_item - item0) * gridDim.x + blockIdx.x) * (G * (kSK + kD) * 2);
+            const int64_t chunk_i = (pend_item - item0) * gridDim.x + blockIdx.x;
+            unsigned char* chunk = p.chunks + chunk_i * (G * (kSK + kD) * 2);
             if (wave == kStreamProbWave && pg < G)  // every wavefront holds all of them: one stores, 16 bytes a lane
                 *reinterpret_cast<uint4*>(chunk + (pg * kSK + kKpl * kgrp) * 2) = pend_e;
             if (key16 < G) {
@@ -825,10 +826,8 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                 for (int b2 = 0; b2 < kDb; b2++)
                     *reinterpret_cast<uint2*>(chunk + (G * kSK + key16 * kD + 16 * (kDb * wave + b2) + 4 * kq) * 2) = pend_o[b2];
             }
-            if (wave == 0 && kgrp == 0 && pg < G) {
-                const int64_t row = ((int64_t)pend_b * a.H + pend_kvh * G + pg) * p.tiles + tile;
-                *reinterpret_cast<float2*>(p.part_ml + row * 2) = make_float2(pend_m, pend_l);
-            }
+            if (wave == 0 && kgrp == 0 && pg < G)  // maximum and sum: G pairs per chunk, in chunk order
+                *reinterpret_cast<float2*>(p.part_ml + (chunk_i * G + pg) * 2) = make_float2(pend_m, pend_l);
         };
 
         // Loads and stores retire in issue order, so "at most n operations outstanding" with n younger
@@ -1013,8 +1012,13 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
     const int64_t row = blockIdx.x;  // b * H + h
     const int tid = threadIdx.x, d4 = tid & 31, grp = tid >> 5;  // 16 groups of 32 threads, 4 dims per thread
     const float* ml = p.part_ml + row * p.tiles * 2;
+    // streaming kernel: the row's results sit in the chunks of the items (tile, b, kvh)
+    const int64_t nbh_s = a.B * a.KVH, total_s = (int64_t)p.tiles * nbh_s;
+    const int G_s = (int)(a.H / a.KVH), g_s = (int)((row % a.H) % G_s);
+    const int64_t bh_s = (row / a.H) * a.KVH + (row % a.H) / G_s;
+    auto chunk_of = [&](int t) { return stream_chunk_of((int64_t)t * nbh_s + bh_s, total_s, p.stream_wgs); };
     float M = -INFINITY;
-    for (int t = tid; t < p.tiles; t += 512) M = fmaxf(M, ml[2 * t]);
+    for (int t = tid; t < p.tiles; t += 512) M = fmaxf(M, AVG ? p.part_ml[(chunk_of(t) * G_s + g_s) * 2] : ml[2 * t]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
     if ((tid & 63) == 0) sh_m[tid >> 6] = M;
@@ -1027,30 +1031,35 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
     float L = 0.f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     const float4* po = reinterpret_cast<const float4*>(p.part_o + row * p.tiles * kD) + d4;
-    // streaming kernel: the row's averages sit in the chunks of the items (tile, b, kvh)
-    const int64_t nbh_s = a.B * a.KVH, total_s = (int64_t)p.tiles * nbh_s;
-    const int G_s = (int)(a.H / a.KVH);
-    const int64_t bh_s = (row / a.H) * a.KVH + (row % a.H) / G_s;
     const int64_t chunk_bytes = (int64_t)G_s * (kSK + kD) * 2;
-    const int64_t in_chunk = ((int64_t)G_s * kSK + (row % a.H) % G_s * kD) * 2 + d4 * 8;
+    const int64_t in_chunk = ((int64_t)G_s * kSK + g_s * kD) * 2 + d4 * 8;
     constexpr int kBatch = 8;
     for (int t0 = grp; t0 < p.tiles; t0 += 16 * kBatch) {
         float4 v[kBatch];
         float2 w[kBatch];
+        // chunk of tile t0 + 16 u: worked out by lane u of the group (the division is the cost) and handed round
+        int64_t ck_mine = 0;
+        if constexpr (AVG) {
+            const int t = t0 + 16 * (d4 & (kBatch - 1));
+            if (t < p.tiles) ck_mine = chunk_of(t);
+        }
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
             const int t = t0 + 16 * u;
             const bool ok = t < p.tiles;
             if constexpr (AVG) {
                 uint2 r = make_uint2(0u, 0u);
-                if (ok)
-                    r = *reinterpret_cast<const uint2*>(
-                        p.chunks + stream_chunk_of((int64_t)t * nbh_s + bh_s, total_s, p.stream_wgs) * chunk_bytes + in_chunk);
+                w[u] = make_float2(-INFINITY, 0.f);
+                const int64_t ck = __shfl(ck_mine, (tid & 32) + u);
+                if (ok) {
+                    r = *reinterpret_cast<const uint2*>(p.chunks + ck * chunk_bytes + in_chunk);
+                    w[u] = *reinterpret_cast<const float2*>(p.part_ml + (ck * G_s + g_s) * 2);
+                }
                 v[u] = make_float4(Mma16<T>::lo(r.x), Mma16<T>::hi(r.x), Mma16<T>::lo(r.y), Mma16<T>::hi(r.y));
             } else {
                 v[u] = ok ? po[(int64_t)t * (kD / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
+                w[u] = ok ? *reinterpret_cast<const float2*>(ml + 2 * t) : make_float2(-INFINITY, 0.f);
             }
-            w[u] = ok ? *reinterpret_cast<const float2*>(ml + 2 * t) : make_float2(-INFINITY, 0.f);
         }
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
@@ -1138,7 +1147,7 @@ __global__ void __launch_bounds__(256) decode_scores_kernel(DecodeParams p, floa
             if constexpr (PROBS) {  // 2^(logit - tile maximum) from the streaming kernel, and that maximum
                 const int64_t ck = stream_chunk_of((n / kSK) * (a.B * a.KVH) + b * a.KVH + kv, p.tiles * (a.B * a.KVH), p.stream_wgs);
                 const float e = (float)reinterpret_cast<const _Float16*>(p.chunks + ck * (G * (kSK + kD) * 2))[g * kSK + n % kSK];
-                const float m = p.part_ml[(row * p.tiles + n / kSK) * 2];
+                const float m = p.part_ml[(ck * G + g) * 2];
                 pt = e == 0.f ? 0.f : round_t<T>(e * __builtin_amdgcn_exp2f(m - p.lse2[row]));
             } else {
                 pt = round_t<T>(__builtin_amdgcn_exp2f(lg[g] - p.lse2[row]));
@@ -1193,14 +1202,13 @@ __global__ void __launch_bounds__(256) decode_scores_probs_kernel(DecodeParams p
     const int64_t n0 = (idx % per) * 8, kvh = (idx / per) % a.KVH, b = idx / (per * a.KVH);
     if (n0 + 8 <= a.num_sink || n0 >= p.N) return;  // sinks keep no score; padding
     float pr[G][8];
-    const unsigned char* chunk =
-        p.chunks + stream_chunk_of((n0 / kSK) * (a.B * a.KVH) + b * a.KVH + kvh, p.tiles * (a.B * a.KVH), p.stream_wgs) *
-                       (G * (kSK + kD) * 2);
+    const int64_t ck = stream_chunk_of((n0 / kSK) * (a.B * a.KVH) + b * a.KVH + kvh, p.tiles * (a.B * a.KVH), p.stream_wgs);
+    const unsigned char* chunk = p.chunks + ck * (G * (kSK + kD) * 2);
 #pragma unroll
     for (int g = 0; g < G; g++) {
         const int64_t row = b * a.H + kvh * G + g;
         const uint4 raw = *reinterpret_cast<const uint4*>(chunk + (g * kSK + n0 % kSK) * 2);
-        const float c = __builtin_amdgcn_exp2f(p.part_ml[(row * p.tiles + n0 / kSK) * 2] - p.lse2[row]);
+        const float c = __builtin_amdgcn_exp2f(p.part_ml[(ck * G + g) * 2] - p.lse2[row]);
         const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
         for (int k = 0; k < 8; k++) {
