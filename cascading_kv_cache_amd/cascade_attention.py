@@ -126,7 +126,7 @@ def cascade_attention(query_states, key_states, value_states, cache: CascadingKV
         stream = torch.cuda.current_stream(query_states.device).cuda_stream
         _abi.check(lib.ckv_attn(C.byref(a), C.c_void_p(stream)), "ckv_attn")
     if update_cache:
-        cache.update(key_states, value_states, L, score_states=new_scores)
+        cache.update_state(key_states, value_states, L, score_states=new_scores)
     return out, new_scores
 
 

@@ -254,6 +254,12 @@ class CascadingKVCache:
 
     def update(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None):
         """cascading_cache.py:1297-1348."""
+        self.update_state(key_states, value_states, layer_idx, score_states)
+        return self.get_vals(layer_idx)
+
+    def update_state(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None):
+        """``update`` without building the tuple of views it returns (the shifted position row of
+        ``get_vals`` is a device operation of its own); for callers that read the state in place."""
         if score_states is None:
             score_states = torch.zeros(self.max_batch_size, self.heads, key_states.size(2),
                                        device=key_states.device, dtype=key_states.dtype)
@@ -274,4 +280,3 @@ class CascadingKVCache:
         # after the kernel, as in the reference (cascading_cache.py:1343-1346)
         self.seen_tokens_by_layer[layer_idx] += key_states.shape[-2]
         self._seen_host[layer_idx] += key_states.shape[-2]
-        return self.get_vals(layer_idx)

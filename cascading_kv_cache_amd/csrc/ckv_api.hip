@@ -63,26 +63,53 @@ namespace {
 __global__ void __launch_bounds__(1024) chunk_positions_kernel(const int64_t* key_pos, int64_t n_key, int64_t key_shift,
                                                                const int64_t* sink_pos, int64_t n_sink, int64_t q_len,
                                                                int64_t* q_pos) {
-    __shared__ int64_t red[1024];
+    __shared__ int64_t red[16];
     const int tid = threadIdx.x;
     int64_t base = 0;
     if (key_pos || sink_pos) {
         int64_t m = INT64_MIN;
-        for (int64_t i = tid; i < n_key; i += 1024) {
-            const int64_t v = key_pos[i] + key_shift;
+        // one workgroup reads the whole row: eight independent 16-byte loads per thread and trip keep
+        // enough requests in flight for that
+        int64_t i0 = 0;
+        if ((reinterpret_cast<uintptr_t>(key_pos) & 15u) == 0) {
+            const longlong2* kp2 = reinterpret_cast<const longlong2*>(key_pos);
+            const int64_t n2 = n_key / 2;
+            int64_t i = tid;
+            for (; i + 7 * 1024 < n2; i += 8 * 1024) {
+                longlong2 v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = kp2[i + u * 1024];
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    const int64_t a = v[u].x > v[u].y ? v[u].x : v[u].y;
+                    m = a > m ? a : m;
+                }
+            }
+            for (; i < n2; i += 1024) {
+                const longlong2 v = kp2[i];
+                const int64_t a = v.x > v.y ? v.x : v.y;
+                m = a > m ? a : m;
+            }
+            i0 = 2 * n2;
+        }
+        for (int64_t i = i0 + tid; i < n_key; i += 1024) {
+            const int64_t v = key_pos[i];
             m = v > m ? v : m;
         }
+        if (m != INT64_MIN) m += key_shift;
         for (int64_t i = tid; i < n_sink; i += 1024) {
             const int64_t v = sink_pos[i];
             m = v > m ? v : m;
         }
-        red[tid] = m;
-        __syncthreads();
-        for (int off = 512; off > 0; off >>= 1) {
-            if (tid < off) red[tid] = red[tid + off] > red[tid] ? red[tid + off] : red[tid];
-            __syncthreads();
+        for (int off = 32; off > 0; off >>= 1) {
+            const int64_t o = __shfl_xor(m, off);
+            m = o > m ? o : m;
         }
-        base = red[0] + 1;
+        if ((tid & 63) == 0) red[tid >> 6] = m;
+        __syncthreads();
+        m = red[0];
+        for (int w = 1; w < 16; w++) m = red[w] > m ? red[w] : m;
+        base = m + 1;
     }
     for (int64_t i = tid; i < q_len; i += 1024) q_pos[i] = base + i;
 }

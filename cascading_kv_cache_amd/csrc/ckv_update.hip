@@ -27,6 +27,8 @@ namespace ckv {
 namespace {
 
 constexpr int kMaxCascades = 64;
+constexpr int kPlanMaxTokens = 8192;   // incoming tokens one plan launch takes at most
+constexpr int kRingPer = 8;            // kPlanMaxTokens / 1024 threads, and enough for 256 tokens on 256 threads
 
 struct UpdateParams {
     ckv_update_args a;
@@ -36,6 +38,7 @@ struct UpdateParams {
     int32_t* first;        // [N*H][K]
     int32_t* next_of;      // [N*H][S]
     int32_t* pos_flag;     // [N*H]: the call put a token into the cascades, so the position ids change
+    int32_t apply_blocks;  // blocks along x that move rows; the blocks behind them write position ids
 };
 
 // exclusive prefix sum of one flag per thread over the whole workgroup; returns the block total
@@ -81,12 +84,17 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
     int32_t* a_trig[2];
     float* a_score[2];
     unsigned char* ptr = smem;
+    // per cascade, fetched once up front so that no cascade waits for global memory on their account:
+    // the acceptance period and the score of the newest slot left by earlier calls
+    int64_t* per_l = reinterpret_cast<int64_t*>(ptr); ptr += 8 * kMaxCascades;
+    float* lead_l = reinterpret_cast<float*>(ptr); ptr += 4 * kMaxCascades;
     for (int i = 0; i < 2; i++) {
         a_src[i] = reinterpret_cast<int32_t*>(ptr); ptr += 4 * (size_t)cap;
         a_trig[i] = reinterpret_cast<int32_t*>(ptr); ptr += 4 * (size_t)cap;
         a_score[i] = reinterpret_cast<float*>(ptr); ptr += 4 * (size_t)cap;
     }
     uint32_t* eflag = reinterpret_cast<uint32_t*>(ptr); ptr += 4 * (size_t)cap;
+    float* ring_l = reinterpret_cast<float*>(ptr); ptr += 4 * (size_t)cap;  // scores of the oldest ring entries
     int32_t* w_src = reinterpret_cast<int32_t*>(ptr); ptr += 4 * (size_t)(cap + 1);
     float* w_score = reinterpret_cast<float*>(ptr); ptr += 4 * (size_t)(cap + 1);
     int32_t* st_l = reinterpret_cast<int32_t*>(ptr); ptr += 4 * kMaxCascades;
@@ -107,8 +115,15 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
     const int n_sink_new = room < cap ? (int)room : cap;
 
     for (int i = tid; i < C; i += T) {
-        st_l[i] = (int32_t)g_stored[i * A.tracker_stride[2]];
-        sx_l[i] = (int32_t)g_start[i * A.tracker_stride[2]];
+        const int32_t st = (int32_t)g_stored[i * A.tracker_stride[2]];
+        const int32_t sx = (int32_t)g_start[i * A.tracker_stride[2]];
+        st_l[i] = st;
+        sx_l[i] = sx;
+        per_l[i] = A.do_cache_every_n[i];
+        // the plan never writes scores, so the newest slot's score can be read before its cascade's turn
+        lead_l[i] = st > 0 ? load_as_float(A.cache_s, cs_base + ((int64_t)i * W + (sx - 1 + st) % st) * A.cache_s_stride[2],
+                                           A.dtype)
+                           : 0.f;
     }
     // level-0 arrivals: the non-sink tokens of this launch, in order (cascading_cache.py:447-462)
     for (int t = tid; t < cap; t += T) {
@@ -141,12 +156,27 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
     for (int i = 0; i < C && nA > 0; i++) {
         const int64_t l = (int64_t)i * W;
         const int stored0 = st_l[i], start0 = sx_l[i];
-        const int64_t per = A.do_cache_every_n[i];
+        const int64_t per = per_l[i];
         const bool per_small = small && per > 0 && per < (1ll << 31);
         const bool per_pow2 = per > 0 && (per & (per - 1)) == 0;
         const int32_t* Asrc = a_src[cur];
         const int32_t* Atrig = a_trig[cur];
         const float* Ascore = a_score[cur];
+
+        // Scores of the ring entries this call can evict (the oldest ones, at most one per arrival beyond
+        // the free room): requested here, parked in LDS after pass 2, read in pass 3, so their way from
+        // memory runs beside passes 1 and 2.
+        int n_ring = stored0 + nA - (int)W;
+        if (n_ring > stored0 - 1) n_ring = stored0 - 1;
+        if (i + 1 >= C) n_ring = 0;
+        float ring_pre[kRingPer];
+#pragma unroll
+        for (int r = 0; r < kRingPer; r++) {
+            const int j = r * T + tid;
+            ring_pre[r] = j < n_ring ? load_as_float(A.cache_s, cs_base + (l + mod_w(start0 + (int64_t)j)) * A.cache_s_stride[2],
+                                                     A.dtype)
+                                     : 0.f;
+        }
 
         // ---- pass 1: insert flags (accept, or the first arrival of an empty cascade:
         //      cascading_cache.py:471-478, 606) and their running index
@@ -174,7 +204,7 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
         const int p_lead = (int)l + (stored0 > 0 ? (start0 - 1 + stored0) % stored0 : 0);
         if (tid == 0 && stored0 > 0) {
             int ws = p_lead;
-            float wv = load_as_float(A.cache_s, cs_base + (int64_t)p_lead * A.cache_s_stride[2], A.dtype);
+            float wv = lead_l[i];
             for (int b = 0; b < nA && !(eflag[b] & 0x80000000u); b++) {
                 if (Ascore[b] >= wv) { ws = Asrc[b]; wv = Ascore[b]; }
             }
@@ -192,6 +222,11 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
             const int e = (int)(ef & 0x7fffffffu);
             w_src[e + 1] = ws;
             w_score[e + 1] = wv;
+        }
+#pragma unroll
+        for (int r = 0; r < kRingPer; r++) {
+            const int j = r * T + tid;
+            if (j < n_ring) ring_l[j] = ring_pre[r];
         }
         __syncthreads();
 
@@ -211,7 +246,7 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
                 float nv;
                 if (mv < stored0 - 1) {     // an old ring entry nobody touched in this call
                     ns = (int)l + mod_w(start0 + (int64_t)mv);
-                    nv = load_as_float(A.cache_s, cs_base + (int64_t)ns * A.cache_s_stride[2], A.dtype);
+                    nv = ring_l[mv];
                 } else {
                     ns = w_src[mv - stored0 + 1];
                     nv = w_score[mv - stored0 + 1];
@@ -250,10 +285,11 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
 // Position pass (cascading_cache.py:728-774, 129-142) after the plan kernel has updated the trackers:
 // slot j of cascade i gets ((j + seg - start) mod seg) + ub - seg, where seg is the number of stored
 // tokens and ub the ids still to hand out (all stored tokens, less a window per earlier cascade).
-// Grid: (chunks of kPosChunk slots over all cascades, N*H), so the whole chip writes.
+// One 256-thread block per kPosChunk slots of a cascade and (batch, kv head), so the whole chip writes; the
+// blocks ride at the end of the apply kernels' grid (they need the plan's trackers, not the moved rows).
 constexpr int kPosChunk = 2048;
 
-__global__ void __launch_bounds__(256) ckv_update_positions_kernel(UpdateParams p) {
+__device__ inline void update_positions_block(const UpdateParams& p, int blk) {
     const ckv_update_args& A = p.a;
     const int64_t bh = blockIdx.y;
     if (!p.pos_flag[bh]) return;
@@ -261,7 +297,7 @@ __global__ void __launch_bounds__(256) ckv_update_positions_kernel(UpdateParams 
     const int C = A.cascades;
     const int W = (int)A.window_size;
     const int per_c = (W + kPosChunk - 1) / kPosChunk;
-    const int i = (int)blockIdx.x / per_c, j0 = ((int)blockIdx.x % per_c) * kPosChunk;
+    const int i = blk / per_c, j0 = (blk % per_c) * kPosChunk;
     const int64_t* g_stored = A.stored_tokens + n * A.tracker_stride[0] + h * A.tracker_stride[1];
     const int64_t* g_start = A.start_indices + n * A.tracker_stride[0] + h * A.tracker_stride[1];
     int64_t ub = 0;
@@ -305,6 +341,10 @@ template <int LANES>
 __global__ void ckv_update_apply_vec_kernel(UpdateParams p) {
     const ckv_update_args& A = p.a;
     constexpr int kGroups = 256 / LANES;
+    if ((int)blockIdx.x >= p.apply_blocks) {
+        update_positions_block(p, (int)blockIdx.x - p.apply_blocks);
+        return;
+    }
     const int g = blockIdx.x * kGroups + threadIdx.x / LANES;
     const int lane = threadIdx.x % LANES;
     if (g >= p.k_sub) return;
@@ -362,15 +402,19 @@ __global__ void ckv_update_apply_vec_kernel(UpdateParams p) {
     int64_t* og = A.og_pos + n * A.og_pos_stride[0] + h * A.og_pos_stride[1];
     uint8_t* mask = A.mask + n * A.mask_stride[0] + h * A.mask_stride[1];
 
+    // The successor of the next slot is requested together with the displaced row, so a hop costs one
+    // trip to memory, not two.
+    int nd = next_of[d];
     for (int hop = 0; hop <= A.cascades; hop++) {  // a chain visits each cascade at most once
-        const int nd = next_of[d];
         RowPiece old;
         uint32_t o_score = 0;
         int64_t o_og = 0;
+        int nnd = -1;
         uint4* kd = reinterpret_cast<uint4*>(ck + (int64_t)d * row_bytes);
         uint4* vd = reinterpret_cast<uint4*>(cv + (int64_t)d * row_bytes);
         const int64_t sidx = cs_base + (int64_t)d * A.cache_s_stride[2];
         if (nd >= 0) {  // the displaced row lives on elsewhere: pick it up before overwriting
+            nnd = next_of[nd];
             if (active) {
                 old.k = kd[lane];
                 old.v = vd[lane];
@@ -399,6 +443,7 @@ __global__ void ckv_update_apply_vec_kernel(UpdateParams p) {
         c_score = o_score;
         c_og = o_og;
         d = nd;
+        nd = nnd;
     }
 }
 
@@ -408,6 +453,10 @@ template <typename U>
 __global__ void ckv_update_apply_elem_kernel(UpdateParams p) {
     const ckv_update_args& A = p.a;
     constexpr int kPerLane = 8;
+    if ((int)blockIdx.x >= p.apply_blocks) {
+        update_positions_block(p, (int)blockIdx.x - p.apply_blocks);
+        return;
+    }
     const int g = blockIdx.x * (256 / CKV_WAVE) + threadIdx.x / CKV_WAVE;
     const int lane = threadIdx.x % CKV_WAVE;
     if (g >= p.k_sub) return;
@@ -501,7 +550,7 @@ __global__ void ckv_update_apply_elem_kernel(UpdateParams p) {
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline size_t plan_lds_bytes(int cap) {
-    return (size_t)cap * 28 + (size_t)(cap + 1) * 8 + kMaxCascades * 8 + 64 * sizeof(int) + 64;
+    return (size_t)cap * 32 + (size_t)(cap + 1) * 8 + kMaxCascades * 20 + 64 * sizeof(int) + 64;
 }
 
 }  // namespace
@@ -553,9 +602,9 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
         (void)hipGetLastError();
         lds_max = 65536;
     }
-    int qmax = (int)((lds_max - 2048) / 36);
+    int qmax = (int)((lds_max - 4096) / 40);
     qmax = qmax / 64 * 64;
-    if (qmax > 8192) qmax = 8192;
+    if (qmax > kPlanMaxTokens) qmax = kPlanMaxTokens;
     if (qmax < 64) return CKV_ERR_UNSUPPORTED;
 
     UpdateParams p;
@@ -579,21 +628,20 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
         {
             StageScope sc(CKV_STAGE_PLAN, stream);
             hipLaunchKernelGGL(ckv_update_plan_kernel, dim3((unsigned)(A.N * A.H)), dim3(T), lds, stream, p);
-            if (p.do_pos) {
-                const int64_t per_c = (A.window_size + kPosChunk - 1) / kPosChunk;
-                hipLaunchKernelGGL(ckv_update_positions_kernel, dim3((unsigned)(per_c * A.cascades), (unsigned)(A.N * A.H)),
-                                   dim3(256), 0, stream, p);
-            }
         }
         CKV_HIP_TRY(hipGetLastError());
         StageScope sc_apply(CKV_STAGE_APPLY, stream);
+        // the position ids of the last launch of a call are written by extra blocks of the apply grid
+        const unsigned pos_blocks =
+            p.do_pos ? (unsigned)(((A.window_size + kPosChunk - 1) / kPosChunk) * A.cascades) : 0u;
 
         if (vec) {
             const int chunks = (int)(A.HID * es / 16);
             int lanes = 1;
             while (lanes < chunks) lanes *= 2;
             const dim3 block(256);
-            const dim3 grid((unsigned)((ksub + 256 / lanes - 1) / (256 / lanes)), (unsigned)(A.N * A.H));
+            p.apply_blocks = (ksub + 256 / lanes - 1) / (256 / lanes);
+            const dim3 grid((unsigned)p.apply_blocks + pos_blocks, (unsigned)(A.N * A.H));
             switch (lanes) {
                 case 1: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<1>, grid, block, 0, stream, p); break;
                 case 2: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<2>, grid, block, 0, stream, p); break;
@@ -605,7 +653,8 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
             }
         } else {
             const dim3 block(256);
-            const dim3 grid((unsigned)((ksub + 3) / 4), (unsigned)(A.N * A.H));
+            p.apply_blocks = (ksub + 3) / 4;
+            const dim3 grid((unsigned)p.apply_blocks + pos_blocks, (unsigned)(A.N * A.H));
             if (es == 4) {
                 hipLaunchKernelGGL(ckv_update_apply_elem_kernel<uint32_t>, grid, block, 0, stream, p);
             } else {
