@@ -394,6 +394,10 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
         bkv_i = (id & 7) + 8 * (jq / p.n_qt);
         qt_i = jq % p.n_qt;
     }
+    // Later query tiles see more chunk keys, so they go first: the compute units that finish the light
+    // tiles of one round early pick up the heavy tiles of the next (two rounds of workgroups then cost
+    // light + heavy everywhere instead of heavy + heavy on the slowest unit).
+    qt_i = p.n_qt - 1 - qt_i;
     const int64_t bkv = bkv_i;
     const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
     const int m0 = qt_i * p.QT;
