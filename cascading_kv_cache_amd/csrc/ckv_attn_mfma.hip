@@ -124,8 +124,10 @@ __device__ __host__ inline int k_image_off(int r, int c) { return (c >> 1) * 204
 __device__ __host__ inline int v_image_off(int d, int c) { return (c >> 1) * 4096 + (c & 1) * 2048 + d * 16; }
 
 // One block of 256 threads stages key tile `tile_i` for the (b, kvh) units split_i, split_i + n_split, ...:
-// thread = (key = tid/4, quarter = tid%4) owns rotation pairs j = 16*quarter .. 16*quarter+15, i.e.
-// elements [16q,16q+16) and [64+16q, 64+16q+16) of its row.
+// thread = (key = tid/4, quarter = tid%4) owns rotation pairs j = 8q .. 8q+7 and 32+8q .. 32+8q+7, i.e. the
+// 16-byte pieces q, 4+q, 8+q and 12+q of its row: the four threads of a row read (and, for queries, write)
+// 64 contiguous bytes per instruction.
+__device__ inline int stage_pair(int quarter, int i) { return i < 8 ? 8 * quarter + i : 24 + 8 * quarter + i; }
 template <typename T>
 __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int split_i, int n_split, T (*v_lds)[kD + 2]) {
     const int tid = threadIdx.x;
@@ -153,48 +155,66 @@ __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int sp
         const int64_t pos = p.seg[sidx].pos[local] + p.seg[sidx].pos_shift;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const int j = 16 * quarter + i;
+            const int j = stage_pair(quarter, i);
             const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
             fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
         }
     }
     const int64_t nbh = p.B * p.KVH;
+    // the rows of unit bh as this thread's eight 16-byte pieces (zeros past the last key)
+    struct Rows {
+        uint4 lo[2], hi[2], vlo[2], vhi[2];
+    };
+    auto load_rows = [&](int64_t bh, Rows& r) {
+        r.lo[0] = r.lo[1] = r.hi[0] = r.hi[1] = r.vlo[0] = r.vlo[1] = r.vhi[0] = r.vhi[1] = make_uint4(0, 0, 0, 0);
+        if (sidx < 0 || bh >= nbh) return;
+        const int64_t b = bh / p.KVH, kvh = bh % p.KVH;
+        const KeySegment& sg = p.seg[sidx];
+        const int64_t off = b * sg.stride[0] + kvh * sg.stride[1] + local * sg.stride[2];
+        const T* kp = (const T*)sg.k + off;
+        const T* vp = (const T*)sg.v + off;
+        if (sg.stride[3] == 1 && ((reinterpret_cast<uintptr_t>(kp) | reinterpret_cast<uintptr_t>(vp)) & 15) == 0) {
+            r.lo[0] = *reinterpret_cast<const uint4*>(kp + 8 * quarter);
+            r.lo[1] = *reinterpret_cast<const uint4*>(kp + 32 + 8 * quarter);
+            r.hi[0] = *reinterpret_cast<const uint4*>(kp + 64 + 8 * quarter);
+            r.hi[1] = *reinterpret_cast<const uint4*>(kp + 96 + 8 * quarter);
+            r.vlo[0] = *reinterpret_cast<const uint4*>(vp + 8 * quarter);
+            r.vlo[1] = *reinterpret_cast<const uint4*>(vp + 32 + 8 * quarter);
+            r.vhi[0] = *reinterpret_cast<const uint4*>(vp + 64 + 8 * quarter);
+            r.vhi[1] = *reinterpret_cast<const uint4*>(vp + 96 + 8 * quarter);
+        } else {
+            T* l0 = reinterpret_cast<T*>(r.lo);
+            T* h0 = reinterpret_cast<T*>(r.hi);
+            T* vl = reinterpret_cast<T*>(r.vlo);
+            T* vh = reinterpret_cast<T*>(r.vhi);
+            for (int i = 0; i < 16; i++) {
+                l0[i] = kp[stage_pair(quarter, i) * sg.stride[3]];
+                h0[i] = kp[(64 + stage_pair(quarter, i)) * sg.stride[3]];
+                vl[i] = vp[stage_pair(quarter, i) * sg.stride[3]];
+                vh[i] = vp[(64 + stage_pair(quarter, i)) * sg.stride[3]];
+            }
+        }
+    };
+    // The rows of the next unit are requested before this unit's rotation, transposition and stores, so
+    // the workgroup always has loads in flight.
+    Rows nxt;
+    load_rows(split_i, nxt);
     for (int64_t bh = split_i; bh < nbh; bh += n_split) {
         const int64_t b = bh / p.KVH, kvh = bh % p.KVH;
-        uint4 lo[2], hi[2], vlo[2], vhi[2];
-        lo[0] = lo[1] = hi[0] = hi[1] = vlo[0] = vlo[1] = vhi[0] = vhi[1] = make_uint4(0, 0, 0, 0);
+        Rows cur = nxt;
+        load_rows(bh + n_split, nxt);
+        uint4(&lo)[2] = cur.lo;
+        uint4(&hi)[2] = cur.hi;
+        uint4(&vlo)[2] = cur.vlo;
+        uint4(&vhi)[2] = cur.vhi;
         if (sidx >= 0) {
             const KeySegment& sg = p.seg[sidx];
-            const int64_t off = b * sg.stride[0] + kvh * sg.stride[1] + local * sg.stride[2];
-            const T* kp = (const T*)sg.k + off;
-            const T* vp = (const T*)sg.v + off;
-            if (sg.stride[3] == 1 && ((reinterpret_cast<uintptr_t>(kp) | reinterpret_cast<uintptr_t>(vp)) & 15) == 0) {
-                lo[0] = *reinterpret_cast<const uint4*>(kp + 16 * quarter);
-                lo[1] = *reinterpret_cast<const uint4*>(kp + 16 * quarter + 8);
-                hi[0] = *reinterpret_cast<const uint4*>(kp + 64 + 16 * quarter);
-                hi[1] = *reinterpret_cast<const uint4*>(kp + 64 + 16 * quarter + 8);
-                vlo[0] = *reinterpret_cast<const uint4*>(vp + 16 * quarter);
-                vlo[1] = *reinterpret_cast<const uint4*>(vp + 16 * quarter + 8);
-                vhi[0] = *reinterpret_cast<const uint4*>(vp + 64 + 16 * quarter);
-                vhi[1] = *reinterpret_cast<const uint4*>(vp + 64 + 16 * quarter + 8);
-            } else {
-                T* l0 = reinterpret_cast<T*>(lo);
-                T* h0 = reinterpret_cast<T*>(hi);
-                T* vl = reinterpret_cast<T*>(vlo);
-                T* vh = reinterpret_cast<T*>(vhi);
-                for (int i = 0; i < 16; i++) {
-                    l0[i] = kp[(16 * quarter + i) * sg.stride[3]];
-                    h0[i] = kp[(64 + 16 * quarter + i) * sg.stride[3]];
-                    vl[i] = vp[(16 * quarter + i) * sg.stride[3]];
-                    vh[i] = vp[(64 + 16 * quarter + i) * sg.stride[3]];
-                }
-            }
             if (rotate) {
                 if (!p.shared_pos) {
                     const int64_t pos = sg.pos[b * sg.pos_stride[0] + kvh * sg.pos_stride[1] + local] + sg.pos_shift;
 #pragma unroll
                     for (int i = 0; i < 16; i++) {
-                        const int j = 16 * quarter + i;
+                        const int j = stage_pair(quarter, i);
                         const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
                         fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
                     }
@@ -210,10 +230,10 @@ __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int sp
             }
         }
         char* kimg = (char*)p.kr + (bh * (p.n_pad / kBN) + tile) * (int64_t)(kD * kBN * sizeof(T));
-        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 2 * quarter)) = lo[0];
-        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 2 * quarter + 1)) = lo[1];
-        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 8 + 2 * quarter)) = hi[0];
-        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 9 + 2 * quarter)) = hi[1];
+        *reinterpret_cast<uint4*>(kimg + k_image_off(key, quarter)) = lo[0];
+        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 4 + quarter)) = lo[1];
+        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 8 + quarter)) = hi[0];
+        *reinterpret_cast<uint4*>(kimg + k_image_off(key, 12 + quarter)) = hi[1];
 
         // V: through LDS into the transposed tile
         __syncthreads();
@@ -222,8 +242,8 @@ __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int sp
             const T* vh = reinterpret_cast<const T*>(vhi);
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                v_lds[key][16 * quarter + i] = vl[i];
-                v_lds[key][64 + 16 * quarter + i] = vh[i];
+                v_lds[key][stage_pair(quarter, i)] = vl[i];
+                v_lds[key][64 + stage_pair(quarter, i)] = vh[i];
             }
         }
         __syncthreads();
@@ -273,65 +293,80 @@ __device__ inline void stage_q_block(const StageQParams& p, int blk, int share_i
         const int64_t pos = p.q_pos[m];
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const int j = 16 * quarter + i;
+            const int j = stage_pair(quarter, i);
             const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
             fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
         }
     }
     const int64_t nbh = p.rows / p.Q;
-    for (int64_t bh = share_i; bh < nbh; bh += n_share) {
+    struct Row {
+        T lo[16], hi[16];
+    };
+    auto load_row = [&](int64_t bh, Row& r) {
+        if (bh >= nbh) return;
         const int64_t b = bh / p.H, h = bh % p.H;
         const T* src = (const T*)p.q + b * p.stride[0] + h * p.stride[1] + m * p.stride[2];
-        T lo[16], hi[16];
         if (p.vec) {  // unit stride and 16-byte aligned rows
-            reinterpret_cast<uint4*>(lo)[0] = *reinterpret_cast<const uint4*>(src + 16 * quarter);
-            reinterpret_cast<uint4*>(lo)[1] = *reinterpret_cast<const uint4*>(src + 16 * quarter + 8);
-            reinterpret_cast<uint4*>(hi)[0] = *reinterpret_cast<const uint4*>(src + 64 + 16 * quarter);
-            reinterpret_cast<uint4*>(hi)[1] = *reinterpret_cast<const uint4*>(src + 64 + 16 * quarter + 8);
+            reinterpret_cast<uint4*>(r.lo)[0] = *reinterpret_cast<const uint4*>(src + 8 * quarter);
+            reinterpret_cast<uint4*>(r.lo)[1] = *reinterpret_cast<const uint4*>(src + 32 + 8 * quarter);
+            reinterpret_cast<uint4*>(r.hi)[0] = *reinterpret_cast<const uint4*>(src + 64 + 8 * quarter);
+            reinterpret_cast<uint4*>(r.hi)[1] = *reinterpret_cast<const uint4*>(src + 96 + 8 * quarter);
         } else {
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                lo[i] = src[(16 * quarter + i) * p.stride[3]];
-                hi[i] = src[(64 + 16 * quarter + i) * p.stride[3]];
+                r.lo[i] = src[stage_pair(quarter, i) * p.stride[3]];
+                r.hi[i] = src[(64 + stage_pair(quarter, i)) * p.stride[3]];
             }
         }
-        // the softmax scale (times log2 e) rides on the staged queries: one rounding to the tensor
-        // dtype after rotation and scaling, and the attention kernels exponentiate the products as
-        // they come out of the matrix pipe
+    };
+    // the softmax scale (times log2 e) rides on the staged queries: one rounding to the tensor
+    // dtype after rotation and scaling, and the attention kernels exponentiate the products as
+    // they come out of the matrix pipe
+    auto finish_row = [&](int64_t bh, Row& r) {
+        if (bh >= nbh) return;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const float x1 = Elem<T>::to_float(lo[i]), x2 = Elem<T>::to_float(hi[i]);
+            const float x1 = Elem<T>::to_float(r.lo[i]), x2 = Elem<T>::to_float(r.hi[i]);
             if (p.q_pos) {
-                lo[i] = Elem<T>::from_float((x1 * cs[i] - x2 * sn[i]) * p.qscale);
-                hi[i] = Elem<T>::from_float((x2 * cs[i] + x1 * sn[i]) * p.qscale);
+                r.lo[i] = Elem<T>::from_float((x1 * cs[i] - x2 * sn[i]) * p.qscale);
+                r.hi[i] = Elem<T>::from_float((x2 * cs[i] + x1 * sn[i]) * p.qscale);
             } else {
-                lo[i] = Elem<T>::from_float(x1 * p.qscale);
-                hi[i] = Elem<T>::from_float(x2 * p.qscale);
+                r.lo[i] = Elem<T>::from_float(x1 * p.qscale);
+                r.hi[i] = Elem<T>::from_float(x2 * p.qscale);
             }
         }
         T* dst = (T*)p.qr + (bh * p.Q + m) * kD;
-        *reinterpret_cast<uint4*>(dst + 16 * quarter) = reinterpret_cast<uint4*>(lo)[0];
-        *reinterpret_cast<uint4*>(dst + 16 * quarter + 8) = reinterpret_cast<uint4*>(lo)[1];
-        *reinterpret_cast<uint4*>(dst + 64 + 16 * quarter) = reinterpret_cast<uint4*>(hi)[0];
-        *reinterpret_cast<uint4*>(dst + 64 + 16 * quarter + 8) = reinterpret_cast<uint4*>(hi)[1];
+        *reinterpret_cast<uint4*>(dst + 8 * quarter) = reinterpret_cast<uint4*>(r.lo)[0];
+        *reinterpret_cast<uint4*>(dst + 32 + 8 * quarter) = reinterpret_cast<uint4*>(r.lo)[1];
+        *reinterpret_cast<uint4*>(dst + 64 + 8 * quarter) = reinterpret_cast<uint4*>(r.hi)[0];
+        *reinterpret_cast<uint4*>(dst + 96 + 8 * quarter) = reinterpret_cast<uint4*>(r.hi)[1];
+    };
+    // two rows per trip, both requested before either is rotated: a block is a chain of trips to
+    // memory, and this halves it
+    for (int64_t bh = share_i; bh < nbh; bh += 2 * n_share) {
+        Row r0, r1;
+        load_row(bh, r0);
+        load_row(bh + n_share, r1);
+        finish_row(bh, r0);
+        finish_row(bh + n_share, r1);
     }
 }
 
-// One launch stages queries and keys: the two are independent, and side by side the shorter one costs
-// nothing.  1-D grid: the query blocks (q_bx x q_by) first, then the key blocks (k_bx x k_by).
+// One launch stages queries and keys: the two are independent.  1-D grid: the key blocks (k_bx x k_by)
+// first, then the query blocks (q_bx x q_by), which are short and fill the ragged end of the key blocks.
 struct StageGrid {
     int q_bx, q_by, k_bx, k_by;
 };
 template <typename T>
 __global__ void __launch_bounds__(256) stage_kernel(StageParams sp, StageQParams sq, StageGrid g) {
     __shared__ T v_lds[kBN][kD + 2];
-    const int nq = g.q_bx * g.q_by;
+    const int nk = g.k_bx * g.k_by;
     int id = blockIdx.x;
-    if (id < nq) {
-        stage_q_block<T>(sq, id % g.q_bx, id / g.q_bx, g.q_by);
-    } else {
-        id -= nq;
+    if (id < nk) {
         stage_keys_block<T>(sp, id % g.k_bx, id / g.k_bx, g.k_by, v_lds);
+    } else {
+        id -= nk;
+        stage_q_block<T>(sq, id % g.q_bx, id / g.q_bx, g.q_by);
     }
 }
 
@@ -1131,7 +1166,15 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         sp.tile_vis = mp.tile_vis;
         sp.B = mp.B; sp.KVH = mp.KVH; sp.n = n; sp.n_pad = n_pad;
         const int64_t nbh = mp.B * mp.KVH;
-        int64_t splits = mp.shared_pos ? (nbh < 4 ? nbh : 4) : nbh;
+        // shared positions: a block walks several (b, kvh) units with one set of cos/sin, the next unit's rows
+        // always on their way
+        int64_t splits = nbh;
+        if (mp.shared_pos) {  // about two workgroups per compute unit
+            const int64_t tiles = n_pad / kBN;
+            splits = (512 + tiles - 1) / tiles;
+            if (splits < 2) splits = 2;
+            if (splits > nbh) splits = nbh;
+        }
         if (splits > 65535) splits = 65535;
         StageQParams sq;
         sq.q = mp.q;
