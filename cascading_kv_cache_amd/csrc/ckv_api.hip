@@ -19,6 +19,24 @@ static bool prof_wanted(int stage) {
     return g_prof_level == 1 || (g_prof_level == 2 && (stage == CKV_STAGE_FWD || stage == CKV_STAGE_DECODE));
 }
 
+bool prof_kernel_events_wanted(int stage) {
+    return g_prof_level == 2 && (stage == CKV_STAGE_FWD || stage == CKV_STAGE_DECODE);
+}
+
+void prof_kernel_events(int stage, hipEvent_t* start, hipEvent_t* stop) {
+    *start = *stop = nullptr;
+    if (!prof_kernel_events_wanted(stage)) return;
+    hipEvent_t e0, e1;
+    if (hipEventCreate(&e0) != hipSuccess) return;
+    if (hipEventCreate(&e1) != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return;
+    }
+    g_spans.push_back(Span{stage, e0, e1});
+    *start = e0;
+    *stop = e1;
+}
+
 void prof_begin(int stage, hipStream_t stream) {
     if (!prof_wanted(stage)) return;
     hipEvent_t e;

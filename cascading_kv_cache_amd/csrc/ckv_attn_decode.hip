@@ -1292,7 +1292,7 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
         CKV_HIP_TRY(hipGetLastError());
     }
     {
-        StageScope sc(CKV_STAGE_DECODE, stream);
+        StageScope sc(CKV_STAGE_DECODE, stream, use_stream);
         const int64_t nbh = a.B * a.KVH;
         // enough workgroups to fill the chip, few enough that cos/sin are amortised over many rows
         int64_t groups = p.shared_pos ? (2048 + p.tiles - 1) / p.tiles : nbh;
@@ -1319,7 +1319,13 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
                 if (wgs > kStreamMaxWgs) wgs = kStreamMaxWgs;
                 if (wgs > p.tiles * nbh) wgs = p.tiles * nbh;
                 p.stream_wgs = (int)wgs;
-                hipLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads), lds_s, stream, p);
+                hipEvent_t ev0, ev1;
+                prof_kernel_events(CKV_STAGE_DECODE, &ev0, &ev1);
+                if (ev0)
+                    hipExtLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads),
+                                          (uint32_t)lds_s, stream, ev0, ev1, 0u, p);
+                else
+                    hipLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads), lds_s, stream, p);
             }
         } else {
             if (lds > 48 * 1024) {

@@ -1205,7 +1205,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
     }
     const int G = (int)(mp.H / mp.KVH);
     {
-        StageScope sc(CKV_STAGE_FWD, stream);
+        StageScope sc(CKV_STAGE_FWD, stream, true);
         FwdParams fp;
         fp.qr = mp.qr; fp.kr = mp.kr; fp.vt = mp.vt; fp.tile_vis = mp.tile_vis;
         fp.out = mp.out;
@@ -1222,8 +1222,11 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         fp.n_qt = (int)grid.x;
         fp.xcd_aware = grid.y % 8 == 0;
-        if (fp.xcd_aware) hipLaunchKernelGGL(fwd_pipe_kernel<T>, dim3(grid.x * grid.y), dim3(512), lds, stream, fp);
-        else hipLaunchKernelGGL(fwd_pipe_kernel<T>, grid, dim3(512), lds, stream, fp);
+        hipEvent_t ev0, ev1;
+        prof_kernel_events(CKV_STAGE_FWD, &ev0, &ev1);
+        const dim3 launch_grid = fp.xcd_aware ? dim3(grid.x * grid.y) : grid;
+        if (ev0) hipExtLaunchKernelGGL(fwd_pipe_kernel<T>, launch_grid, dim3(512), (uint32_t)lds, stream, ev0, ev1, 0u, fp);
+        else hipLaunchKernelGGL(fwd_pipe_kernel<T>, launch_grid, dim3(512), lds, stream, fp);
         CKV_HIP_TRY(hipGetLastError());
     }
     if (mp.colsum) {

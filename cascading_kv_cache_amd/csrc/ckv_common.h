@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
@@ -65,11 +66,24 @@ struct Elem<__half> {
 // stage timing hooks (ckv_profile_enable / ckv_profile_read); no-ops while disabled
 void prof_begin(int stage, hipStream_t stream);
 void prof_end(int stage, hipStream_t stream);
+// Timing of a single kernel by events attached to its own dispatch (hipExtLaunchKernelGGL): unlike an
+// event record in the stream, this puts nothing between the kernel and its neighbours.  Used when only
+// the attention main kernels are timed.
+bool prof_kernel_events_wanted(int stage);
+void prof_kernel_events(int stage, hipEvent_t* start, hipEvent_t* stop);  // both null unless wanted
 struct StageScope {
     int stage;
     hipStream_t stream;
-    StageScope(int s, hipStream_t st) : stage(s), stream(st) { prof_begin(s, st); }
-    ~StageScope() { prof_end(stage, stream); }
+    bool own;
+    // kernel_events: the stage is a single kernel whose launch site takes its start / stop events from
+    // prof_kernel_events; the scope then records nothing itself when only main kernels are timed
+    StageScope(int s, hipStream_t st, bool kernel_events = false)
+        : stage(s), stream(st), own(!(kernel_events && prof_kernel_events_wanted(s))) {
+        if (own) prof_begin(s, st);
+    }
+    ~StageScope() {
+        if (own) prof_end(stage, stream);
+    }
 };
 
 inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
