@@ -24,10 +24,12 @@ def default_inv_freq(head_dim: int, theta: float, device) -> torch.Tensor:
     return inv.to(device)
 
 
-def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_pos: bool = False) -> torch.Tensor:
+def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_pos: bool = False,
+                    _stream: Optional[int] = None) -> torch.Tensor:
     """Position ids of the incoming chunk (cascade_attention.py:119-150) without a host sync:
     0.. on the first call, otherwise one past the largest id among sinks and cache slots
-    (stale and masked entries included, as in the reference).  One small kernel of the library."""
+    (stale and masked entries included, as in the reference).  One small kernel of the library.
+    ``_stream``: raw stream handle when the caller already holds the device context."""
     _require_device(cache.key_cache[layer_idx], "the cache")
     dev = cache.key_cache[layer_idx].device
     out = torch.empty(q_len, device=dev, dtype=torch.long)
@@ -45,11 +47,60 @@ def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_p
             srow = cache.sink_pos[layer_idx][0, 0]
             assert srow.is_contiguous()
             sink_ptr, n_sink = srow.data_ptr(), srow.numel()
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
-        _abi.check(_abi.lib().ckv_chunk_positions(key_ptr, n_key, shift, sink_ptr, n_sink, q_len, out.data_ptr(), stream),
+    if _stream is None:
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            _abi.check(_abi.lib().ckv_chunk_positions(key_ptr, n_key, shift, sink_ptr, n_sink, q_len, out.data_ptr(), stream),
+                       "ckv_chunk_positions")
+    else:
+        _abi.check(_abi.lib().ckv_chunk_positions(key_ptr, n_key, shift, sink_ptr, n_sink, q_len, out.data_ptr(), _stream),
                    "ckv_chunk_positions")
     return out
+
+
+def _describe_attention(query_states, key_states, value_states, cache, L, inv_freq, reduction, homogeneous_heads,
+                        do_og_pos, scale, out, new_scores):
+    """The argument block of ``ckv_attn`` for one layer and input layout; everything in it except the
+    pointers of the per-call tensors and the sink shift stays valid from call to call."""
+    lib = _abi.lib()
+    B, H, Q, D = query_states.shape
+    KVH = key_states.size(1)
+    NS, S = cache.num_sink_tokens, cache.max_seq_len[L]
+    a = _abi.AttnArgs()
+    _abi.set_strides(a.q_stride, query_states)
+    _abi.set_strides(a.kv_new_stride, key_states)
+    a.sink_k, a.sink_v = cache.sink_keys[L].data_ptr(), cache.sink_values[L].data_ptr()
+    _abi.set_strides(a.sink_stride, cache.sink_keys[L])
+    a.cache_k, a.cache_v = cache.key_cache[L].data_ptr(), cache.value_cache[L].data_ptr()
+    _abi.set_strides(a.cache_stride, cache.key_cache[L])
+    assert cache.sink_mask[L].stride(-1) == 1 and cache.mask[L].stride(-1) == 1
+    a.sink_mask, a.mask = cache.sink_mask[L].data_ptr(), cache.mask[L].data_ptr()  # row [0, 0]
+    assert cache.sink_pos[L].stride(-1) == 1 and cache.pos[L].stride(-1) == 1 and cache.og_pos[L].stride(-1) == 1
+    a.sink_pos = cache.sink_pos[L].data_ptr()
+    a.sink_pos_stride[0], a.sink_pos_stride[1] = 0, 0
+    if do_og_pos:  # every (batch, head) rotates its keys at their original positions (:161-164)
+        a.pos = cache.og_pos[L].data_ptr()
+        a.pos_stride[0], a.pos_stride[1] = cache.og_pos[L].stride(0), cache.og_pos[L].stride(1)
+    else:
+        a.pos = cache.pos[L].data_ptr()
+        a.pos_stride[0], a.pos_stride[1] = 0, 0
+    a.cache_s = cache.score_cache[L].data_ptr()
+    _abi.set_strides(a.cache_s_stride, cache.score_cache[L])
+    _abi.set_strides(a.out_stride, out)
+    _abi.set_strides(a.new_scores_stride, new_scores)
+    a.lse = None
+    a.B, a.H, a.KVH, a.Q, a.D = B, H, KVH, Q, D
+    a.num_sink, a.S = NS, S
+    a.scale = float(scale)
+    a.rope_theta = 0.0
+    assert inv_freq.dtype == torch.float32 and inv_freq.numel() == D // 2 and inv_freq.is_contiguous()
+    a.inv_freq = inv_freq.data_ptr()
+    a.beta = float(cache.beta)
+    a.head_reduction = _abi.CKV_REDUCE[reduction]
+    a.homogeneous_heads = int(bool(homogeneous_heads))
+    a.dtype = _abi.dtype_code(query_states.dtype)
+    a._need = lib.ckv_attn_workspace_bytes(B, H, KVH, Q, D, NS, S, a.dtype)
+    return a
 
 
 def cascade_attention(query_states, key_states, value_states, cache: CascadingKVCache, layer_idx: int,
@@ -69,64 +120,42 @@ def cascade_attention(query_states, key_states, value_states, cache: CascadingKV
     assert key_states.shape == (B, KVH, Q, D) and value_states.shape == (B, KVH, Q, D)
     assert _abi.same_layout(key_states, value_states)
     dtype = query_states.dtype
+    dev = query_states.device
     L = layer_idx
-    NS, S = cache.num_sink_tokens, cache.max_seq_len[L]
     reduction = head_reduction or cache.head_reduction
     if scale is None:
         scale = 1 / math.sqrt(D)
 
-    q_pos = chunk_positions(cache, L, Q, do_og_pos)
-    out = torch.empty((B, H, Q, D), dtype=dtype, device=query_states.device)
-    new_scores = torch.empty((B, KVH, Q), dtype=dtype, device=query_states.device)
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        q_pos = chunk_positions(cache, L, Q, do_og_pos, _stream=stream)
+        out = torch.empty((B, H, Q, D), dtype=dtype, device=dev)
+        new_scores = torch.empty((B, KVH, Q), dtype=dtype, device=dev)
 
-    a = _abi.AttnArgs()
-    a.q = query_states.data_ptr()
-    _abi.set_strides(a.q_stride, query_states)
-    a.k_new, a.v_new = key_states.data_ptr(), value_states.data_ptr()
-    _abi.set_strides(a.kv_new_stride, key_states)
-    a.sink_k, a.sink_v = cache.sink_keys[L].data_ptr(), cache.sink_values[L].data_ptr()
-    _abi.set_strides(a.sink_stride, cache.sink_keys[L])
-    a.cache_k, a.cache_v = cache.key_cache[L].data_ptr(), cache.value_cache[L].data_ptr()
-    _abi.set_strides(a.cache_stride, cache.key_cache[L])
-    assert cache.sink_mask[L].stride(-1) == 1 and cache.mask[L].stride(-1) == 1
-    a.sink_mask, a.mask = cache.sink_mask[L].data_ptr(), cache.mask[L].data_ptr()  # row [0, 0]
-    a.q_pos = q_pos.data_ptr()
-    assert cache.sink_pos[L].stride(-1) == 1 and cache.pos[L].stride(-1) == 1 and cache.og_pos[L].stride(-1) == 1
-    a.sink_pos = cache.sink_pos[L].data_ptr()
-    a.sink_pos_stride[0], a.sink_pos_stride[1] = 0, 0
-    if do_og_pos:  # every (batch, head) rotates its keys at their original positions (:161-164)
-        a.pos = cache.og_pos[L].data_ptr()
-        a.pos_stride[0], a.pos_stride[1] = cache.og_pos[L].stride(0), cache.og_pos[L].stride(1)
-        a.pos_shift = 0
-    else:
-        a.pos = cache.pos[L].data_ptr()
-        a.pos_stride[0], a.pos_stride[1] = 0, 0
-        a.pos_shift = cache.pos_shift(L)
-    a.cache_s = cache.score_cache[L].data_ptr()
-    _abi.set_strides(a.cache_s_stride, cache.score_cache[L])
-    a.out = out.data_ptr()
-    _abi.set_strides(a.out_stride, out)
-    a.new_scores = new_scores.data_ptr()
-    _abi.set_strides(a.new_scores_stride, new_scores)
-    a.lse = None
-    a.B, a.H, a.KVH, a.Q, a.D = B, H, KVH, Q, D
-    a.num_sink, a.S = NS, S
-    a.scale = float(scale)
-    a.rope_theta = 0.0
-    assert inv_freq.dtype == torch.float32 and inv_freq.numel() == D // 2 and inv_freq.is_contiguous()
-    a.inv_freq = inv_freq.data_ptr()
-    a.beta = float(cache.beta)
-    a.head_reduction = _abi.CKV_REDUCE[reduction]
-    a.homogeneous_heads = int(bool(homogeneous_heads))
-    a.dtype = _abi.dtype_code(dtype)
-    need = lib.ckv_attn_workspace_bytes(B, H, KVH, Q, D, NS, S, a.dtype)
-    ws = workspace(query_states.device, need)
-    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
-    with torch.cuda.device(query_states.device):
-        stream = torch.cuda.current_stream(query_states.device).cuda_stream
+        # the argument block is described once per layer and input layout (single-token steps at batch 1
+        # are bound by this host code, not by the device)
+        key = (L, query_states.shape, query_states.stride(), key_states.shape, key_states.stride(), dtype,
+               key_states.dtype, value_states.dtype, dev, key_states.device, value_states.device, reduction,
+               bool(homogeneous_heads), bool(do_og_pos), float(scale), float(cache.beta), inv_freq.data_ptr(),
+               inv_freq.dtype, cache._state_key(L))
+        a = cache._attn_memo.get(key)
+        if a is None:
+            a = _describe_attention(query_states, key_states, value_states, cache, L, inv_freq, reduction,
+                                    homogeneous_heads, do_og_pos, scale, out, new_scores)
+            if len(cache._attn_memo) > 64:
+                cache._attn_memo.clear()
+            cache._attn_memo[key] = a
+        a.q = query_states.data_ptr()
+        a.k_new, a.v_new = key_states.data_ptr(), value_states.data_ptr()
+        a.q_pos = q_pos.data_ptr()
+        a.pos_shift = 0 if do_og_pos else cache.pos_shift(L)
+        a.out = out.data_ptr()
+        a.new_scores = new_scores.data_ptr()
+        ws = workspace(dev, a._need)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
         _abi.check(lib.ckv_attn(C.byref(a), C.c_void_p(stream)), "ckv_attn")
-    if update_cache:
-        cache.update_state(key_states, value_states, L, score_states=new_scores)
+        if update_cache:
+            cache.update_state(key_states, value_states, L, score_states=new_scores, _stream=stream)
     return out, new_scores
 
 

@@ -211,6 +211,7 @@ class CascadingKVCache:
         if self.verbose:
             print(f"INIT CLEAN HIP CACHE {self.cascade_func=}")
         self._seen_tokens = 0
+        self._update_memo, self._attn_memo = {}, {}  # argument blocks described once per input layout
         # host mirror of seen_tokens_by_layer: lets callers branch without a device sync
         self._seen_host = [0 for _ in range(L)]
         self.seen_tokens_by_layer = torch.zeros(L, dtype=torch.long, device=dev)
@@ -252,31 +253,64 @@ class CascadingKVCache:
             self.og_pos[layer_idx],
         )
 
+    def _state_key(self, L: int):
+        """Identity of the layer's state tensors: a memoised argument block is only reused while the
+        cache still holds the very tensors it was described from."""
+        return (id(self.key_cache[L]), id(self.value_cache[L]), id(self.score_cache[L]), id(self.sink_keys[L]),
+                id(self.sink_values[L]), id(self.mask[L]), id(self.sink_mask[L]), id(self.pos[L]), id(self.og_pos[L]),
+                id(self.sink_pos[L]), id(self.stored_tokens[L]), id(self.start_indices[L]), id(self.stored_sinks[L]),
+                id(self.do_cache_every_n[L]), id(self.seen_tokens_by_layer), self.key_cache[L].data_ptr())
+
     def update(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None):
         """cascading_cache.py:1297-1348."""
         self.update_state(key_states, value_states, layer_idx, score_states)
         return self.get_vals(layer_idx)
 
-    def update_state(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None):
+    def update_state(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None,
+                     _stream: Optional[int] = None):
         """``update`` without building the tuple of views it returns (the shifted position row of
-        ``get_vals`` is a device operation of its own); for callers that read the state in place."""
+        ``get_vals`` is a device operation of its own); for callers that read the state in place.
+
+        The argument block of ``ckv_update`` is described once per layer and input layout and reused:
+        between two calls of the same shape only the three input pointers change (single-token steps
+        at batch 1 are bound by this host code, not by the device).  ``_stream``: raw stream handle when
+        the caller already holds the device context."""
         if score_states is None:
             score_states = torch.zeros(self.max_batch_size, self.heads, key_states.size(2),
                                        device=key_states.device, dtype=key_states.dtype)
         if layer_idx == 0:
             self._seen_tokens += key_states.shape[-2]
 
-        sink_cache(
-            key_states, value_states, score_states,
-            self.sink_keys[layer_idx], self.sink_values[layer_idx],
-            self.sink_mask[layer_idx], self.sink_pos[layer_idx],
-            self.key_cache[layer_idx], self.value_cache[layer_idx], self.score_cache[layer_idx],
-            self.mask[layer_idx], self.pos[layer_idx], self.og_pos[layer_idx],
-            self.do_cache[layer_idx], self.do_cache_every_n[layer_idx],
-            self.stored_tokens[layer_idx], self.start_indices[layer_idx], self.stored_sinks[layer_idx],
-            self.num_sink_tokens, self.window_length[layer_idx],
-            self.seen_tokens_by_layer[layer_idx], self.max_seq_len[layer_idx], self.eager_fill,
-        )
+        L = layer_idx
+        key = (L, key_states.shape, key_states.stride(), value_states.shape, value_states.stride(),
+               score_states.shape, score_states.stride(), key_states.dtype, value_states.dtype, score_states.dtype,
+               key_states.device, value_states.device, score_states.device, self._state_key(L))
+        memo = self._update_memo
+        a = memo.get(key)
+        if a is None:
+            _require_device(key_states, "k")
+            a = _abi.fill_update_args(
+                key_states, value_states, score_states,
+                self.sink_keys[L], self.sink_values[L], self.sink_mask[L], self.sink_pos[L],
+                self.key_cache[L], self.value_cache[L], self.score_cache[L],
+                self.mask[L], self.pos[L], self.og_pos[L], self.do_cache_every_n[L],
+                self.stored_tokens[L], self.start_indices[L], self.stored_sinks[L],
+                self.num_sink_tokens, self.window_length[L], self.seen_tokens_by_layer[L], self.max_seq_len[L],
+                self.eager_fill)
+            a._need = _abi.lib().ckv_update_workspace_bytes(a.N, a.H, a.K, a.max_seq_len, a.cascades)
+            if len(memo) > 64:
+                memo.clear()
+            memo[key] = a
+        else:
+            a.k, a.v, a.s = key_states.data_ptr(), value_states.data_ptr(), score_states.data_ptr()
+        ws = workspace(key_states.device, a._need)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+        if _stream is None:
+            with torch.cuda.device(key_states.device):
+                stream = torch.cuda.current_stream(key_states.device).cuda_stream
+                _abi.check(_abi.lib().ckv_update(C.byref(a), C.c_void_p(stream)), "ckv_update")
+        else:
+            _abi.check(_abi.lib().ckv_update(C.byref(a), C.c_void_p(_stream)), "ckv_update")
         # after the kernel, as in the reference (cascading_cache.py:1343-1346)
         self.seen_tokens_by_layer[layer_idx] += key_states.shape[-2]
         self._seen_host[layer_idx] += key_states.shape[-2]
