@@ -129,7 +129,7 @@ __device__ __host__ inline int v_image_off(int d, int c) { return (c >> 1) * 409
 // 64 contiguous bytes per instruction.
 __device__ inline int stage_pair(int quarter, int i) { return i < 8 ? 8 * quarter + i : 24 + 8 * quarter + i; }
 template <typename T>
-__device__ inline void stage_keys_block(const StageParams& p, int tile_i, int split_i, int n_split, T (*v_lds)[kD + 2]) {
+__device__ inline void stage_keys_block(const StageParams& p, int tile_i, int split_i, int n_split, uint32_t (*v_lds)[kD / 2 + 1]) {
     const int tid = threadIdx.x;
     const int key = tid >> 2, quarter = tid & 3;
     const int64_t tile = tile_i;
@@ -235,33 +235,41 @@ __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int sp
         *reinterpret_cast<uint4*>(kimg + k_image_off(key, 8 + quarter)) = hi[0];
         *reinterpret_cast<uint4*>(kimg + k_image_off(key, 12 + quarter)) = hi[1];
 
-        // V: through LDS into the transposed tile
+        // V: through LDS into the transposed tile.  A thread holds elements j and j + 64 of its key row for
+        // the same 16 values of j, so the two travel as one dword: 16 four-byte LDS writes per thread, and on
+        // the way out thread (j, group of 16 key slots) reads 16 dwords and owns 32 bytes of dim row j and of
+        // dim row j + 64, which the 64 lanes of a wavefront store as 1 KiB runs of the image.
         __syncthreads();
         {
-            const T* vl = reinterpret_cast<const T*>(vlo);
-            const T* vh = reinterpret_cast<const T*>(vhi);
+            const uint16_t* vl = reinterpret_cast<const uint16_t*>(vlo);
+            const uint16_t* vh = reinterpret_cast<const uint16_t*>(vhi);
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                v_lds[key][stage_pair(quarter, i)] = vl[i];
-                v_lds[key][64 + stage_pair(quarter, i)] = vh[i];
-            }
+            for (int i = 0; i < 16; i++) v_lds[key][stage_pair(quarter, i)] = (uint32_t)vl[i] | ((uint32_t)vh[i] << 16);
         }
         __syncthreads();
         char* vimg = (char*)p.vt + (bh * (p.n_pad / kBN) + tile) * (int64_t)(kD * kBN * sizeof(T));
-        // thread -> (d = tid/2, half of the 64 slots): 32 slots = 4 x 16 bytes
         {
-            const int d = tid >> 1, sh = (tid & 1) * 32;
-            T tmp[32];
+            const int j = tid & 63, g = tid >> 6;
+            uint32_t w[16];
 #pragma unroll
-            for (int sl = 0; sl < 32; sl++) {
-                const int slot = sh + sl;
-                // inverse of vt_slot: slot = 16s + 8h + 4a + e  ->  key = 16s + 8a + 4h + e
-                const int s = slot >> 4, h = (slot >> 3) & 1, a = (slot >> 2) & 1, e = slot & 3;
-                tmp[sl] = v_lds[16 * s + 8 * a + 4 * h + e][d];
+            for (int sl = 0; sl < 16; sl++) {
+                // inverse of vt_slot: slot = 16g + 8h + 4a + e  ->  key = 16g + 8a + 4h + e
+                const int h = (sl >> 3) & 1, a = (sl >> 2) & 1, e = sl & 3;
+                w[sl] = v_lds[16 * g + 8 * a + 4 * h + e][j];
             }
-            const uint4* src = reinterpret_cast<const uint4*>(tmp);
+            uint32_t lo_row[8], hi_row[8];
 #pragma unroll
-            for (int i = 0; i < 4; i++) *reinterpret_cast<uint4*>(vimg + v_image_off(d, sh / 8 + i)) = src[i];
+            for (int k = 0; k < 8; k++) {
+                lo_row[k] = (w[2 * k] & 0xffffu) | (w[2 * k + 1] << 16);
+                hi_row[k] = (w[2 * k] >> 16) | (w[2 * k + 1] & 0xffff0000u);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                *reinterpret_cast<uint4*>(vimg + v_image_off(j, 2 * g + i)) =
+                    make_uint4(lo_row[4 * i], lo_row[4 * i + 1], lo_row[4 * i + 2], lo_row[4 * i + 3]);
+                *reinterpret_cast<uint4*>(vimg + v_image_off(j + 64, 2 * g + i)) =
+                    make_uint4(hi_row[4 * i], hi_row[4 * i + 1], hi_row[4 * i + 2], hi_row[4 * i + 3]);
+            }
         }
     }
 }
@@ -359,7 +367,7 @@ struct StageGrid {
 };
 template <typename T>
 __global__ void __launch_bounds__(256) stage_kernel(StageParams sp, StageQParams sq, StageGrid g) {
-    __shared__ T v_lds[kBN][kD + 2];
+    __shared__ uint32_t v_lds[kBN][kD / 2 + 1];  // (d, d + 64) pairs of a key row, odd pitch
     const int nk = g.k_bx * g.k_by;
     int id = blockIdx.x;
     if (id < nk) {
