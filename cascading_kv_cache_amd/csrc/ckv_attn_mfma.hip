@@ -52,6 +52,9 @@ struct Mma<__hip_bfloat16> {
         const uint32_t u = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
         return __uint_as_float(u << 16);
     }
+    // the two elements of a packed pair as floats
+    __device__ static float lo_f(uint32_t w) { return __uint_as_float(w << 16); }
+    __device__ static float hi_f(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
     // acc + both halves of a packed pair (one v_dot2c with a pair of ones)
     __device__ static float sum2(uint32_t w, float acc) {
         return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), __builtin_bit_cast(bf16x2, 0x3f803f80u), acc, false);
@@ -68,6 +71,8 @@ struct Mma<__half> {
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
     }
     __device__ static float round1(float v) { return (float)(_Float16)v; }
+    __device__ static float lo_f(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
+    __device__ static float hi_f(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
     __device__ static float sum2(uint32_t w, float acc) {
         return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), __builtin_bit_cast(f16x2, 0x3c003c00u), acc, false);
     }
@@ -219,13 +224,16 @@ __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int sp
                         fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
                     }
                 }
-                T* l0 = reinterpret_cast<T*>(lo);
-                T* h0 = reinterpret_cast<T*>(hi);
+                // on packed pairs: two elements per word, converted and rounded (to nearest even, like the
+                // element-wise casts) by the packed conversion instructions
+                uint32_t* lw = reinterpret_cast<uint32_t*>(lo);
+                uint32_t* hw = reinterpret_cast<uint32_t*>(hi);
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const float x1 = Elem<T>::to_float(l0[i]), x2 = Elem<T>::to_float(h0[i]);
-                    l0[i] = Elem<T>::from_float(x1 * cs[i] - x2 * sn[i]);
-                    h0[i] = Elem<T>::from_float(x2 * cs[i] + x1 * sn[i]);
+                for (int k = 0; k < 8; k++) {
+                    const float x1a = Mma<T>::lo_f(lw[k]), x1b = Mma<T>::hi_f(lw[k]);
+                    const float x2a = Mma<T>::lo_f(hw[k]), x2b = Mma<T>::hi_f(hw[k]);
+                    lw[k] = Mma<T>::pack2(x1a * cs[2 * k] - x2a * sn[2 * k], x1b * cs[2 * k + 1] - x2b * sn[2 * k + 1]);
+                    hw[k] = Mma<T>::pack2(x2a * cs[2 * k] + x1a * sn[2 * k], x2b * cs[2 * k + 1] + x1b * sn[2 * k + 1]);
                 }
             }
         }
@@ -332,15 +340,20 @@ __device__ inline void stage_q_block(const StageQParams& p, int blk, int share_i
     // they come out of the matrix pipe
     auto finish_row = [&](int64_t bh, Row& r) {
         if (bh >= nbh) return;
+        uint32_t* lw = reinterpret_cast<uint32_t*>(r.lo);
+        uint32_t* hw = reinterpret_cast<uint32_t*>(r.hi);
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const float x1 = Elem<T>::to_float(r.lo[i]), x2 = Elem<T>::to_float(r.hi[i]);
+        for (int k = 0; k < 8; k++) {  // on packed pairs, as in stage_keys_block
+            const float x1a = Mma<T>::lo_f(lw[k]), x1b = Mma<T>::hi_f(lw[k]);
+            const float x2a = Mma<T>::lo_f(hw[k]), x2b = Mma<T>::hi_f(hw[k]);
             if (p.q_pos) {
-                r.lo[i] = Elem<T>::from_float((x1 * cs[i] - x2 * sn[i]) * p.qscale);
-                r.hi[i] = Elem<T>::from_float((x2 * cs[i] + x1 * sn[i]) * p.qscale);
+                lw[k] = Mma<T>::pack2((x1a * cs[2 * k] - x2a * sn[2 * k]) * p.qscale,
+                                      (x1b * cs[2 * k + 1] - x2b * sn[2 * k + 1]) * p.qscale);
+                hw[k] = Mma<T>::pack2((x2a * cs[2 * k] + x1a * sn[2 * k]) * p.qscale,
+                                      (x2b * cs[2 * k + 1] + x1b * sn[2 * k + 1]) * p.qscale);
             } else {
-                r.lo[i] = Elem<T>::from_float(x1 * p.qscale);
-                r.hi[i] = Elem<T>::from_float(x2 * p.qscale);
+                lw[k] = Mma<T>::pack2(x1a * p.qscale, x1b * p.qscale);
+                hw[k] = Mma<T>::pack2(x2a * p.qscale, x2b * p.qscale);
             }
         }
         T* dst = (T*)p.qr + (bh * p.Q + m) * kD;
@@ -1250,7 +1263,9 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         cp.first_chunk_blk = (int)(cp.Nc / 256);
         cp.nbkv = (int)(mp.B * mp.KVH);
         cp.xcd_aware = cp.nbkv % 8 == 0;
-        cp.gsplit = G;  // one head per workgroup
+        // two heads per workgroup where the group allows it: the keys a workgroup holds in registers and its
+        // pipeline start serve twice the work, and the units stay small enough for an even last round
+        cp.gsplit = (G % 2 == 0 && G >= 4) ? G / 2 : G;
         const dim3 grid((unsigned)(cp.nkb * cp.nbkv * cp.gsplit));
         const int lds = 2 * kCsStage + (int)mp.Q * 4;
         CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(colsum_mfma_kernel<T>),
