@@ -11,12 +11,13 @@
 //          a forest of disjoint move chains in global memory:
 //              first[t]   = slot the incoming token t finally lands in (-1: dropped)
 //              next_of[d] = slot the OLD content of slot d finally lands in (-1: dropped)
-//          plus the trackers, and the position ids in closed form (cascading_cache.py:112-142,
-//          728-774).
+//          plus the updated trackers.
 //   apply  one lane group per incoming token.  Follows the chain of its token from the head,
 //          carrying a whole row (K, V, score, original index) in registers with 16-byte lanes:
 //          read the displaced row, write the carried one, move on.  Chains are vertex-disjoint
 //          and only ever move towards higher cascades, so groups never touch each other's slots.
+//          The same launch writes the position ids in closed form from the updated trackers
+//          (cascading_cache.py:112-142, 728-774) with extra blocks at the end of its grid.
 //
 // Why this equals the serial loop: within one cascade the n-th insert of a call always lands in
 // ring position (start + stored + n) mod W whatever the scores are; only WHICH arrival owns a
