@@ -115,6 +115,7 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
         mp.lse2 = w.lse2;
         mp.colsum = want_scores ? w.colsum : nullptr;
         mp.w_ema = w.w_ema; mp.w_new = w.w_new;
+        mp.beta = a.beta;
         mp.new_mode = 1;
         mp.B = a.B; mp.H = a.H; mp.KVH = a.KVH; mp.Q = a.Q; mp.n = N; mp.n_pad = mfma_n_pad(N);
         mp.scale = a.scale;
@@ -228,6 +229,7 @@ extern "C" int ckv_attn_dense(const ckv_dense_args* args, void* stream_) {
         mp.lse2 = w.lse2;
         mp.colsum = a.scores ? w.colsum : nullptr;
         mp.w_ema = w.w_ema; mp.w_new = w.w_new;
+        mp.beta = a.beta;
         mp.new_mode = 0;  // every key is weighted by the query row alone (flash_attention.py:73-77)
         mp.B = a.B; mp.H = a.H; mp.KVH = a.H; mp.Q = a.n_ctx; mp.n = a.n_kv; mp.n_pad = mfma_n_pad(a.n_kv);
         mp.scale = a.scale;

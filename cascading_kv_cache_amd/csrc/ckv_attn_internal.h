@@ -96,6 +96,7 @@ struct MfmaProblem {
     float* colsum;         // (B, H, n) or null
     const float* w_ema;
     const float* w_new;
+    double beta;           // the EMA factor the weights were built from
     int new_mode;
     int64_t B, H, KVH, Q, n, n_pad;
     float scale;

@@ -18,6 +18,7 @@
 //                inside a lane (S = Q K^T orientation).
 #include "ckv_attn_internal.h"
 
+#include <cstring>
 #include <type_traits>
 
 namespace ckv {
@@ -857,6 +858,8 @@ struct ColsumParams {
     int new_mode;
     float scale_log2;
     int nkb, first_chunk_blk, nbkv, xcd_aware, gsplit;  // block order and head split, see the kernel
+    int wnew_uniform;     // every entry of w_new has the value wnew_value (beta rounds to one in the tensor dtype)
+    float wnew_value;
 };
 
 constexpr int kQT2 = 128;                     // query rows per LDS tile of the column pass
@@ -1066,7 +1069,21 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
                     sacc[0] = Mma<T>::mma(a, kreg[0][kk], sacc[0]);
                     sacc[1] = Mma<T>::mma(a, kreg[1][kk], sacc[1]);
                 }
-                if (fast_new) {
+                if (fast_new && p.wnew_uniform && __builtin_amdgcn_ballot_w64(!(chunk_lane[0] && chunk_lane[1])) == 0ull) {
+                    // every key of the wavefront is a chunk key and all of them weigh the same: P and the
+                    // products are rounded to the tensor dtype two at a time by the packed conversions, and
+                    // the rounded products join the sum through a dot product with a pair of ones
+                    const float wu = p.wnew_value;
+#pragma unroll
+                    for (int v = 0; v < 16; v += 2) {
+#pragma unroll
+                        for (int ks = 0; ks < 2; ks++) {
+                            const uint32_t u = Mma<T>::pack2(__builtin_amdgcn_exp2f(sacc[ks][v]),
+                                                             __builtin_amdgcn_exp2f(sacc[ks][v + 1]));
+                            acc[ks] = Mma<T>::sum2(Mma<T>::pack2(Mma<T>::lo_f(u) * wu, Mma<T>::hi_f(u) * wu), acc[ks]);
+                        }
+                    }
+                } else if (fast_new) {
                     // no masks; the eager path holds P and the products of chunk keys in the tensor dtype
 #pragma unroll
                     for (int v4 = 0; v4 < 4; v4++) {
@@ -1258,6 +1275,22 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         cp.B = mp.B; cp.H = mp.H; cp.KVH = mp.KVH; cp.Q = mp.Q; cp.N = n; cp.Nc = n - mp.Q; cp.n_pad = n_pad;
         cp.G = G;
         cp.new_mode = mp.new_mode;
+        {
+            // w_new[k] = round((1 - beta) * round(round(beta)^k)) in the tensor dtype: one value for every k when
+            // beta rounds to one there (0.9999999 does in both 16-bit formats)
+            auto round_t_host = [](float v) -> float {
+                if (std::is_same<T, __half>::value) return (float)(_Float16)v;
+                uint32_t u;
+                memcpy(&u, &v, 4);
+                u += 0x7fffu + ((u >> 16) & 1u);  // to nearest even on the upper 16 bits (finite values)
+                u &= 0xffff0000u;
+                float r;
+                memcpy(&r, &u, 4);
+                return r;
+            };
+            cp.wnew_uniform = round_t_host((float)mp.beta) == 1.0f ? 1 : 0;
+            cp.wnew_value = round_t_host((float)(1.0 - mp.beta));
+        }
         cp.scale_log2 = 1.f;  // already on the staged queries
         cp.nkb = (int)((n + 255) / 256);
         cp.first_chunk_blk = (int)(cp.Nc / 256);
