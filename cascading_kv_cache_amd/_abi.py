@@ -126,6 +126,27 @@ def fill_update_args(k, v, s, sink_k, sink_v, sink_mask, sink_pos, cache_k, cach
             raise TypeError("index tensors must be torch.int64")
     if not do_cache_every_n.is_contiguous():
         raise ValueError("do_cache_every_n must be contiguous")
+    # The kernel addresses every state tensor with the sizes of k: a chunk with more streams, heads or a
+    # wider row than the cache holds would be written past the allocations.
+    S, C_ = int(max_seq_len), int(stored_tokens.size(-1))
+    want = {
+        "cache_k": (cache_k, (H, S, HID)), "sink_k": (sink_k, (H, int(num_sink), HID)),
+        "cache_s": (cache_s, (H, S)), "mask": (mask, (H, S)), "pos": (pos, (H, S)), "og_pos": (og_pos, (H, S)),
+        "sink_mask": (sink_mask, (H, int(num_sink))), "sink_pos": (sink_pos, (H, int(num_sink))),
+        "stored_tokens": (stored_tokens, (H, C_)), "stored_sinks": (stored_sinks, (H,)),
+    }
+    for name, (t, tail) in want.items():
+        if tuple(t.shape[1:]) != tail or t.size(0) < N:
+            raise ValueError(f"{name} has shape {tuple(t.shape)}; a chunk of shape {tuple(k.shape)} needs "
+                             f"(>= {N}, {', '.join(str(x) for x in tail)})")
+    if s.ndim != 3 or s.size(0) < N or s.size(1) < H or s.size(2) != K:
+        raise ValueError(f"scores have shape {tuple(s.shape)}; expected ({N}, >= {H}, {K})")
+    if do_cache_every_n.numel() != C_ or C_ * int(window_size) != S:
+        raise ValueError("cascades * window_size must equal max_seq_len, one acceptance period per cascade")
+    for t in (v, s, sink_k, cache_k, cache_s, mask, pos, og_pos, stored_tokens, stored_sinks, do_cache_every_n,
+              real_token_idx):
+        if t.device != k.device:
+            raise ValueError(f"all tensors of an update must live on one device, got {t.device} and {k.device}")
 
     a = UpdateArgs()
     a.k, a.v, a.s = k.data_ptr(), v.data_ptr(), s.data_ptr()

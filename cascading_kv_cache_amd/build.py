@@ -1,18 +1,24 @@
 """Build ``csrc/libckv.so`` for gfx950 with hipcc (cross-compiles without a GPU).
 
-    python -m cascading_kv_cache_amd.build
+    python -m cascading_kv_cache_amd.build            # compile every source, link
+    python -m cascading_kv_cache_amd.build --changed  # only sources newer than their object
+
+Every ``.hip`` file is compiled to an object of its own (in parallel) and the objects are linked
+into one shared library; objects live in ``csrc/build/`` (git-ignored).
 """
 import glob
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(CSRC, "build")
 OUT = os.path.join(CSRC, "libckv.so")
 
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Wall", "-Wno-unused-function",
     # keep the compiler from forming packed-fp32 VALU ops out of scalar float code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -23,14 +29,41 @@ def sources():
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
 
-def build(verbose: bool = True) -> str:
-    cmd = ["hipcc", *FLAGS, "-o", OUT, *sources()]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True, cwd=CSRC)
+def _headers_mtime():
+    hs = glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(os.path.join(HERE, "..", "include", "*.h"))
+    return max(os.path.getmtime(h) for h in hs)
+
+
+def build(verbose: bool = True, only_changed: bool = False) -> str:
+    os.makedirs(OBJ, exist_ok=True)
+    hdr = _headers_mtime()
+    jobs = []
+    objs = []
+    for src in sources():
+        obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
+        objs.append(obj)
+        fresh = os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), hdr)
+        if only_changed and fresh:
+            continue
+        jobs.append(["hipcc", *FLAGS, "-c", src, "-o", obj])
+
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        r = subprocess.run(cmd, cwd=CSRC, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        # the host pass does not know the packed-fp32 feature and says so once per kernel: harmless
+        out = "\n".join(l for l in r.stdout.splitlines() if "is not a recognized feature for this target" not in l)
+        if out.strip():
+            print(out, flush=True)
+        if r.returncode != 0:
+            raise subprocess.CalledProcessError(r.returncode, cmd)
+
+    with ThreadPoolExecutor(max_workers=min(6, max(1, len(jobs)))) as ex:
+        list(ex.map(run, jobs))
+    run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", OUT, *objs])
     return OUT
 
 
 if __name__ == "__main__":
-    build()
+    build(only_changed="--changed" in sys.argv[1:])
     sys.exit(0)

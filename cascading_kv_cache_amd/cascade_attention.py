@@ -58,6 +58,31 @@ def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_p
     return out
 
 
+def check_against_cache(query_states, key_states, value_states, cache: CascadingKVCache, L: int):
+    """The kernels index the cache tensors with the sizes of the incoming chunk, so every size the two
+    share is checked here, on the host, before any pointer leaves: a mismatch raises instead of reading
+    or writing past the cache allocations (the reference fails with a torch shape or dtype error at its
+    ``torch.cat`` / ``einsum`` calls, cascade_attention.py:212-218, 284-291)."""
+    B, H, Q, D = query_states.shape
+    KVH = key_states.size(1)
+    if not 0 <= L < cache.layers:
+        raise ValueError(f"layer {L} outside the cache's {cache.layers} layers")
+    kc = cache.key_cache[L]
+    if H % KVH != 0:
+        raise ValueError(f"{H} query heads are not a multiple of {KVH} kv heads")
+    if B > kc.size(0):
+        raise ValueError(f"batch {B} exceeds the cache's max_batch_size {kc.size(0)}")
+    if KVH != kc.size(1):
+        raise ValueError(f"{KVH} kv heads, but the cache holds {kc.size(1)}")
+    if D != kc.size(3):
+        raise ValueError(f"head_dim {D}, but the cache holds rows of {kc.size(3)}")
+    for name, t in (("query_states", query_states), ("key_states", key_states), ("value_states", value_states)):
+        if t.dtype != kc.dtype:
+            raise TypeError(f"{name} is {t.dtype}, the cache is {kc.dtype}")
+        if t.device != kc.device:
+            raise ValueError(f"{name} lives on {t.device}, the cache on {kc.device}")
+
+
 def _describe_attention(query_states, key_states, value_states, cache, L, inv_freq, reduction, homogeneous_heads,
                         do_og_pos, scale, out, new_scores):
     """The argument block of ``ckv_attn`` for one layer and input layout; everything in it except the
@@ -139,7 +164,8 @@ def cascade_attention(query_states, key_states, value_states, cache: CascadingKV
                bool(homogeneous_heads), bool(do_og_pos), float(scale), float(cache.beta), inv_freq.data_ptr(),
                inv_freq.dtype, cache._state_key(L))
         a = cache._attn_memo.get(key)
-        if a is None:
+        if a is None:  # a layout not seen before: validated once, then described
+            check_against_cache(query_states, key_states, value_states, cache, L)
             a = _describe_attention(query_states, key_states, value_states, cache, L, inv_freq, reduction,
                                     homogeneous_heads, do_og_pos, scale, out, new_scores)
             if len(cache._attn_memo) > 64:
@@ -151,7 +177,7 @@ def cascade_attention(query_states, key_states, value_states, cache: CascadingKV
         a.pos_shift = 0 if do_og_pos else cache.pos_shift(L)
         a.out = out.data_ptr()
         a.new_scores = new_scores.data_ptr()
-        ws = workspace(dev, a._need)
+        ws = workspace(dev, a._need, stream)
         a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
         _abi.check(lib.ckv_attn(C.byref(a), C.c_void_p(stream)), "ckv_attn")
         if update_cache:
@@ -177,11 +203,9 @@ class CascadeAttention(nn.Module):
         raise ValueError("unknown custom attention")
 
     def qkv(self, x, size, kv_size):
-        q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
-        q = q.view(*size).transpose(1, 2)
-        k = k.view(*kv_size).transpose(1, 2)
-        v = v.view(*kv_size).transpose(1, 2)
-        return q, k, v
+        """Projections reshaped to (batch, heads, tokens, head_dim) (cascade_attention.py:74-80)."""
+        return (self.q_proj(x).view(*size).transpose(1, 2), self.k_proj(x).view(*kv_size).transpose(1, 2),
+                self.v_proj(x).view(*kv_size).transpose(1, 2))
 
     def forward_cascade(self, hidden_states, attention_mask=None, position_ids=None, past_key_value=None,
                         output_attentions=False, use_cache=False, cache_position=None, use_flash=True,
@@ -202,16 +226,26 @@ class CascadeAttention(nn.Module):
         return out, None, past_key_value
 
     def calc_scores(self, scores, homogeneous_heads, n_keys, q_len):
-        """Head reduction of per-head score sums (cascade_attention.py:231-248), for callers
-        that hold per-head scores of their own; the fused path reduces inside the kernels."""
+        """Head reduction of per-head score sums ``(B, H, n)`` with the semantics of
+        cascade_attention.py:231-248, for callers that hold per-head scores of their own (``attention``
+        returns them); the fused path reduces inside the kernels.  The heads are viewed as
+        ``(groups, members)``: one group of all heads when ``homogeneous_heads`` (its result serves every kv
+        head), otherwise one group per kv head.  Returns the reduced scores of the first ``n_keys`` keys
+        ``(B, groups, n_keys)`` and of the last ``q_len`` keys ``(B, KVH, q_len)``."""
         kvh = self.num_key_value_heads
-        func = {"mean": torch.mean, "max": torch.amax,
-                "median": lambda x, **kw: torch.median(x, **kw).values}[self.config._head_reduction]
-        if homogeneous_heads:
-            ema_scores = func(scores[:, :, :n_keys], dim=1, keepdim=True)
-            scores = func(scores[:, :, -q_len:], dim=1, keepdim=True).repeat(1, kvh, 1)
+        b, h, _ = scores.shape
+        groups = 1 if homogeneous_heads else kvh
+        grouped = scores.view(b, groups, h // groups, -1)
+        how = self.config._head_reduction
+        if how == "mean":
+            reduced = grouped.mean(dim=2)
+        elif how == "max":
+            reduced = grouped.amax(dim=2)
+        elif how == "median":
+            reduced = grouped.median(dim=2).values
         else:
-            b, h, s = scores.size()
-            ema_scores = func(scores[:, :, :n_keys].view(b, kvh, h // kvh, -1), dim=2)
-            scores = func(scores[:, :, -q_len:].view(b, kvh, h // kvh, -1), dim=2)
-        return ema_scores, scores
+            raise KeyError(how)
+        new_scores = reduced[:, :, -q_len:]
+        if homogeneous_heads:
+            new_scores = new_scores.repeat(1, kvh, 1)
+        return reduced[:, :, :n_keys], new_scores

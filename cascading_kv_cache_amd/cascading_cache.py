@@ -17,9 +17,13 @@ from . import _abi
 _WORKSPACES = {}
 
 
-def workspace(device: torch.device, nbytes: int) -> Tensor:
-    """A per-device scratch buffer, grown on demand and reused by stream-ordered calls."""
-    key = (device.type, device.index)
+def workspace(device: torch.device, nbytes: int, stream: int = 0) -> Tensor:
+    """Scratch for one library call: one buffer per (device, stream), grown on demand.  Calls on one
+    stream run in order, so they can share a buffer; calls on different streams of a device may
+    overlap and get buffers of their own.  ``stream`` is the raw stream handle (0: the null stream).
+    A buffer that is outgrown is dropped only after the stream has passed the calls that used it
+    (torch's caching allocator keeps a freed block tied to the stream it was allocated on)."""
+    key = (device.type, device.index, int(stream))
     buf = _WORKSPACES.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
@@ -54,10 +58,10 @@ def sink_cache(
                               og_pos, do_cache_every_n, stored_tokens, start_indices, stored_sinks, num_sink,
                               window_size, real_token_idx, max_seq_len, eager_fill)
     need = lib.ckv_update_workspace_bytes(a.N, a.H, a.K, a.max_seq_len, a.cascades)
-    ws = workspace(k.device, need)
-    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     with torch.cuda.device(k.device):
         stream = torch.cuda.current_stream(k.device).cuda_stream
+        ws = workspace(k.device, need, stream)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
         _abi.check(lib.ckv_update(C.byref(a), C.c_void_p(stream)), "ckv_update")
     if BENCHMARK:
         ev1.record()
@@ -254,41 +258,30 @@ class CascadingKVCache:
         )
 
     def _state_key(self, L: int):
-        """Identity of the layer's state tensors: a memoised argument block is only reused while the
-        cache still holds the very tensors it was described from."""
-        return (id(self.key_cache[L]), id(self.value_cache[L]), id(self.score_cache[L]), id(self.sink_keys[L]),
-                id(self.sink_values[L]), id(self.mask[L]), id(self.sink_mask[L]), id(self.pos[L]), id(self.og_pos[L]),
-                id(self.sink_pos[L]), id(self.stored_tokens[L]), id(self.start_indices[L]), id(self.stored_sinks[L]),
-                id(self.do_cache_every_n[L]), id(self.seen_tokens_by_layer), self.key_cache[L].data_ptr())
+        """Where the layer's state tensors live and how they are laid out: a memoised argument block holds
+        raw device pointers and strides, so it is reused only while every state tensor is still at the address
+        it was described from.  (Object identity would not do: callers may assign a new tensor to
+        ``score_cache[l]`` every step, as cascade_attention.py:222-224 does, and a freed object's id is
+        handed out again.)"""
+        ts = (self.key_cache[L], self.value_cache[L], self.score_cache[L], self.sink_keys[L], self.sink_values[L],
+              self.mask[L], self.sink_mask[L], self.pos[L], self.og_pos[L], self.sink_pos[L], self.stored_tokens[L],
+              self.start_indices[L], self.stored_sinks[L], self.do_cache_every_n[L], self.seen_tokens_by_layer)
+        return tuple(t.data_ptr() for t in ts) + (self.score_cache[L].stride(), self.score_cache[L].dtype)
 
     def update(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None):
         """cascading_cache.py:1297-1348."""
         self.update_state(key_states, value_states, layer_idx, score_states)
         return self.get_vals(layer_idx)
 
-    def update_state(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None,
-                     _stream: Optional[int] = None):
-        """``update`` without building the tuple of views it returns (the shifted position row of
-        ``get_vals`` is a device operation of its own); for callers that read the state in place.
-
-        The argument block of ``ckv_update`` is described once per layer and input layout and reused:
-        between two calls of the same shape only the three input pointers change (single-token steps
-        at batch 1 are bound by this host code, not by the device).  ``_stream``: raw stream handle when
-        the caller already holds the device context."""
-        if score_states is None:
-            score_states = torch.zeros(self.max_batch_size, self.heads, key_states.size(2),
-                                       device=key_states.device, dtype=key_states.dtype)
-        if layer_idx == 0:
-            self._seen_tokens += key_states.shape[-2]
-
-        L = layer_idx
+    def _update_args(self, key_states: Tensor, value_states: Tensor, score_states: Tensor, L: int):
+        """The ``ckv_update`` argument block for these inputs: described once per layer, input layout and
+        placement of the state tensors, then reused with only the three input pointers refreshed."""
         key = (L, key_states.shape, key_states.stride(), value_states.shape, value_states.stride(),
                score_states.shape, score_states.stride(), key_states.dtype, value_states.dtype, score_states.dtype,
                key_states.device, value_states.device, score_states.device, self._state_key(L))
         memo = self._update_memo
         a = memo.get(key)
         if a is None:
-            _require_device(key_states, "k")
             a = _abi.fill_update_args(
                 key_states, value_states, score_states,
                 self.sink_keys[L], self.sink_values[L], self.sink_mask[L], self.sink_pos[L],
@@ -303,13 +296,34 @@ class CascadingKVCache:
             memo[key] = a
         else:
             a.k, a.v, a.s = key_states.data_ptr(), value_states.data_ptr(), score_states.data_ptr()
-        ws = workspace(key_states.device, a._need)
-        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+        return a
+
+    def update_state(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None,
+                     _stream: Optional[int] = None):
+        """``update`` without building the tuple of views it returns (the shifted position row of
+        ``get_vals`` is a device operation of its own); for callers that read the state in place.
+
+        The argument block of ``ckv_update`` is described once per layer and input layout and reused:
+        between two calls of the same shape only the three input pointers change (single-token steps
+        at batch 1 are bound by this host code, not by the device).  ``_stream``: raw stream handle when
+        the caller already holds the device context."""
+        _require_device(key_states, "k")
+        if score_states is None:
+            score_states = torch.zeros(self.max_batch_size, self.heads, key_states.size(2),
+                                       device=key_states.device, dtype=key_states.dtype)
+        if layer_idx == 0:
+            self._seen_tokens += key_states.shape[-2]
+
+        a = self._update_args(key_states, value_states, score_states, layer_idx)
         if _stream is None:
             with torch.cuda.device(key_states.device):
                 stream = torch.cuda.current_stream(key_states.device).cuda_stream
+                ws = workspace(key_states.device, a._need, stream)
+                a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
                 _abi.check(_abi.lib().ckv_update(C.byref(a), C.c_void_p(stream)), "ckv_update")
         else:
+            ws = workspace(key_states.device, a._need, _stream)
+            a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
             _abi.check(_abi.lib().ckv_update(C.byref(a), C.c_void_p(_stream)), "ckv_update")
         # after the kernel, as in the reference (cascading_cache.py:1343-1346)
         self.seen_tokens_by_layer[layer_idx] += key_states.shape[-2]

@@ -2,6 +2,8 @@
 #include "ckv_common.h"
 
 #include <cstdint>
+#include <mutex>
+#include <unordered_map>
 #include <vector>
 
 namespace ckv {
@@ -13,7 +15,46 @@ struct Span {
 int g_prof_level = 0;  // 0 off, 1 every stage, 2 attention main kernels only
 std::vector<Span> g_spans;
 hipEvent_t g_open[CKV_STAGE_COUNT];
+std::mutex g_prof_mutex;  // guards g_spans and g_open: calls on several host threads may time stages at once
+
+constexpr int kMaxDevices = 64;
+std::mutex g_dev_mutex;
+DeviceInfo g_dev[kMaxDevices];
+bool g_dev_known[kMaxDevices];
+std::unordered_map<const void*, int> g_lds_set[kMaxDevices];  // dynamic LDS limit already set per kernel
 }  // namespace
+
+int current_device_info(DeviceInfo* info) {
+    int dev = 0;
+    CKV_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return CKV_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_dev_mutex);
+    if (!g_dev_known[dev]) {
+        DeviceInfo d;
+        d.device = dev;
+        d.cus = 256;
+        d.lds_max = 65536;
+        CKV_HIP_TRY(hipDeviceGetAttribute(&d.cus, hipDeviceAttributeMultiprocessorCount, dev));
+        CKV_HIP_TRY(hipDeviceGetAttribute(&d.lds_max, hipDeviceAttributeMaxSharedMemoryPerBlock, dev));
+        g_dev[dev] = d;
+        g_dev_known[dev] = true;
+    }
+    *info = g_dev[dev];
+    return CKV_OK;
+}
+
+int ensure_dynamic_lds(const void* func, int bytes) {
+    if (bytes <= 48 * 1024) return CKV_OK;  // within the limit every kernel starts with
+    int dev = 0;
+    CKV_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return CKV_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_dev_mutex);
+    int& have = g_lds_set[dev][func];
+    if (have >= bytes) return CKV_OK;
+    CKV_HIP_TRY(hipFuncSetAttribute(func, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    have = bytes;
+    return CKV_OK;
+}
 
 static bool prof_wanted(int stage) {
     return g_prof_level == 1 || (g_prof_level == 2 && (stage == CKV_STAGE_FWD || stage == CKV_STAGE_DECODE));
@@ -32,7 +73,10 @@ void prof_kernel_events(int stage, hipEvent_t* start, hipEvent_t* stop) {
         (void)hipEventDestroy(e0);
         return;
     }
-    g_spans.push_back(Span{stage, e0, e1});
+    {
+        std::lock_guard<std::mutex> lock(g_prof_mutex);
+        g_spans.push_back(Span{stage, e0, e1});
+    }
     *start = e0;
     *stop = e1;
 }
@@ -42,10 +86,12 @@ void prof_begin(int stage, hipStream_t stream) {
     hipEvent_t e;
     if (hipEventCreate(&e) != hipSuccess) return;
     (void)hipEventRecord(e, stream);
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
     g_open[stage] = e;
 }
 
 void prof_end(int stage, hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_prof_mutex);
     if (!g_open[stage]) return;
     hipEvent_t e;
     if (hipEventCreate(&e) != hipSuccess) return;
@@ -63,6 +109,7 @@ extern "C" int ckv_profile_enable(int on) {
 
 extern "C" int ckv_profile_read(double* ms, int64_t* launches) {
     if (!ms || !launches) return CKV_ERR_NULL;
+    std::lock_guard<std::mutex> lock(ckv::g_prof_mutex);
     for (auto& s : ckv::g_spans) {
         float t = 0.f;
         if (hipEventSynchronize(s.t1) == hipSuccess && hipEventElapsedTime(&t, s.t0, s.t1) == hipSuccess) {

@@ -1283,7 +1283,7 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
     DecodeParams p = p_in;
     const ckv_attn_args& a = p.a;
     const bool use_stream =
-        !std::is_same<T, float>::value && G <= 4 && p.shared_pos && stream_offsets_fit(a) && !getenv("CKV_DECODE_OLD");
+        !std::is_same<T, float>::value && G <= 4 && p.shared_pos && stream_offsets_fit(a);
     if (use_stream) p.tiles = (int)((p.N + kSK - 1) / kSK);  // the streaming kernel has its own tile size
     p.Np = (int64_t)p.tiles * kSK;
     {
@@ -1300,22 +1300,17 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
         if (groups > nbh) groups = nbh;
         const int lds = (16 * G * kD + 32 * G + 4 * 32 * 8) * (int)sizeof(float);
         if constexpr (std::is_same<T, float>::value) {
-            if (lds > 48 * 1024) {
-                CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_main_kernel<T, G>),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-            }
+            if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(decode_main_kernel<T, G>), lds)) return rc;
             hipLaunchKernelGGL((decode_main_kernel<T, G>), dim3((unsigned)p.tiles, (unsigned)groups), dim3(256), lds,
                                stream, p);
         } else if (use_stream) {
             // streaming kernel: as many workgroups as run at once, items dealt out evenly
             if constexpr (G <= 4) {
                 const int lds_s = kStreamLds;
-                CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_stream_kernel<T, G>),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_s));
-                int dev = 0, cus = 0;
-                CKV_HIP_TRY(hipGetDevice(&dev));
-                CKV_HIP_TRY(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-                int64_t wgs = (cus > 0 ? cus : 256) * kStreamWgPerCu;
+                if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(decode_stream_kernel<T, G>), lds_s)) return rc;
+                DeviceInfo di;
+                if (int rc = current_device_info(&di)) return rc;
+                int64_t wgs = (di.cus > 0 ? di.cus : 256) * kStreamWgPerCu;
                 if (wgs > kStreamMaxWgs) wgs = kStreamMaxWgs;
                 if (wgs > p.tiles * nbh) wgs = p.tiles * nbh;
                 p.stream_wgs = (int)wgs;
@@ -1328,10 +1323,7 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
                     hipLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads), lds_s, stream, p);
             }
         } else {
-            if (lds > 48 * 1024) {
-                CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(decode_main_mfma_kernel<T, G>),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-            }
+            if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(decode_main_mfma_kernel<T, G>), lds)) return rc;
             hipLaunchKernelGGL((decode_main_mfma_kernel<T, G>), dim3((unsigned)p.tiles, (unsigned)groups), dim3(256), lds,
                                stream, p);
         }

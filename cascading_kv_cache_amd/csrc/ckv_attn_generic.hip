@@ -309,10 +309,7 @@ int core_generic_t(const CoreProblem& p, hipStream_t stream) {
     if (p.colsum) {
         const int64_t chunks = (p.N + CKV_WAVE - 1) / CKV_WAVE;
         const size_t lds = (size_t)CKV_WAVE * (p.D + 1) * sizeof(float);
-        if (lds > 48 * 1024) {
-            CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(colsum_generic_kernel<T>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        }
+        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(colsum_generic_kernel<T>), (int)lds)) return rc;
         {
             StageScope sc(CKV_STAGE_SCORES, stream);
             hipLaunchKernelGGL(colsum_generic_kernel<T>, dim3((unsigned)(p.B * p.H * chunks)), dim3(CKV_WAVE), lds,

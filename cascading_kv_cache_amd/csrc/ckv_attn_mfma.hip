@@ -1256,8 +1256,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         fp.scale_log2 = 1.f;  // already on the staged queries
         const dim3 grid((unsigned)((mp.Q + fp.QT - 1) / fp.QT), (unsigned)(mp.B * mp.KVH));
         const int lds = pipe_lds_bytes(n_pad);
-        CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(fwd_pipe_kernel<T>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fwd_pipe_kernel<T>), lds)) return rc;
         fp.n_qt = (int)grid.x;
         fp.xcd_aware = grid.y % 8 == 0;
         hipEvent_t ev0, ev1;
@@ -1301,8 +1300,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         cp.gsplit = (G % 2 == 0 && G >= 4) ? G / 2 : G;
         const dim3 grid((unsigned)(cp.nkb * cp.nbkv * cp.gsplit));
         const int lds = 2 * kCsStage + (int)mp.Q * 4;
-        CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(colsum_mfma_kernel<T>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(colsum_mfma_kernel<T>), lds)) return rc;
         hipLaunchKernelGGL(colsum_mfma_kernel<T>, grid, dim3(256), lds, stream, cp);
         CKV_HIP_TRY(hipGetLastError());
     }

@@ -88,6 +88,17 @@ struct StageScope {
 
 inline int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
 
+// Facts about the current device, asked of the runtime once per device and process.
+struct DeviceInfo {
+    int device;        // ordinal of the current device
+    int cus;           // compute units
+    int lds_max;       // bytes of LDS one workgroup may use
+};
+int current_device_info(DeviceInfo* info);  // CKV_OK or CKV_ERR_LAUNCH
+// Raises the dynamic LDS limit of `func` on the current device to at least `bytes`; the runtime is asked
+// only when the limit this process has already set for (device, func) is smaller.
+int ensure_dynamic_lds(const void* func, int bytes);
+
 
 // sin and cos of an fp32 angle for the 16-bit cache paths: exact range reduction in double (the
 // angle is position * frequency, tens of thousands of radians for long contexts), then the hardware

@@ -597,12 +597,9 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
                      (A.sink_stride[2] * es) % 16 == 0;
     if (!vec && A.HID > 8 * CKV_WAVE) return CKV_ERR_UNSUPPORTED;
 
-    int dev = 0, lds_max = 65536;
-    CKV_HIP_TRY(hipGetDevice(&dev));
-    if (hipDeviceGetAttribute(&lds_max, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) {
-        (void)hipGetLastError();
-        lds_max = 65536;
-    }
+    DeviceInfo di;
+    if (int rc = current_device_info(&di)) return rc;
+    const int lds_max = di.lds_max;
     int qmax = (int)((lds_max - 4096) / 40);
     qmax = qmax / 64 * 64;
     if (qmax > kPlanMaxTokens) qmax = kPlanMaxTokens;
@@ -622,10 +619,7 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
         p.do_pos = (off + ksub == A.K) ? 1 : 0;
         const int T = ksub <= 256 ? 256 : 1024;  // few tokens: a small block plans them
         const size_t lds = plan_lds_bytes(ksub);
-        if (lds > 48 * 1024) {
-            CKV_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(ckv_update_plan_kernel),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        }
+        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(ckv_update_plan_kernel), (int)lds)) return rc;
         {
             StageScope sc(CKV_STAGE_PLAN, stream);
             hipLaunchKernelGGL(ckv_update_plan_kernel, dim3((unsigned)(A.N * A.H)), dim3(T), lds, stream, p);

@@ -52,9 +52,9 @@ def attention(q, k, v, causal, sm_scale, mask, beta):
     a.causal = int(bool(causal))
     a.dtype = _abi.dtype_code(q.dtype)
     need = lib.ckv_dense_workspace_bytes(B, H, n_ctx, n_kv, D, a.dtype)
-    ws = workspace(q.device, need)
-    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
+        ws = workspace(q.device, need, stream)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
         _abi.check(lib.ckv_attn_dense(C.byref(a), C.c_void_p(stream)), "ckv_attn_dense")
     return o, scores

@@ -135,3 +135,61 @@ def test_fill_update_args_enforces_reference_preconditions():
         fill(mask=torch.ones(1, 2, 4))
     with pytest.raises(TypeError):
         fill(pos=torch.zeros(1, 2, 4, dtype=torch.int32))
+
+
+def test_memoised_update_arguments_follow_reassigned_state_tensors():
+    """The reference reassigns ``score_cache[l]`` every call (cascade_attention.py:222-224).  The memoised
+    argument block holds raw pointers, so it must follow the tensor the cache holds NOW, also when a freed
+    tensor's Python id is handed to a new one."""
+    from cascading_kv_cache_amd.cascading_cache import CascadingKVCache
+
+    c = CascadingKVCache(window_length=4, num_sink_tokens=2, max_batch_size=1, heads=2, dim=8, max_seq_len=8,
+                         device="cpu", dtype=torch.float32, layers=1, verbose=False)
+    k, v, s = torch.zeros(1, 2, 3, 8), torch.zeros(1, 2, 3, 8), torch.zeros(1, 2, 3)
+    keep = []  # keeps every tensor alive so each reassignment lands at a new address
+    for step in range(80):  # more steps than the memo holds entries
+        fresh = c.score_cache[0] * 0.5 + 1.0
+        keep.append(fresh)
+        c.score_cache[0] = fresh
+        a = c._update_args(k, v, s, 0)
+        assert a.cache_s == fresh.data_ptr(), f"step {step}: stale score-cache pointer in the argument block"
+        assert a.cache_k == c.key_cache[0].data_ptr() and a.k == k.data_ptr()
+    # the same address again -> the same block is reused, with the input pointers refreshed
+    k2 = torch.ones(1, 2, 3, 8)
+    b = c._update_args(k2, v, s, 0)
+    assert b is a and b.k == k2.data_ptr()
+    # ids may repeat, addresses of live tensors cannot: drop and re-create without keeping
+    for step in range(80):
+        c.score_cache[0] = c.score_cache[0] * 0.5
+        assert c._update_args(k, v, s, 0).cache_s == c.score_cache[0].data_ptr()
+
+
+def test_chunk_is_checked_against_the_cache_before_any_pointer_leaves():
+    from cascading_kv_cache_amd.cascade_attention import check_against_cache
+    from cascading_kv_cache_amd.cascading_cache import CascadingKVCache
+
+    c = CascadingKVCache(window_length=4, num_sink_tokens=2, max_batch_size=2, heads=2, dim=8, max_seq_len=8,
+                         device="cpu", dtype=torch.float16, layers=1, verbose=False)
+
+    def chunk(B=2, H=4, KVH=2, Q=3, D=8, dtype=torch.float16):
+        return torch.zeros(B, H, Q, D, dtype=dtype), torch.zeros(B, KVH, Q, D, dtype=dtype), torch.zeros(B, KVH, Q, D, dtype=dtype)
+
+    check_against_cache(*chunk(), c, 0)
+    check_against_cache(*chunk(B=1), c, 0)                    # fewer streams than the cache holds is fine
+    for bad in (dict(B=3), dict(KVH=1, H=4), dict(D=16), dict(H=3)):
+        with pytest.raises(ValueError):
+            check_against_cache(*chunk(**bad), c, 0)
+    with pytest.raises(TypeError):                            # a bf16 chunk over an fp16 cache is not reinterpreted
+        check_against_cache(*chunk(dtype=torch.bfloat16), c, 0)
+    with pytest.raises(ValueError):
+        check_against_cache(*chunk(), c, 1)
+    # the update operator checks the same sizes
+    k = torch.zeros(3, 2, 3, 8, dtype=torch.float16)
+    with pytest.raises(ValueError):
+        c._update_args(k, k.clone(), torch.zeros(3, 2, 3, dtype=torch.float16), 0)
+    k = torch.zeros(2, 2, 3, 16, dtype=torch.float16)
+    with pytest.raises(ValueError):
+        c._update_args(k, k.clone(), torch.zeros(2, 2, 3, dtype=torch.float16), 0)
+    k = torch.zeros(2, 2, 3, 8, dtype=torch.float16)
+    with pytest.raises(ValueError):
+        c._update_args(k, k.clone(), torch.zeros(2, 1, 3, dtype=torch.float16), 0)
