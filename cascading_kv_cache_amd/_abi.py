@@ -205,6 +205,10 @@ def lib():
         L = C.CDLL(LIB_PATH)
         L.ckv_update.argtypes = [C.POINTER(UpdateArgs), VP]
         L.ckv_update.restype = C.c_int
+        L.ckv_update_static.argtypes = [C.POINTER(UpdateArgs), VP]
+        L.ckv_update_static.restype = C.c_int
+        L.ckv_update_static_scratch_bytes.argtypes = []
+        L.ckv_update_static_scratch_bytes.restype = I64
         L.ckv_update_workspace_bytes.argtypes = [I64, I64, I64, I64, C.c_int32]
         L.ckv_update_workspace_bytes.restype = I64
         L.ckv_attn.argtypes = [C.POINTER(AttnArgs), VP]

@@ -204,6 +204,7 @@ extern "C" const char* ckv_strerror(int status) {
         case CKV_ERR_WORKSPACE: return "workspace missing or too small";
         case CKV_ERR_UNSUPPORTED: return "request outside what the kernels implement";
         case CKV_ERR_LAUNCH: return "the HIP runtime rejected a launch";
+        case CKV_ERR_TOO_LARGE: return "sizes exceed the fixed scratch of ckv_update_static (use ckv_update with a workspace)";
         default: return "unknown ckv status";
     }
 }

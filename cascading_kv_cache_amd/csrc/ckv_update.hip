@@ -24,6 +24,8 @@
 // slot depends on scores, and that is decided inside the group of arrivals between two inserts.
 #include "ckv_common.h"
 
+#include <mutex>
+
 namespace ckv {
 namespace {
 
@@ -565,26 +567,36 @@ extern "C" int64_t ckv_update_workspace_bytes(int64_t N, int64_t H, int64_t K, i
            ckv::align_up(N * H * (int64_t)sizeof(int32_t), 256) + 256;
 }
 
-extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
-    using namespace ckv;
-    if (!args) return CKV_ERR_NULL;
-    const ckv_update_args& A = *args;
-    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
-    if (A.dtype != CKV_F32 && A.dtype != CKV_F16 && A.dtype != CKV_BF16) return CKV_ERR_DTYPE;
-    if (A.N <= 0 || A.H <= 0 || A.K < 0 || A.HID <= 0 || A.num_sink < 0) return CKV_ERR_SHAPE;
-    if (A.window_size <= 0 || A.cascades <= 0 || A.cascades > kMaxCascades) return CKV_ERR_SHAPE;
-    if ((int64_t)A.cascades * A.window_size != A.max_seq_len) return CKV_ERR_SHAPE;
-    if (A.max_seq_len + A.num_sink >= (int64_t)1 << 30 || A.K >= (int64_t)1 << 30) return CKV_ERR_SHAPE;
-    if (A.N * A.H > 65535) return CKV_ERR_UNSUPPORTED;
-    if (!A.cache_k || !A.cache_v || !A.cache_s || !A.mask || !A.pos || !A.og_pos || !A.stored_tokens ||
-        !A.start_indices || !A.stored_sinks || !A.do_cache_every_n || !A.real_token_idx)
-        return CKV_ERR_NULL;
-    if (A.num_sink > 0 && (!A.sink_k || !A.sink_v || !A.sink_mask || !A.sink_pos)) return CKV_ERR_NULL;
-    if (A.K == 0) return CKV_OK;
-    if (!A.k || !A.v || !A.s) return CKV_ERR_NULL;
-    const int64_t need = ckv_update_workspace_bytes(A.N, A.H, A.K, A.max_seq_len, A.cascades);
-    if (!A.workspace || A.workspace_bytes < need) return CKV_ERR_WORKSPACE;
+// Scratch of the entry point that allocates nothing (ckv_update_static): one array per device, part of the
+// code object, held until the process ends.  In host code its name is a stand-in, not a device address:
+// the address is looked up once per device (static_scratch below) and only that address is ever handed to
+// kernels.
+constexpr int64_t kStaticScratchBytes = (int64_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
+namespace ckv {
+namespace {
+
+constexpr int kScratchDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kScratchDevices];
+
+int static_scratch(void** out) {
+    int dev = 0;
+    CKV_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kScratchDevices) return CKV_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        CKV_HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));  // the current device's copy of the array
+        if (!ptr) return CKV_ERR_LAUNCH;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return CKV_OK;
+}
+
+int run_update(const ckv_update_args& A, void* workspace, hipStream_t stream) {
     const int es = (int)elem_bytes(A.dtype);
     const bool vec = A.kv_stride[3] == 1 && A.cache_stride[3] == 1 && (A.num_sink == 0 || A.sink_stride[3] == 1) &&
                      (A.HID * es) % 16 == 0 && A.HID * es <= 16 * 64 && aligned16(A.k) && aligned16(A.v) &&
@@ -607,9 +619,9 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
 
     UpdateParams p;
     p.a = A;
-    p.first = reinterpret_cast<int32_t*>(A.workspace);
+    p.first = reinterpret_cast<int32_t*>(workspace);
     p.next_of = p.first + A.N * A.H * A.K;
-    p.pos_flag = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(A.workspace) +
+    p.pos_flag = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(workspace) +
                                             align_up(A.N * A.H * (A.K + A.max_seq_len) * (int64_t)sizeof(int32_t), 256));
 
     for (int64_t off = 0; off < A.K; off += qmax) {
@@ -659,4 +671,57 @@ extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
         CKV_HIP_TRY(hipGetLastError());
     }
     return CKV_OK;
+}
+
+// everything ckv_update checks before it looks at the scratch; *empty: nothing to do
+int check_update_args(const ckv_update_args* args, bool* empty) {
+    *empty = false;
+    if (!args) return CKV_ERR_NULL;
+    const ckv_update_args& A = *args;
+    if (A.dtype != CKV_F32 && A.dtype != CKV_F16 && A.dtype != CKV_BF16) return CKV_ERR_DTYPE;
+    if (A.N <= 0 || A.H <= 0 || A.K < 0 || A.HID <= 0 || A.num_sink < 0) return CKV_ERR_SHAPE;
+    if (A.window_size <= 0 || A.cascades <= 0 || A.cascades > kMaxCascades) return CKV_ERR_SHAPE;
+    if ((int64_t)A.cascades * A.window_size != A.max_seq_len) return CKV_ERR_SHAPE;
+    if (A.max_seq_len + A.num_sink >= (int64_t)1 << 30 || A.K >= (int64_t)1 << 30) return CKV_ERR_SHAPE;
+    if (A.N * A.H > 65535) return CKV_ERR_UNSUPPORTED;
+    if (!A.cache_k || !A.cache_v || !A.cache_s || !A.mask || !A.pos || !A.og_pos || !A.stored_tokens ||
+        !A.start_indices || !A.stored_sinks || !A.do_cache_every_n || !A.real_token_idx)
+        return CKV_ERR_NULL;
+    if (A.num_sink > 0 && (!A.sink_k || !A.sink_v || !A.sink_mask || !A.sink_pos)) return CKV_ERR_NULL;
+    if (A.K == 0) {
+        *empty = true;
+        return CKV_OK;
+    }
+    if (!A.k || !A.v || !A.s) return CKV_ERR_NULL;
+    return CKV_OK;
+}
+
+}  // namespace
+}  // namespace ckv
+
+extern "C" int ckv_update(const ckv_update_args* args, void* stream_) {
+    using namespace ckv;
+    bool empty;
+    if (int rc = check_update_args(args, &empty)) return rc;
+    if (empty) return CKV_OK;
+    const ckv_update_args& A = *args;
+    const int64_t need = ckv_update_workspace_bytes(A.N, A.H, A.K, A.max_seq_len, A.cascades);
+    if (!A.workspace || A.workspace_bytes < need) return CKV_ERR_WORKSPACE;
+    return run_update(A, A.workspace, reinterpret_cast<hipStream_t>(stream_));
+}
+
+extern "C" int64_t ckv_update_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int ckv_update_static(const ckv_update_args* args, void* stream_) {
+    using namespace ckv;
+    bool empty;
+    if (int rc = check_update_args(args, &empty)) return rc;
+    if (empty) return CKV_OK;
+    const ckv_update_args& A = *args;
+    if (ckv_update_workspace_bytes(A.N, A.H, A.K, A.max_seq_len, A.cascades) > kStaticScratchBytes) return CKV_ERR_TOO_LARGE;
+    void* ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    // Nothing in the scratch has to start at zero: the plan kernel writes every chain entry and flag the
+    // apply kernel reads, whatever the last call left there.
+    return run_update(A, ws, reinterpret_cast<hipStream_t>(stream_));
 }

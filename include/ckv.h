@@ -50,7 +50,8 @@ typedef enum ckv_status {
     CKV_ERR_DTYPE = -4,       /* unknown dtype */
     CKV_ERR_WORKSPACE = -5,   /* workspace missing or too small */
     CKV_ERR_UNSUPPORTED = -6, /* valid request outside what the kernels implement */
-    CKV_ERR_LAUNCH = -7       /* the HIP runtime rejected a launch */
+    CKV_ERR_LAUNCH = -7,      /* the HIP runtime rejected a launch */
+    CKV_ERR_TOO_LARGE = -8    /* sizes beyond the fixed scratch of ckv_update_static */
 } ckv_status;
 
 typedef enum ckv_head_reduction {
@@ -122,6 +123,17 @@ int64_t ckv_update_workspace_bytes(int64_t N, int64_t H, int64_t K, int64_t max_
  * _update_kv_cache_inner (cascading_cache.py:381-774) would, and rewrites `pos`.  The caller
  * adds K to its token counter afterwards (cascading_cache.py:1346). */
 int ckv_update(const ckv_update_args* args, void* stream);
+
+/* ckv_update for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same kernels and
+ * same results as ckv_update, except that `workspace` / `workspace_bytes` are ignored: the scratch is a
+ * fixed array inside the library (ckv_update_static_scratch_bytes() = 32 MiB per device, held until the
+ * process ends), so the call allocates nothing and needs no workspace from the caller.  Sizes whose
+ * ckv_update_workspace_bytes(...) exceeds that array are refused with CKV_ERR_TOO_LARGE.  All calls on
+ * one device share the array: calls that overlap in time on one device (different streams, or different
+ * host threads) race on it; calls on one stream are ordered and safe. */
+int64_t ckv_update_static_scratch_bytes(void);
+int ckv_update_static(const ckv_update_args* args, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Attention over [sink | cascades | current chunk] with RoPE from the cache's position ids,

@@ -54,7 +54,7 @@ def test_ctypes_mirrors_match_struct_sizes(lib):
 
 def test_status_strings(lib):
     seen = set()
-    for code in range(0, -8, -1):
+    for code in range(0, -9, -1):
         text = lib.ckv_strerror(code).decode()
         assert text and text not in seen
         seen.add(text)
