@@ -173,6 +173,7 @@ class OracleCascadeAttention:
         scores = scores.repeat(1, query_states.size(1), 1)
         self.last_new_scores = scores
         self.last_ema = ema_scores
+        self.last_score_cache = cache.score_cache.clone()  # what the update's evictions will carry
 
         cache.update(key_states, value_states, score_states=scores)
         if return_probs:

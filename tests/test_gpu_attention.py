@@ -15,9 +15,8 @@ from oracle.update import OracleCache
 
 pytestmark = pytest.mark.gpu
 
-STATE = ("key_cache", "value_cache", "score_cache", "sink_keys", "sink_values", "mask", "sink_mask", "pos",
-         "og_pos", "sink_pos", "stored_tokens", "start_indices", "stored_sinks")
-META = ("mask", "sink_mask", "pos", "sink_pos", "stored_tokens", "start_indices", "stored_sinks")
+from parity_helpers import (META, STATE, FlipLedger, assert_scores_close, check_update_against_replay, clone_oracle,
+                            flip_margins, push_state, tol)
 
 
 def make_pair(B, KVH, D, NS, W, C, dtype, func="pow2", eager=True, reduction="mean"):
@@ -31,30 +30,14 @@ def make_pair(B, KVH, D, NS, W, C, dtype, func="pow2", eager=True, reduction="me
     return gpu, cpu
 
 
-def push_state(gpu, cpu):
-    """Teacher forcing: the GPU cache restarts every chunk from the oracle's state."""
-    for name in STATE:
-        getattr(gpu, name)[0].copy_(getattr(cpu, name))
-    gpu.seen_tokens_by_layer[0] = int(cpu.seen_tokens)
-    gpu._seen_host[0] = int(cpu.seen_tokens)
-
-
-def tol(dtype):
-    return 1e-4 if dtype == torch.float32 else 2e-2
-
-
-def assert_scores_close(got, want, dtype, what):
-    got, want = got.float().cpu(), want.float().cpu()
-    scale = want.abs().max().item() + 1e-30
-    ulp = {torch.float32: 2.0 ** -23, torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -10}[dtype]
-    # float16 scores live among the subnormals (1e-7 ~ 2 * 2^-24): allow two quanta of the format
-    quantum = 2.0 ** -24 if dtype == torch.float16 else 0.0
-    err = (got - want).abs().max().item()
-    assert err <= (tol(dtype) + ulp) * scale + 2 * quantum, f"{what}: max err {err:.3e} vs scale {scale:.3e}"
-
-
 def run_teacher_forced(B, H, KVH, D, NS, W, C, Q, chunks, dtype, seed, reduction="mean", homogeneous=False,
-                       eager=True, theta=5e5, std=1.0, q_last=None, do_og_pos=False):
+                       eager=True, theta=5e5, std=1.0, q_last=None, do_og_pos=False, steps=None):
+    """Stream chunks through the library and the oracle, the GPU cache restarting every chunk from the
+    oracle's state.  Per chunk: outputs and both score inputs of the update within tolerance, metadata
+    bit-exact, the library's update equal to the oracle's update run on the library's scores, K/V of every
+    slot that holds the same token bit-exact, and every slot that holds a different token explained by an
+    oracle margin below twice the largest score difference.  ``steps``: chunk lengths (overrides Q / chunks /
+    q_last).  Returns the ledger of differing slots."""
     from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
 
     gpu, cpu = make_pair(B, KVH, D, NS, W, C, dtype, eager=eager, reduction=reduction)
@@ -62,74 +45,95 @@ def run_teacher_forced(B, H, KVH, D, NS, W, C, Q, chunks, dtype, seed, reduction
                                    homogeneous_heads=homogeneous, do_og_pos=do_og_pos)
     inv_freq = default_inv_freq(D, theta, "cuda:0")
     gen = torch.Generator().manual_seed(seed)
-    flips = 0
-    compared = 0
-    for c in range(chunks):
-        qn = q_last if (q_last is not None and c == chunks - 1) else Q
+    ledger = FlipLedger(dtype)
+    if steps is None:
+        steps = [q_last if (q_last is not None and c == chunks - 1) else Q for c in range(chunks)]
+    for c, qn in enumerate(steps):
         q = (torch.randn(B, H, qn, D, generator=gen) * std).to(dtype)
         k = (torch.randn(B, KVH, qn, D, generator=gen) * std).to(dtype)
         v = (torch.randn(B, KVH, qn, D, generator=gen) * std).to(dtype)
         push_state(gpu, cpu)
+        replay = clone_oracle(cpu)
+        pre = {"og_pos": cpu.og_pos.clone(), "mask": cpu.mask.clone()}
+        seen_before = int(cpu.seen_tokens)
         out_g, new_g = cascade_attention(q.cuda(), k.cuda(), v.cuda(), gpu, 0, inv_freq, head_reduction=reduction,
                                          homogeneous_heads=homogeneous, update_cache=False, do_og_pos=do_og_pos)
+        scores_g = gpu.score_cache[0].cpu().clone()   # after the attention call, before the update
         gpu.update(k.cuda(), v.cuda(), 0, score_states=new_g)
         out_c = layer.forward(q, k, v, cpu)
         torch.cuda.synchronize()
+        ctx = f"chunk {c} (q={qn})"
         err = (out_g.float().cpu() - out_c.float()).abs().max().item()
-        assert err <= tol(dtype), f"chunk {c}: out max err {err:.3e}"
-        assert_scores_close(new_g, layer.last_new_scores[:, :KVH], dtype, f"chunk {c} new-token scores")
+        assert err <= tol(dtype), f"{ctx}: out max err {err:.3e}"
+        new_c = layer.last_new_scores[:, :KVH]
+        eps = assert_scores_close(new_g, new_c, dtype, f"{ctx} new-token scores")
+        eps = max(eps, assert_scores_close(scores_g, layer.last_score_cache, dtype, f"{ctx} score cache after attention"))
         for name in META:
-            assert torch.equal(getattr(gpu, name)[0].cpu(), getattr(cpu, name)), f"chunk {c}: {name}"
-        same = gpu.og_pos[0].cpu() == cpu.og_pos
-        flips += int((~same).sum())
-        compared += same.numel()
-        if bool(same.all()):
-            assert_scores_close(gpu.score_cache[0], cpu.score_cache, dtype, f"chunk {c} score cache")
-    return flips, compared
+            assert torch.equal(getattr(gpu, name)[0].cpu(), getattr(cpu, name)), f"{ctx}: {name}"
+        # the update itself: bit-exact against the oracle's update on the same (the library's) scores
+        check_update_against_replay(gpu, replay, k, v, scores_g, new_g.cpu(), ctx=ctx)
+        # slots that hold the same token as in the oracle: K and V bit-exact, scores within tolerance
+        og_g = gpu.og_pos[0].cpu()
+        same = og_g == cpu.og_pos
+        for name in ("key_cache", "value_cache"):
+            g, w = getattr(gpu, name)[0].cpu(), getattr(cpu, name)
+            assert torch.equal(g[same].view(torch.uint8), w[same].view(torch.uint8)), f"{ctx}: {name} of unflipped slots"
+        sg, sw = gpu.score_cache[0].cpu().float(), cpu.score_cache.float()
+        assert_scores_close(torch.where(same, sg, sw), sw, dtype, f"{ctx} score cache of unflipped slots")
+        # slots that hold a different token: the oracle's own margin between the two must be tie-level.
+        # A chunk shorter than two windows cannot evict what it has just placed in a deeper cascade, so every
+        # differing slot is one tournament decided differently.
+        margins = flip_margins(og_g, cpu, pre, seen_before, layer.last_score_cache, new_c)
+        ledger.record(margins, eps, same.numel(), primary_only=qn < 2 * W, ctx=ctx)
+    print(ledger.summary())
+    return ledger
 
 
 def test_config1_float32_stream():
     """The float32 benchmark case: B=1, 32q/8kv heads, D=128, sink 4, window 512 in C=4, 4096 tokens in
     chunks of 256, theta 5e5, float32."""
-    flips, compared = run_teacher_forced(1, 32, 8, 128, 4, 128, 4, 256, 16, torch.float32, seed=1)
-    assert flips == 0, f"{flips} of {compared} slots differ in og_pos (eviction decisions flipped)"
+    led = run_teacher_forced(1, 32, 8, 128, 4, 128, 4, 256, 16, torch.float32, seed=1)
+    assert led.flips == 0, f"{led.flips} of {led.compared} slots differ in og_pos (eviction decisions flipped)"
 
 
 @pytest.mark.parametrize("reduction,homogeneous", [("mean", False), ("max", False), ("median", False),
                                                    ("mean", True), ("max", True), ("median", True)])
 def test_small_float32_reductions(reduction, homogeneous):
-    flips, compared = run_teacher_forced(2, 6, 2, 16, 3, 8, 4, 12, 10, torch.float32, seed=2, reduction=reduction,
-                                         homogeneous=homogeneous, eager=False, theta=1e4)
-    assert flips == 0
+    led = run_teacher_forced(2, 6, 2, 16, 3, 8, 4, 12, 10, torch.float32, seed=2, reduction=reduction,
+                             homogeneous=homogeneous, eager=False, theta=1e4)
+    assert led.flips == 0
 
 
 def test_ragged_last_chunk_and_decode_steps_float32():
-    flips, _ = run_teacher_forced(1, 4, 2, 32, 4, 16, 2, 10, 6, torch.float32, seed=3, q_last=3)
-    assert flips == 0
-    flips, _ = run_teacher_forced(2, 4, 4, 64, 2, 8, 2, 1, 40, torch.float32, seed=4)
-    assert flips == 0
+    assert run_teacher_forced(1, 4, 2, 32, 4, 16, 2, 10, 6, torch.float32, seed=3, q_last=3).flips == 0
+    assert run_teacher_forced(2, 4, 4, 64, 2, 8, 2, 1, 40, torch.float32, seed=4).flips == 0
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_sixteen_bit_stream(dtype):
-    flips, compared = run_teacher_forced(2, 8, 2, 128, 8, 64, 4, 64, 8, dtype, seed=5, std=0.5)
-    # 16-bit scores tie or differ by one ulp all the time, so decisions may flip; report only
-    print(f"{dtype}: {flips}/{compared} slots chose a different token (tie-level score differences)")
+    led = run_teacher_forced(2, 8, 2, 128, 8, 64, 4, 64, 8, dtype, seed=5, std=0.5)
+    # 16-bit scores tie or differ in the last place all the time, so a few decisions go the other way; each one
+    # is checked against the oracle's margin inside run_teacher_forced, and they stay a small minority
+    assert led.flips <= 0.05 * led.compared, led.summary()
 
 
-@pytest.mark.parametrize("H,KVH,Q,W,C,NS,eager,dtype", [
-    (8, 2, 128, 256, 4, 64, True, torch.bfloat16),     # G = 4, the Llama grouping
-    (14, 2, 96, 128, 4, 64, True, torch.bfloat16),     # G = 7, the Qwen2 grouping
-    (4, 4, 200, 128, 2, 8, False, torch.bfloat16),     # G = 1, ragged chunk, sparse fill
-    (16, 2, 64, 64, 8, 64, True, torch.float16),       # G = 8
-    (8, 2, 300, 128, 4, 64, False, torch.bfloat16),    # chunk longer than a cascade window
-])
-def test_mfma_prefill_head128(H, KVH, Q, W, C, NS, eager, dtype):
+REDUCTIONS = [("max", False), ("median", False), ("mean", True), ("max", True), ("median", True)]
+
+
+@pytest.mark.parametrize("H,KVH,Q,W,C,NS,eager,dtype,reduction,homogeneous", [
+    (8, 2, 128, 256, 4, 64, True, torch.bfloat16, "mean", False),     # G = 4, the Llama grouping
+    (14, 2, 96, 128, 4, 64, True, torch.bfloat16, "mean", False),     # G = 7, the Qwen2 grouping
+    (4, 4, 200, 128, 2, 8, False, torch.bfloat16, "mean", False),     # G = 1, ragged chunk, sparse fill
+    (16, 2, 64, 64, 8, 64, True, torch.float16, "mean", False),       # G = 8
+    (8, 2, 300, 128, 4, 64, False, torch.bfloat16, "mean", False),    # chunk longer than two cascade windows
+] + [(8, 2, 128, 256, 4, 64, True, torch.bfloat16, r, h) for r, h in REDUCTIONS]     # cascade_attention.py:231-248
+  + [(14, 2, 96, 128, 4, 64, False, torch.float16, r, h) for r, h in REDUCTIONS])
+def test_mfma_prefill_head128(H, KVH, Q, W, C, NS, eager, dtype, reduction, homogeneous):
     """head_dim 128 in 16-bit takes the MFMA kernels: stream chunks while the cache fills up and
-    starts evicting, teacher-forced against the oracle."""
-    flips, compared = run_teacher_forced(2, H, KVH, 128, NS, W, C, Q, 8, dtype, seed=11, eager=eager, std=0.7,
-                                         q_last=Q - 37)
-    print(f"{flips}/{compared} slots chose a different token")
+    starts evicting, teacher-forced against the oracle, for every head reduction and both head modes."""
+    led = run_teacher_forced(2, H, KVH, 128, NS, W, C, Q, 8, dtype, seed=11, eager=eager, std=0.7,
+                             q_last=Q - 37, reduction=reduction, homogeneous=homogeneous)
+    assert led.flips <= 0.05 * led.compared, led.summary()
 
 
 @pytest.mark.parametrize("dtype,std", [(torch.bfloat16, 0.05), (torch.bfloat16, 1.0), (torch.bfloat16, 3.0),
@@ -160,41 +164,26 @@ def test_mfma_prefill_wide_range_of_logits(dtype, std):
         assert torch.isfinite(new_scores.float()).all() and torch.isfinite(cache.score_cache[0].float()).all()
 
 
-@pytest.mark.parametrize("H,KVH,W,C,NS,eager,dtype", [
-    (8, 2, 64, 4, 8, True, torch.bfloat16),      # G = 4
-    (14, 2, 32, 4, 4, False, torch.bfloat16),    # G = 7
-    (4, 4, 32, 2, 4, True, torch.float16),       # G = 1
-    (16, 2, 16, 8, 64, True, torch.bfloat16),    # G = 8
-    (8, 4, 64, 2, 6, True, torch.float32),       # G = 2, float32
-])
-def test_decode_head128(H, KVH, W, C, NS, eager, dtype):
+@pytest.mark.parametrize("H,KVH,W,C,NS,eager,dtype,reduction,homogeneous", [
+    (8, 2, 64, 4, 8, True, torch.bfloat16, "mean", False),      # G = 4: the streaming kernel
+    (14, 2, 32, 4, 4, False, torch.bfloat16, "mean", False),    # G = 7: the tile-per-workgroup kernel
+    (4, 4, 32, 2, 4, True, torch.float16, "mean", False),       # G = 1
+    (16, 2, 16, 8, 64, True, torch.bfloat16, "mean", False),    # G = 8
+    (8, 4, 64, 2, 6, True, torch.float32, "mean", False),       # G = 2, float32
+    (8, 4, 64, 2, 6, True, torch.float32, "median", True),
+] + [(8, 2, 64, 4, 8, True, torch.bfloat16, r, h) for r, h in REDUCTIONS]       # cascade_attention.py:231-248
+  + [(14, 2, 32, 4, 4, False, torch.float16, r, h) for r, h in REDUCTIONS])
+def test_decode_head128(H, KVH, W, C, NS, eager, dtype, reduction, homogeneous):
     """q == 1 with head_dim 128 takes the bandwidth-bound decode kernels: fill part of the cache
-    with a few chunks, then run single-token steps (cache still filling, then evicting)."""
-    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
-
-    B, D = 2, 128
-    gpu, cpu = make_pair(B, KVH, D, NS, W, C, dtype, eager=eager)
-    layer = OracleCascadeAttention(H, KVH, D, rope_theta=5e5)
-    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
-    gen = torch.Generator().manual_seed(21)
+    with a few chunks, then run single-token steps (cache still filling, then evicting), for every head
+    reduction and both head modes."""
     steps = [W * C // 2 + NS, 17] + [1] * (W * C // 2 + 40)
-    for c, qn in enumerate(steps):
-        q = (torch.randn(B, H, qn, D, generator=gen) * 0.7).to(dtype)
-        k = (torch.randn(B, KVH, qn, D, generator=gen) * 0.7).to(dtype)
-        v = (torch.randn(B, KVH, qn, D, generator=gen) * 0.7).to(dtype)
-        push_state(gpu, cpu)
-        out_g, new_g = cascade_attention(q.cuda(), k.cuda(), v.cuda(), gpu, 0, inv_freq)
-        if c == 0:
-            layer.query_pos = None
-        out_c = layer.forward(q, k, v, cpu)
-        torch.cuda.synchronize()
-        err = (out_g.float().cpu() - out_c.float()).abs().max().item()
-        assert err <= tol(dtype), f"step {c} (q={qn}): out max err {err:.3e}"
-        assert_scores_close(new_g, layer.last_new_scores[:, :KVH], dtype, f"step {c} new-token scores")
-        for name in META:
-            assert torch.equal(getattr(gpu, name)[0].cpu(), getattr(cpu, name)), f"step {c}: {name}"
-        if bool((gpu.og_pos[0].cpu() == cpu.og_pos).all()):
-            assert_scores_close(gpu.score_cache[0], cpu.score_cache, dtype, f"step {c} score cache")
+    led = run_teacher_forced(2, H, KVH, 128, NS, W, C, None, None, dtype, seed=21, eager=eager, std=0.7, steps=steps,
+                             reduction=reduction, homogeneous=homogeneous)
+    if dtype == torch.float32:
+        assert led.flips == 0, led.summary()
+    else:
+        assert led.flips <= 0.05 * led.compared, led.summary()
 
 
 @pytest.mark.parametrize("H,KVH,dtype,fill", [
@@ -254,10 +243,10 @@ def test_original_position_mode(dtype, D, H, KVH, Q, q_last):
     """cascade_attention.py:141-144, 161-164 (do_og_pos): cached keys are rotated per (batch, head) at the index
     of the token a slot holds; without eager fill the heads soon keep different tokens."""
     chunks = 40 if Q == 1 else 8
-    flips, compared = run_teacher_forced(2, H, KVH, D, 4, 16, 2, Q, chunks, dtype, seed=21, eager=False, std=0.7,
-                                         q_last=q_last, do_og_pos=True)
+    led = run_teacher_forced(2, H, KVH, D, 4, 16, 2, Q, chunks, dtype, seed=21, eager=False, std=0.7,
+                             q_last=q_last, do_og_pos=True)
     if dtype == torch.float32:
-        assert flips == 0, f"{flips} of {compared} slots differ in og_pos"
+        assert led.flips == 0, led.summary()
 
 
 @pytest.mark.parametrize("do_og_pos", [False, True])

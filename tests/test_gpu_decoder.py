@@ -7,6 +7,9 @@ import torch
 from oracle.attention import OracleCascadeAttention
 from oracle.update import OracleCache
 
+from parity_helpers import (META, FlipLedger, assert_scores_close, check_update_against_replay, clone_oracle,
+                            flip_margins, push_state, tol)
+
 pytestmark = pytest.mark.gpu
 
 
@@ -52,6 +55,68 @@ def test_small_decoder_prefill_and_greedy_steps_against_the_oracle(dtype):
     for i, oc in enumerate(caches):
         for name in ("mask", "sink_mask", "pos", "sink_pos", "stored_tokens", "start_indices", "stored_sinks", "og_pos"):
             assert torch.equal(getattr(cache, name)[i].cpu(), getattr(oc, name)), f"layer {i}: {name}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_decoder_layers_past_the_window_teacher_forced(dtype):
+    """The multi-layer path once the cascades evict: a stream of more than twice the window goes through a
+    two-layer decoder in strides and then token by token.  Every layer's cache layer restarts each step from
+    that layer's oracle state and the oracle's attention gets the device's own q/k/v, so a tie-level decision
+    cannot snowball; per layer and step the attention output, both score inputs, the metadata, the update
+    (against the oracle's update on the library's scores) and the margin of every differing slot are checked."""
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
+    from cascading_kv_cache_amd.decoder import PRESETS, CascadeDecoder
+
+    cfg = PRESETS["tiny"]
+    model = CascadeDecoder(cfg, dtype=dtype, device="cuda:0", seed=7)
+    B, NS, W, C = 2, 4, 32, 4
+    cache = model.new_cache(W * C, C, batch=B, num_sink_tokens=NS)
+    caches = [OracleCache(window_length=W, num_sink_tokens=NS, max_batch_size=B, heads=cfg.num_kv_heads,
+                          dim=cfg.head_dim, max_seq_len=W * C, dtype=dtype) for _ in range(cfg.num_layers)]
+    oracles = [OracleCascadeAttention(cfg.num_heads, cfg.num_kv_heads, cfg.head_dim, rope_theta=cfg.rope_theta,
+                                      head_reduction=cfg.head_reduction) for _ in range(cfg.num_layers)]
+    inv_freq = default_inv_freq(cfg.head_dim, cfg.rope_theta, "cuda:0")
+    steps = [48] * 6 + [1] * 14          # 302 tokens through a 4 + 128-slot cache
+    ids = torch.randint(0, cfg.vocab_size, (B, sum(steps)), generator=torch.Generator().manual_seed(8)).cuda()
+    ledger = FlipLedger(dtype)
+    done = 0
+    with torch.no_grad():
+        for n, qn in enumerate(steps):
+            x = model.embed_tokens(ids[:, done:done + qn])
+            for li, layer in enumerate(model.layers):
+                oc, attn_o = caches[li], oracles[li]
+                h = layer.input_layernorm(x)
+                qs, ks, vs = layer.self_attn.qkv(h, (B, qn, cfg.num_heads, cfg.head_dim),
+                                                 (B, qn, cfg.num_kv_heads, cfg.head_dim))
+                push_state(cache, oc, layer=li)
+                replay = clone_oracle(oc)
+                pre = {"og_pos": oc.og_pos.clone(), "mask": oc.mask.clone()}
+                seen_before = int(oc.seen_tokens)
+                out_g, new_g = cascade_attention(qs, ks, vs, cache, li, inv_freq, head_reduction=cfg.head_reduction,
+                                                 update_cache=False)
+                scores_g = cache.score_cache[li].cpu().clone()
+                cache.update(ks, vs, li, score_states=new_g)
+                qc, kc, vc = qs.cpu(), ks.cpu(), vs.cpu()
+                out_c = attn_o.forward(qc, kc, vc, oc)
+                ctx = f"step {n} (q={qn}) layer {li}"
+                err = (out_g.float().cpu() - out_c.float()).abs().max().item()
+                assert err <= tol(dtype), f"{ctx}: out max err {err:.3e}"
+                new_c = attn_o.last_new_scores[:, :cfg.num_kv_heads]
+                eps = assert_scores_close(new_g, new_c, dtype, f"{ctx} new-token scores")
+                eps = max(eps, assert_scores_close(scores_g, attn_o.last_score_cache, dtype, f"{ctx} score cache"))
+                for name in META:
+                    assert torch.equal(getattr(cache, name)[li].cpu(), getattr(oc, name)), f"{ctx}: {name}"
+                check_update_against_replay(cache, replay, kc, vc, scores_g, new_g.cpu(), layer=li, ctx=ctx)
+                og_g = cache.og_pos[li].cpu()
+                margins = flip_margins(og_g, oc, pre, seen_before, attn_o.last_score_cache, new_c)
+                ledger.record(margins, eps, og_g.numel(), primary_only=qn < 2 * W, ctx=ctx)
+                x = x + layer.self_attn.o_proj(out_g.transpose(1, 2).reshape(B, qn, -1))
+                x = x + layer.mlp(layer.post_attention_layernorm(x))
+            done += qn
+    print(ledger.summary())
+    assert cache.seen_tokens_by_layer.cpu().tolist() == [done] * cfg.num_layers
+    assert not bool(caches[0].mask.any()) and int(caches[0].start_indices.sum()) > 0, "the cascades must have evicted"
+    assert ledger.flips <= 0.05 * ledger.compared, ledger.summary()
 
 
 def test_generate_streams_past_the_window():

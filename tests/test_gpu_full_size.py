@@ -1,6 +1,10 @@
-"""Size-independent properties at the full benchmark sizes (no oracle: the CPU restatement would take
-minutes here).  Config 2: B=2, 32q/8kv heads, head_dim 128, 64 sinks + 8 x 2048 slots, 2048-token
-chunks; config 3: B=16, 64 sinks + 4 x 8192 slots, one token."""
+"""The benchmark configurations at their real shapes.  The oracle's attention would take minutes here, so
+attention is checked through size-independent properties and sampled rows against float64 dense attention;
+the cache update is cheap enough on the CPU to be compared bit for bit at full size.
+Config 2: B=2, 32q/8kv heads, head_dim 128, 64 sinks + 8 x 2048 slots, 2048-token chunks; config 3: B=16,
+64 sinks + 4 x 8192 slots, one token; config 4 (one layer of it): B=1, 64 sinks + 8 x 8192 slots, 4096-token
+chunks; config 5 (one layer): B=4, 28q/4kv heads, 64 sinks + 16 x 2048 slots, 4096-token chunks (longer than
+a cascade window)."""
 import pytest
 import torch
 
@@ -37,20 +41,27 @@ def restore(cache, snap):
     cache.seen_tokens_by_layer.copy_(seen)
 
 
+CFG2 = dict(B=2, H=32, KVH=8, D=128, NS=64, S=16384, C=8, Q=2048, fill=10, fill_q=2048, theta=5e5)
+CFG4 = dict(B=1, H=32, KVH=8, D=128, NS=64, S=65536, C=8, Q=4096, fill=18, fill_q=4096, theta=5e5)
+CFG5 = dict(B=4, H=28, KVH=4, D=128, NS=64, S=32768, C=16, Q=4096, fill=10, fill_q=4096, theta=1e6)
+
+
 @pytest.mark.parametrize("cfg", [
-    dict(B=2, H=32, KVH=8, D=128, NS=64, S=16384, C=8, Q=2048, fill=10),   # chunked prefill, cache full and evicting
-    dict(B=16, H=32, KVH=8, D=128, NS=64, S=32768, C=4, Q=1, fill=3),      # decode, cache partly filled
-])
+    CFG2,                                                                               # cache full and evicting
+    dict(B=16, H=32, KVH=8, D=128, NS=64, S=32768, C=4, Q=1, fill=3, fill_q=2048, theta=5e5),   # decode, cache partly filled
+    CFG4, CFG5,
+    dict(CFG4, Q=1), dict(CFG5, Q=1),                                                   # single-token steps on the same caches
+], ids=["cfg2", "cfg3-partly-filled", "cfg4", "cfg5", "cfg4-decode", "cfg5-decode"])
 def test_full_size_properties(cfg):
     from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
 
     dtype = torch.bfloat16
     B, H, KVH, D, Q = cfg["B"], cfg["H"], cfg["KVH"], cfg["D"], cfg["Q"]
     cache = make_cache(B, KVH, D, cfg["NS"], cfg["S"], cfg["C"], dtype)
-    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    inv_freq = default_inv_freq(D, cfg["theta"], "cuda:0")
     gen = torch.Generator().manual_seed(7)
-    for _ in range(cfg["fill"]):   # 2048-token chunks through the real path
-        cascade_attention(*chunk(B, H, KVH, 2048, D, gen, dtype), cache, 0, inv_freq)
+    for _ in range(cfg["fill"]):   # chunks through the real path
+        cascade_attention(*chunk(B, H, KVH, cfg["fill_q"], D, gen, dtype), cache, 0, inv_freq)
     q, k, v = chunk(B, H, KVH, Q, D, gen, dtype)
     snap = snapshot(cache)
 
@@ -100,9 +111,10 @@ def _rope64(x, pos, theta=5e5):
 
 
 @pytest.mark.parametrize("cfg", [
-    dict(B=2, H=32, KVH=8, D=128, NS=64, S=16384, C=8, Q=2048, fill=10),
-    dict(B=16, H=32, KVH=8, D=128, NS=64, S=32768, C=4, Q=1, fill=17),     # decode with the cache full
-])
+    CFG2,
+    dict(B=16, H=32, KVH=8, D=128, NS=64, S=32768, C=4, Q=1, fill=17, fill_q=2048, theta=5e5),   # decode with the cache full
+    CFG4, CFG5, dict(CFG4, Q=1), dict(CFG5, Q=1),
+], ids=["cfg2", "cfg3", "cfg4", "cfg5", "cfg4-decode", "cfg5-decode"])
 def test_full_size_sampled_rows_against_dense_attention(cfg):
     """At the benchmark sizes the whole oracle takes minutes, a few rows of it do not: for sampled
     (batch, head, query) rows, softmax(q K^T / sqrt(D)) V over exactly the visible keys in float64, with
@@ -113,10 +125,11 @@ def test_full_size_sampled_rows_against_dense_attention(cfg):
     B, H, KVH, D, Q, NS = cfg["B"], cfg["H"], cfg["KVH"], cfg["D"], cfg["Q"], cfg["NS"]
     G = H // KVH
     cache = make_cache(B, KVH, D, NS, cfg["S"], cfg["C"], dtype)
-    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    theta = cfg["theta"]
+    inv_freq = default_inv_freq(D, theta, "cuda:0")
     gen = torch.Generator().manual_seed(9)
     for _ in range(cfg["fill"]):
-        cascade_attention(*chunk(B, H, KVH, 2048, D, gen, dtype), cache, 0, inv_freq)
+        cascade_attention(*chunk(B, H, KVH, cfg["fill_q"], D, gen, dtype), cache, 0, inv_freq)
     q, k, v = chunk(B, H, KVH, Q, D, gen, dtype)
     # what the call will see: the state before it
     vals = [t.clone() for t in cache.get_vals(0)]
@@ -127,17 +140,72 @@ def test_full_size_sampled_rows_against_dense_attention(cfg):
     sv, cvalid = (~sink_mask[0, 0]).cpu(), (~key_mask[0, 0]).cpu()
     assert int(cvalid.sum()) == cfg["S"], "the cache should be full at this point"
     sink_pos, key_pos = sink_pos[0].cpu(), key_pos[0].cpu()
-    rows = [(0, 0, 0), (B - 1, H - 1, Q - 1), (B // 2, 5, Q // 2), (0, 17, min(Q - 1, 63)), (B - 1, 30, min(Q - 1, 64)),
+    rows = [(0, 0, 0), (B - 1, H - 1, Q - 1), (B // 2, 5, Q // 2), (0, 17, min(Q - 1, 63)), (B - 1, 30 % H, min(Q - 1, 64)),
             (0, 9, max(0, Q - 700))]
     worst = 0.0
     for b, h, m in rows:
         kvh = h // G
-        keys = torch.cat((_rope64(sink_k[b, kvh].cpu()[sv], sink_pos[sv]),
-                          _rope64(ck[b, kvh].cpu()[cvalid], key_pos[cvalid]),
-                          _rope64(k[b, kvh, : m + 1].cpu(), q_pos[: m + 1])), dim=0)
+        keys = torch.cat((_rope64(sink_k[b, kvh].cpu()[sv], sink_pos[sv], theta),
+                          _rope64(ck[b, kvh].cpu()[cvalid], key_pos[cvalid], theta),
+                          _rope64(k[b, kvh, : m + 1].cpu(), q_pos[: m + 1], theta)), dim=0)
         valv = torch.cat((sink_v[b, kvh].cpu()[sv], cv[b, kvh].cpu()[cvalid], v[b, kvh, : m + 1].cpu()), dim=0).double()
-        qr = _rope64(q[b, h, m].cpu(), q_pos[m])
+        qr = _rope64(q[b, h, m].cpu(), q_pos[m], theta)
         p = torch.softmax(keys @ qr / (D ** 0.5), dim=0)
         want = p @ valv
         worst = max(worst, (out[b, h, m].double().cpu() - want).abs().max().item())
     assert worst <= 2e-2, f"sampled rows differ from dense attention by {worst:.3e}"
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(B=1, KVH=8, D=128, NS=64, W=8192, C=8, q=4096, calls=20),      # config 4: 81920 tokens through 65536 slots
+    dict(B=4, KVH=4, D=128, NS=64, W=2048, C=16, q=4096, calls=12),     # config 5: calls longer than a cascade window
+], ids=["cfg4", "cfg5"])
+def test_update_bit_exact_at_benchmark_shapes(cfg):
+    """ckv_update against the serial oracle at the cache shapes of configs 4 and 5, for enough calls that every
+    cascade is full and evicting: every state tensor bit-identical after every call (tie-heavy scores)."""
+    from test_gpu_update import make_pair, run_stream
+
+    dtype = torch.bfloat16
+    gpu, cpu = make_pair(cfg["B"], cfg["KVH"], cfg["D"], cfg["NS"], cfg["W"], cfg["C"], dtype)
+    gen = torch.Generator().manual_seed(41)
+    run_stream(gpu, cpu, cfg["q"] * cfg["calls"], lambda: cfg["q"], gen, dtype, "ties", transposed=True)
+    assert not bool(cpu.mask.any()) and int(cpu.start_indices[..., -1].sum()) > 0, "the last cascade must have evicted"
+
+
+def test_config3_consecutive_decode_steps_update_bit_exact():
+    """Config 3 at full size: B=16, 8 kv heads, 64 sinks + 4 x 8192 slots, cache full.  Eight single-token steps in a
+    row through the real path (attention, score EMA, update); after every step the whole cache state must equal
+    the oracle's update run on the same scores, bit for bit."""
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
+    from parity_helpers import STATE, bits, push_state
+    from test_gpu_update import make_pair
+
+    dtype = torch.bfloat16
+    B, H, KVH, D, NS, W, C = 16, 32, 8, 128, 64, 8192, 4
+    gpu, cpu = make_pair(B, KVH, D, NS, W, C, dtype)
+    gen = torch.Generator().manual_seed(43)
+    for _ in range(5):  # 40960 tokens through the oracle alone: cache full, every cascade evicting
+        n = 8192
+        k = torch.randn(B, KVH, n, D, generator=gen).to(dtype)
+        v = torch.randn(B, KVH, n, D, generator=gen).to(dtype)
+        cpu.update(k, v, (torch.rand(B, KVH, n, generator=gen) * 1e-6).to(dtype))
+    del k, v
+    push_state(gpu, cpu)
+    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    for step in range(8):
+        q = torch.randn(B, H, 1, D, generator=gen).to(dtype)
+        k = torch.randn(B, KVH, 1, D, generator=gen).to(dtype)
+        v = torch.randn(B, KVH, 1, D, generator=gen).to(dtype)
+        out, new_g = cascade_attention(q.cuda(), k.cuda(), v.cuda(), gpu, 0, inv_freq, update_cache=False)
+        assert torch.isfinite(out.float()).all()
+        cpu.score_cache.copy_(gpu.score_cache[0])          # the update's score inputs are the library's own
+        gpu.update(k.cuda(), v.cuda(), 0, score_states=new_g)
+        cpu.update(k, v, new_g.cpu())
+        torch.cuda.synchronize()
+        heavy = step in (0, 3, 7)                          # the 1 GiB K and V caches are pulled back on these steps
+        for name in STATE:
+            if name in ("key_cache", "value_cache") and not heavy:
+                continue
+            g, w = bits(getattr(gpu, name)[0].cpu()), bits(getattr(cpu, name))
+            assert torch.equal(g, w), f"step {step}: {name} differs from the oracle"
+        assert int(gpu.seen_tokens_by_layer[0]) == int(cpu.seen_tokens)
