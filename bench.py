@@ -1,21 +1,27 @@
 #!/usr/bin/env python3
 """Throughput of the cascade attention hot path on one MI355X.
 
-A "step" is one pass of the path over one batch of synthetic input: the attention of one
-2048-token chunk per stream over [64 sinks | 8 cascades x 2048 slots | chunk] plus the cascading
-cache update, on a Llama-3.1-8B-shaped attention layer (32 query / 8 kv heads, head_dim 128,
-bf16, 2 streams) whose cache is already full (steady state of the 65536-token stream).
+Headline workload = one attention layer of the Llama-3.1-8B shape (32 query / 8 kv heads, head_dim 128, bf16,
+one stream) over a 64 sinks + 65536-slot cache split into 8 cascades (8 x 8192), the cache already full (steady
+state of a long stream).  A "step" is one pass of the path in the proportions of the 131072-token prompt + 256
+greedy tokens the workload is quoted on: the attention + score EMA + cache update of one 4096-token prefill
+chunk, followed by 8 single-token decode steps on the same cache.  `value` = tokens (prefill + decode) per
+second with every input resident in HBM.
 
-Prints ONE JSON line.  `value` = tokens/s of chunked prefill with inputs resident in HBM;
-`roofline` prices the dominant kernel (the flash forward) against the dense bf16 MFMA peak from
-HIP-event timings taken inside the timed region; `decode` reports the single-token path
-(16 streams, 4 cascades x 8192 slots) against HBM bandwidth; `cpu_baseline` times the CPU oracle
-(the reference's eager PyTorch path restated, plus the serial update) on a bounded sample.
+Prints ONE JSON line.  `roofline` prices the dominant kernel (the flash forward of the prefill chunk) against
+the dense bf16 MFMA peak from HIP-event timings of that kernel's own dispatch inside the timed region.  Named
+sub-records carry their own roofline: `decode` (the single-token steps of the headline workload against HBM
+bandwidth), `update` (the cache update of the headline chunk against HBM bandwidth, bytes counted from the
+state difference), `cfg2_prefill` (B=2, 8 x 2048 slots, 2048-token chunks) and `cfg3_decode` (B=16,
+4 x 8192 slots, one token).  `cpu_baseline` times the CPU oracle (the reference's eager PyTorch path restated,
+plus the serial update) on a bounded sample of the headline workload on the box's host cores.
 """
 import argparse
+import hashlib
 import json
 import math
 import os
+import re
 import sys
 import time
 
@@ -27,13 +33,39 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
-# HBM bytes per launch of the dominant kernels on the bench workloads, measured with rocprofv3 --pmc
-# FETCH_SIZE and WRITE_SIZE (one pass each), each scaled by the reading for a 512 MiB device copy in the
-# same run (profiles/hbm_traffic_bench_kernels.md).  Counters cannot be read inside this process.
-TRAFFIC_BYTES = {"fwd_pipe_kernel": 0.220e9, "decode_stream_kernel": 2.256e9}
 
-PREFILL = dict(B=2, H=32, KVH=8, D=128, NS=64, S=16384, C=8, Q=2048, theta=5e5, seed=2)
-DECODE = dict(B=16, H=32, KVH=8, D=128, NS=64, S=32768, C=4, Q=1, theta=5e5, seed=3)
+LAYER = dict(name="llama3.1-8b layer, 64K window", B=1, H=32, KVH=8, D=128, NS=64, S=65536, C=8, Q=4096, theta=5e5,
+             seed=4, decode_per_chunk=8)
+CFG2 = dict(name="cfg2", B=2, H=32, KVH=8, D=128, NS=64, S=16384, C=8, Q=2048, theta=5e5, seed=2)
+CFG3 = dict(name="cfg3", B=16, H=32, KVH=8, D=128, NS=64, S=32768, C=4, Q=1, theta=5e5, seed=3)
+
+STATE = ("key_cache", "value_cache", "score_cache", "sink_keys", "sink_values", "mask", "sink_mask", "pos", "og_pos",
+         "sink_pos", "stored_tokens", "start_indices", "stored_sinks")
+
+
+def measured_traffic(kernel, workload):
+    """HBM bytes per launch of `kernel` on `workload` from the committed counter summary
+    (profiles/hbm_traffic_bench_kernels.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy of known
+    size).  Counters cannot be read inside this process, so the summary is the only source; it records the
+    hash of the kernel's source file, and a figure taken from another version of that file is not reported."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic_bench_kernels.md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    for line in text.splitlines():
+        m = re.match(r"\|\s*`(\w+)`\s*\|\s*([\w.-]+)\s*\|\s*([\w./]+)\s*\|\s*([0-9a-f]{16})\s*\|\s*([0-9.]+)\s*\|\s*([0-9.]+)\s*\|", line)
+        if not m or m.group(1) != kernel or m.group(2) != workload:
+            continue
+        src = os.path.join(ROOT, "cascading_kv_cache_amd", "csrc", m.group(3))
+        try:
+            digest = hashlib.sha256(open(src, "rb").read()).hexdigest()[:16]
+        except OSError:
+            return None
+        if digest != m.group(4):
+            return None  # the kernel's source changed since the counters were read
+        return (float(m.group(5)) + float(m.group(6))) * 1e9
+    return None
 
 
 def make_cache(cfg, dtype, device):
@@ -44,9 +76,9 @@ def make_cache(cfg, dtype, device):
                             cascade_func="pow2", head_reduction="mean", layers=1, eager_fill=True, verbose=False)
 
 
-def chunk_pool(cfg, n, dtype, device, q_len=None, scale=1.0):
+def chunk_pool(cfg, n, dtype, device, q_len=None, scale=1.0, seed_offset=0):
     """Seeded synthetic chunks, generated on the CPU so every run sees the same bits."""
-    g = torch.Generator().manual_seed(cfg["seed"])
+    g = torch.Generator().manual_seed(cfg["seed"] + seed_offset)
     B, H, KVH, D = cfg["B"], cfg["H"], cfg["KVH"], cfg["D"]
     Q = q_len or cfg["Q"]
     pool = []
@@ -64,75 +96,227 @@ def fill_to_steady_state(cache, cfg, pool, inv_freq):
     need = cfg["S"] + cfg["NS"]
     done = 0
     i = 0
-    while done <= need + cfg["Q"]:
+    while done <= need + pool[0][0].size(2):
         q, k, v = pool[i % len(pool)]
         cascade_attention(q, k, v, cache, 0, inv_freq)
         done += q.size(2)
         i += 1
     torch.cuda.synchronize()
+    assert int(cache.mask[0].sum()) == 0, "cache must be full before the timed region"
 
 
-def run_prefill(steps, warmup, dtype, device):
+def prefill_flops(cfg):
+    """Algorithmic flops of one forward launch: QK^T and PV over the visible keys only (masked slots and the
+    causal upper triangle excluded), 2 flop per multiply-add."""
+    n_cached = cfg["NS"] + cfg["S"]
+    return 4.0 * cfg["B"] * cfg["H"] * cfg["D"] * cfg["Q"] * (n_cached + (cfg["Q"] + 1) / 2.0)
+
+
+def decode_bytes(cfg, es=2):
+    """Algorithmic bytes of one single-token step: K and V of every visible key once, the score cache read and
+    written once, q and out."""
+    n_valid = cfg["NS"] + cfg["S"]
+    return (2.0 * cfg["B"] * cfg["KVH"] * n_valid * cfg["D"] * es + 2.0 * cfg["B"] * cfg["KVH"] * cfg["S"] * es +
+            2.0 * cfg["B"] * cfg["H"] * cfg["D"] * es)
+
+
+def update_bytes(cache, cfg, k, v, new_scores, es=2):
+    """Algorithmic bytes of one cache update, counted from the state difference (untimed): per (b, kv head) the
+    incoming rows read once, every old row that ends in a different slot read once, every slot whose content
+    differs afterwards written once (row = K, V, score, original index), plus the position ids of every slot."""
+    B, KVH, D, S = cfg["B"], cfg["KVH"], cfg["D"], cfg["S"]
+    q_len = k.size(2)
+    before = cache.og_pos[0].clone()
+    before_valid = ~cache.mask[0].clone()
+    snap = {n: getattr(cache, n)[0].clone() for n in STATE}
+    seen_host, seen_dev = cache._seen_host[0], cache.seen_tokens_by_layer.clone()
+    cache.update_state(k, v, 0, new_scores)
+    torch.cuda.synchronize()
+    after = cache.og_pos[0]
+    after_valid = ~cache.mask[0]
+    changed = ((after != before) | (after_valid != before_valid)) & after_valid
+    n_changed = int(changed.sum())
+    n_reloc = 0
+    for b in range(B):
+        for h in range(KVH):
+            moved = after[b, h][changed[b, h]]
+            n_reloc += int(torch.isin(moved, before[b, h][before_valid[b, h]]).sum())
+    for n, t in snap.items():  # leave the cache as it was
+        getattr(cache, n)[0].copy_(t)
+    cache._seen_host[0] = seen_host
+    cache.seen_tokens_by_layer.copy_(seen_dev)
+    row = 2 * D * es + es + 8
+    total = B * KVH * q_len * (2 * D * es + es) + (n_reloc + n_changed) * row + B * KVH * S * 8
+    return float(total), dict(rows_in=B * KVH * q_len, rows_relocated=n_reloc, slots_rewritten=n_changed)
+
+
+def stage_table(stages):
+    return {k: (ms / n if n else 0.0) for k, (ms, n) in stages.items()}
+
+
+def run_layer(steps, warmup, dtype, device):
+    """The headline: per step one 4096-token chunk and 8 single-token steps on the 64K-window cache."""
     from cascading_kv_cache_amd import _abi
     from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
 
-    cfg = PREFILL
+    cfg = LAYER
     cache = make_cache(cfg, dtype, device)
     inv_freq = default_inv_freq(cfg["D"], cfg["theta"], device)
-    pool = chunk_pool(cfg, 4, dtype, device, scale=1.0 / math.sqrt(cfg["D"]))
+    pool = chunk_pool(cfg, 3, dtype, device, scale=1.0 / math.sqrt(cfg["D"]))
+    dpool = chunk_pool(cfg, 8, dtype, device, q_len=1, seed_offset=100)
     fill_to_steady_state(cache, cfg, pool, inv_freq)
-    assert int(cache.mask[0].sum()) == 0, "cache must be full before the timed region"
-    for i in range(warmup):
+    n_dec = cfg["decode_per_chunk"]
+
+    def step(i):
         q, k, v = pool[i % len(pool)]
         cascade_attention(q, k, v, cache, 0, inv_freq)
+        for j in range(n_dec):
+            q1, k1, v1 = dpool[(i * n_dec + j) % len(dpool)]
+            cascade_attention(q1, k1, v1, cache, 0, inv_freq)
+
+    for i in range(warmup):
+        step(i)
     torch.cuda.synchronize()
-    # timed region: only the dominant kernel is bracketed by HIP events (two records per step); an event
-    # record between every pair of kernels would open a ~10 us gap each
+    # timed region: only the two dominant kernels carry HIP events, attached to their own dispatch (an event
+    # record in the stream between every pair of kernels would open a ~10 us gap each)
     _abi.profile_enable(2)
     _abi.profile_read()
     t0 = time.perf_counter()
     for i in range(steps):
-        q, k, v = pool[i % len(pool)]
-        cascade_attention(q, k, v, cache, 0, inv_freq)
+        step(i)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    main_stage = _abi.profile_read()
-    # untimed pass with every stage bracketed, for the per-stage table
-    _abi.profile_enable(1)
-    for i in range(min(steps, 10)):
-        q, k, v = pool[i % len(pool)]
-        cascade_attention(q, k, v, cache, 0, inv_freq)
-    torch.cuda.synchronize()
-    stages = _abi.profile_read()
+    timed = stage_table(_abi.profile_read())
     _abi.profile_enable(0)
 
-    B, H, D, Q = cfg["B"], cfg["H"], cfg["D"], cfg["Q"]
+    # untimed: the two phases apart (wall clock), then with every stage bracketed for the per-stage tables
+    def phase(fn, reps):
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for i in range(reps):
+            fn(i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / reps
+
+    def one_chunk(i):
+        q, k, v = pool[i % len(pool)]
+        cascade_attention(q, k, v, cache, 0, inv_freq)
+
+    def one_token(i):
+        q1, k1, v1 = dpool[i % len(dpool)]
+        cascade_attention(q1, k1, v1, cache, 0, inv_freq)
+
+    chunk_s = phase(one_chunk, max(3, min(steps, 10)))
+    token_s = phase(one_token, 64)
+    _abi.profile_enable(1)
+    _abi.profile_read()
+    for i in range(max(3, min(steps, 10))):
+        one_chunk(i)
+    torch.cuda.synchronize()
+    pre_stages = stage_table(_abi.profile_read())
+    for i in range(32):
+        one_token(i)
+    torch.cuda.synchronize()
+    dec_stages = stage_table(_abi.profile_read())
+    _abi.profile_enable(0)
+
+    B, Q = cfg["B"], cfg["Q"]
+    flops = prefill_flops(cfg)
+    fwd_ms = timed["fwd"]
+    achieved = flops / (fwd_ms * 1e-3) / 1e12 if fwd_ms else 0.0
+    attn_ms = pre_stages["prep"] + pre_stages["fwd"] + pre_stages["scores"] + pre_stages["finish"]
     n_cached = cfg["NS"] + cfg["S"]
-    # algorithmic flops of one forward launch: QK^T and PV over the visible keys only
-    flops_fwd = 4.0 * B * H * D * Q * (n_cached + (Q + 1) / 2.0)
-    fwd_ms, fwd_n = main_stage["fwd"]  # from the timed region
-    fwd_avg_ms = fwd_ms / max(fwd_n, 1)
-    achieved = flops_fwd / (fwd_avg_ms * 1e-3) / 1e12
-    stage_ms = {k: (ms / n if n else 0.0) for k, (ms, n) in stages.items()}
-    attn_ms = stage_ms["prep"] + stage_ms["fwd"] + stage_ms["scores"] + stage_ms["finish"]
+    dec_ms = timed["decode"]
+    dbytes = decode_bytes(cfg)
+    dec_achieved = dbytes / (dec_ms * 1e-3) / 1e9 if dec_ms else 0.0
+    # cache update of the headline chunk: bytes from the state difference, time from the stage timers
+    q, k, v = pool[0]
+    new_scores = torch.rand(B, cfg["KVH"], Q, device=device).mul_(1e-6).to(dtype)
+    ubytes, ucount = update_bytes(cache, cfg, k, v, new_scores)
+    upd_ms = pre_stages["plan"] + pre_stages["apply"]
     res = dict(
         ms_per_step=dt / steps * 1e3,
-        tokens_per_s=B * Q * steps / dt,
+        tokens_per_s=B * (Q + n_dec) * steps / dt,
         roofline=dict(bound="mfma", achieved=achieved, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
-                      frac=achieved / PEAK_BF16_TFLOPS, traffic=TRAFFIC_BYTES["fwd_pipe_kernel"], kernel="fwd_pipe_kernel",
-                      kernel_ms=fwd_avg_ms, algorithmic_tflop_per_launch=flops_fwd / 1e12),
-        stage_ms=stage_ms,
-        attention_tflops_all_stages=(flops_fwd + 2.0 * B * H * Q * (n_cached + Q)) / (attn_ms * 1e-3) / 1e12
-        if attn_ms else None,
+                      frac=achieved / PEAK_BF16_TFLOPS,
+                      traffic=measured_traffic("fwd_pipe_kernel", "layer64k"), kernel="fwd_pipe_kernel",
+                      kernel_ms=fwd_ms, algorithmic_tflop_per_launch=flops / 1e12),
+        prefill=dict(tokens_per_s=B * Q / chunk_s, ms_per_chunk=chunk_s * 1e3, stage_ms=pre_stages,
+                     attention_tflops_all_stages=(flops + 2.0 * B * cfg["H"] * Q * (n_cached + Q)) / (attn_ms * 1e-3) / 1e12
+                     if attn_ms else None),
+        decode=dict(workload="single-token steps on the headline cache (B=1, 64 sinks + 8 x 8192 slots, full)",
+                    tokens_per_s=B / token_s, ms_per_step=token_s * 1e3, stage_ms=dec_stages,
+                    roofline=dict(bound="hbm", achieved=dec_achieved, peak=PEAK_HBM_GBPS, unit="GB/s",
+                                  frac=dec_achieved / PEAK_HBM_GBPS,
+                                  traffic=measured_traffic("decode_stream_kernel", "layer64k"),
+                                  kernel="decode_stream_kernel", kernel_ms=dec_ms,
+                                  algorithmic_gb_per_launch=dbytes / 1e9),
+                    whole_step_gbps=dbytes / token_s / 1e9),
+        update=dict(workload="cache update of one 4096-token chunk into the full headline cache",
+                    roofline=dict(bound="hbm", achieved=ubytes / (upd_ms * 1e-3) / 1e9 if upd_ms else 0.0,
+                                  peak=PEAK_HBM_GBPS, unit="GB/s",
+                                  frac=ubytes / (upd_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS if upd_ms else 0.0, traffic=None,
+                                  kernel="ckv_update_plan_kernel + ckv_update_apply_vec_kernel", kernel_ms=upd_ms,
+                                  algorithmic_gb_per_launch=ubytes / 1e9), **ucount),
     )
     return res, cache, pool
 
 
-def run_decode(steps, warmup, dtype, device):
+def run_cfg2(steps, warmup, dtype, device):
     from cascading_kv_cache_amd import _abi
     from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
 
-    cfg = DECODE
+    cfg = CFG2
+    cache = make_cache(cfg, dtype, device)
+    inv_freq = default_inv_freq(cfg["D"], cfg["theta"], device)
+    pool = chunk_pool(cfg, 4, dtype, device, scale=1.0 / math.sqrt(cfg["D"]))
+    fill_to_steady_state(cache, cfg, pool, inv_freq)
+    for i in range(warmup):
+        cascade_attention(*pool[i % len(pool)], cache, 0, inv_freq)
+    torch.cuda.synchronize()
+    _abi.profile_enable(2)
+    _abi.profile_read()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        cascade_attention(*pool[i % len(pool)], cache, 0, inv_freq)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    timed = stage_table(_abi.profile_read())
+    _abi.profile_enable(1)
+    for i in range(min(steps, 10)):
+        cascade_attention(*pool[i % len(pool)], cache, 0, inv_freq)
+    torch.cuda.synchronize()
+    stages = stage_table(_abi.profile_read())
+    _abi.profile_enable(0)
+    B, H, Q = cfg["B"], cfg["H"], cfg["Q"]
+    flops = prefill_flops(cfg)
+    fwd_ms = timed["fwd"]
+    achieved = flops / (fwd_ms * 1e-3) / 1e12 if fwd_ms else 0.0
+    attn_ms = stages["prep"] + stages["fwd"] + stages["scores"] + stages["finish"]
+    q, k, v = pool[0]
+    new_scores = torch.rand(B, cfg["KVH"], Q, device=device).mul_(1e-6).to(dtype)
+    ubytes, ucount = update_bytes(cache, cfg, k, v, new_scores)
+    upd_ms = stages["plan"] + stages["apply"]
+    return dict(
+        workload="chunked prefill: B=2, 32q/8kv heads, head_dim 128, sink 64 + 8 cascades x 2048 slots (full), 2048-token chunks",
+        ms_per_step=dt / steps * 1e3, tokens_per_s=B * Q * steps / dt,
+        roofline=dict(bound="mfma", achieved=achieved, peak=PEAK_BF16_TFLOPS, unit="TFLOP/s",
+                      frac=achieved / PEAK_BF16_TFLOPS, traffic=measured_traffic("fwd_pipe_kernel", "cfg2"),
+                      kernel="fwd_pipe_kernel", kernel_ms=fwd_ms, algorithmic_tflop_per_launch=flops / 1e12),
+        stage_ms=stages,
+        attention_tflops_all_stages=(flops + 2.0 * B * H * Q * (cfg["NS"] + cfg["S"] + Q)) / (attn_ms * 1e-3) / 1e12
+        if attn_ms else None,
+        update_roofline=dict(bound="hbm", achieved=ubytes / (upd_ms * 1e-3) / 1e9 if upd_ms else 0.0, peak=PEAK_HBM_GBPS,
+                             unit="GB/s", frac=ubytes / (upd_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS if upd_ms else 0.0,
+                             traffic=None, kernel_ms=upd_ms, algorithmic_gb_per_launch=ubytes / 1e9, **ucount),
+    )
+
+
+def run_cfg3(steps, warmup, dtype, device):
+    from cascading_kv_cache_amd import _abi
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
+
+    cfg = CFG3
     cache = make_cache(cfg, dtype, device)
     inv_freq = default_inv_freq(cfg["D"], cfg["theta"], device)
     # pre-filled full: K, V ~ N(0, 1), trackers as after S + NS tokens
@@ -158,61 +342,79 @@ def run_decode(steps, warmup, dtype, device):
     cache._seen_host[0] = seen
     pool = chunk_pool(cfg, 8, dtype, device)
     for i in range(warmup):
-        q, k, v = pool[i % len(pool)]
-        cascade_attention(q, k, v, cache, 0, inv_freq)
+        cascade_attention(*pool[i % len(pool)], cache, 0, inv_freq)
     torch.cuda.synchronize()
-    # timed region: only the dominant kernel is bracketed by HIP events (two records per step); an event
-    # record between every pair of kernels would open a ~10 us gap each
     _abi.profile_enable(2)
     _abi.profile_read()
     t0 = time.perf_counter()
     for i in range(steps):
-        q, k, v = pool[i % len(pool)]
-        cascade_attention(q, k, v, cache, 0, inv_freq)
+        cascade_attention(*pool[i % len(pool)], cache, 0, inv_freq)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    main_stage = _abi.profile_read()
-    # untimed pass with every stage bracketed, for the per-stage table
+    timed = stage_table(_abi.profile_read())
     _abi.profile_enable(1)
     for i in range(min(steps, 10)):
-        q, k, v = pool[i % len(pool)]
-        cascade_attention(q, k, v, cache, 0, inv_freq)
+        cascade_attention(*pool[i % len(pool)], cache, 0, inv_freq)
     torch.cuda.synchronize()
-    stages = _abi.profile_read()
+    stages = stage_table(_abi.profile_read())
     _abi.profile_enable(0)
-    B, H, KVH, D = cfg["B"], cfg["H"], cfg["KVH"], cfg["D"]
-    n_valid = cfg["NS"] + cfg["S"]
-    es = 2
-    # K and V of every visible key once, the score cache read and written once, q and out
-    algo_bytes = 2.0 * B * KVH * n_valid * D * es + 2.0 * B * KVH * cfg["S"] * es + 2.0 * B * H * D * es
-    stage_ms = {k: (ms / n if n else 0.0) for k, (ms, n) in stages.items()}
-    timed = {k: (ms / n if n else 0.0) for k, (ms, n) in main_stage.items()}  # from the timed region
+    B = cfg["B"]
+    algo = decode_bytes(cfg)
     main_ms = timed["decode"] if timed["decode"] > 0 else timed["fwd"]
-    achieved = algo_bytes / (main_ms * 1e-3) / 1e9 if main_ms else 0.0
+    achieved = algo / (main_ms * 1e-3) / 1e9 if main_ms else 0.0
+    q, k, v = pool[0]
+    new_scores = torch.rand(B, cfg["KVH"], 1, device=device).mul_(1e-6).to(dtype)
+    ubytes, ucount = update_bytes(cache, cfg, k, v, new_scores)
+    upd_ms = stages["plan"] + stages["apply"]
     return dict(
         workload="decode: B=16, 32q/8kv heads, head_dim 128, sink 64 + 4 cascades x 8192 slots (full), q=1",
-        ms_per_step=dt / steps * 1e3,
-        tokens_per_s=B * steps / dt,
+        ms_per_step=dt / steps * 1e3, tokens_per_s=B * steps / dt,
         roofline=dict(bound="hbm", achieved=achieved, peak=PEAK_HBM_GBPS, unit="GB/s", frac=achieved / PEAK_HBM_GBPS,
-                      traffic=TRAFFIC_BYTES["decode_stream_kernel"], kernel="decode_stream_kernel", kernel_ms=main_ms,
-                      algorithmic_gb_per_launch=algo_bytes / 1e9),
-        stage_ms=stage_ms,
+                      traffic=measured_traffic("decode_stream_kernel", "cfg3"), kernel="decode_stream_kernel",
+                      kernel_ms=main_ms, algorithmic_gb_per_launch=algo / 1e9),
+        stage_ms=stages,
+        update_roofline=dict(bound="hbm", achieved=ubytes / (upd_ms * 1e-3) / 1e9 if upd_ms else 0.0, peak=PEAK_HBM_GBPS,
+                             unit="GB/s", frac=ubytes / (upd_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS if upd_ms else 0.0,
+                             traffic=None, kernel_ms=upd_ms, algorithmic_gb_per_launch=ubytes / 1e9, **ucount),
     )
 
 
+def host_threads():
+    """Threads for the CPU leg: every core this process may use.  os.cpu_count() reports the whole host; the
+    scheduler affinity and the OMP_NUM_THREADS the box exports say what this job's share is."""
+    n = os.cpu_count() or 1
+    try:
+        n = min(n, len(os.sched_getaffinity(0)))
+    except (AttributeError, OSError):
+        pass
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit() and int(env) > 0:
+        n = min(n, int(env))
+    return n
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def run_cpu_baseline(cache, pool, dtype):
-    """The oracle on the host: the reference's eager path restated, on a bounded sample of the
-    prefill workload (same cache contents, a 64-token chunk instead of 2048)."""
+    """The oracle on the host: the reference's eager path restated, on a bounded sample of the headline
+    workload (the same full cache contents, a 64-token chunk instead of 4096)."""
     from oracle.attention import OracleCascadeAttention
     from oracle.update import OracleCache
 
-    cfg = PREFILL
-    threads = min(os.cpu_count() or 1, 16)
+    cfg = LAYER
+    threads = host_threads()
     torch.set_num_threads(threads)
     o = OracleCache(window_length=cfg["S"] // cfg["C"], num_sink_tokens=cfg["NS"], max_batch_size=cfg["B"],
                     heads=cfg["KVH"], dim=cfg["D"], max_seq_len=cfg["S"], dtype=dtype)
-    for name in ("key_cache", "value_cache", "score_cache", "sink_keys", "sink_values", "mask", "sink_mask", "pos",
-                 "og_pos", "sink_pos", "stored_tokens", "start_indices", "stored_sinks"):
+    for name in STATE:
         getattr(o, name).copy_(getattr(cache, name)[0].cpu())
     o.seen_tokens.fill_(int(cache._seen_host[0]))
     layer = OracleCascadeAttention(cfg["H"], cfg["KVH"], cfg["D"], rope_theta=cfg["theta"])
@@ -222,15 +424,38 @@ def run_cpu_baseline(cache, pool, dtype):
     layer.forward(q, k, v, o)  # untimed: first-touch of the cache copy and thread start-up
     t0 = time.perf_counter()
     reps = 0
-    while True:  # a bounded sample: about ten seconds of CPU work
+    while True:  # a bounded sample: about fifteen seconds of CPU work
         layer.forward(q, k, v, o)
         reps += 1
-        if time.perf_counter() - t0 > 10.0 or reps >= 256:
+        if time.perf_counter() - t0 > 15.0 or reps >= 256:
             break
     dt = time.perf_counter() - t0
     return dict(value=cfg["B"] * q_s * reps / dt, unit="tokens/s", cores=threads, kind="port",
-                sample=f"{reps} x (2 streams x {q_s}-token chunk over the full 64+16384-slot cache), i.e. 1/32 of one "
-                       f"step's tokens per repetition; eager attention + score EMA + serial update in bf16")
+                host_cores_reported=os.cpu_count(), cpu=cpu_model(),
+                sample=f"{reps} x (one {q_s}-token chunk over the full 64+65536-slot cache), i.e. 1/64 of one prefill "
+                       f"chunk's tokens per repetition; eager attention + score EMA + serial update in bf16 on "
+                       f"{threads} threads")
+
+
+def run_cpu_config1():
+    """Config 1 in full on the host (the float32 CPU case the oracle exists for): B=1, 32q/8kv heads, head_dim
+    128, sink 4, window 512 in 4 cascades, 4096 tokens in chunks of 256."""
+    from oracle.attention import OracleCascadeAttention
+    from oracle.update import OracleCache
+
+    torch.set_num_threads(host_threads())
+    o = OracleCache(window_length=128, num_sink_tokens=4, max_batch_size=1, heads=8, dim=128, max_seq_len=512,
+                    dtype=torch.float32)
+    layer = OracleCascadeAttention(32, 8, 128, rope_theta=5e5)
+    g = torch.Generator().manual_seed(1)
+    chunks = [(torch.randn(1, 32, 256, 128, generator=g), torch.randn(1, 8, 256, 128, generator=g),
+               torch.randn(1, 8, 256, 128, generator=g)) for _ in range(16)]
+    t0 = time.perf_counter()
+    for q, k, v in chunks:
+        layer.forward(q, k, v, o)
+    dt = time.perf_counter() - t0
+    return dict(value=4096 / dt, unit="tokens/s", seconds=dt, cores=host_threads(), kind="port",
+                sample="config 1 in full: 4096 tokens in 16 chunks of 256, float32")
 
 
 def main():
@@ -239,7 +464,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-decode", action="store_true", help="skip the decode leg")
+    ap.add_argument("--no-sub", action="store_true", help="skip the cfg2 / cfg3 sub-records")
+    ap.add_argument("--only", choices=["layer", "cfg2", "cfg3"], default=None,
+                    help="run one workload only (for profiler runs); the JSON line then carries that record alone")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 512 MiB device copy, the known-size reference that scales the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
@@ -253,38 +480,57 @@ def main():
         sys.exit(1)
     device = torch.device("cuda:0")
     dtype = torch.bfloat16
-    pre, cache, pool = run_prefill(args.steps, args.warmup, dtype, device)
+
+    def calibrate():
+        if args.calibrate_copy:
+            src = torch.ones(512 << 20, dtype=torch.uint8, device=device)
+            dst = torch.empty_like(src)
+            torch.cuda.synchronize()
+            dst.copy_(src)
+            torch.cuda.synchronize()
+
+    if args.only in ("cfg2", "cfg3"):
+        rec = (run_cfg2 if args.only == "cfg2" else run_cfg3)(max(args.steps, 3), args.warmup, dtype, device)
+        calibrate()
+        print(json.dumps({args.only: rec}))
+        return
+    layer, cache, pool = run_layer(args.steps, args.warmup, dtype, device)
     cpu = None if args.no_cpu else run_cpu_baseline(cache, pool, dtype)
+    cpu1 = None if args.no_cpu else run_cpu_config1()
     del cache, pool
     torch.cuda.empty_cache()
-    dec = None if args.no_decode else run_decode(max(args.steps, 20), args.warmup, dtype, device)
-    if args.calibrate_copy:
-        src = torch.ones(512 << 20, dtype=torch.uint8, device=device)
-        dst = torch.empty_like(src)
-        torch.cuda.synchronize()
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+    sub = args.no_sub or args.only == "layer"
+    cfg2 = None if sub else run_cfg2(max(args.steps, 20), args.warmup, dtype, device)
+    torch.cuda.empty_cache()
+    cfg3 = None if sub else run_cfg3(max(args.steps, 20), args.warmup, dtype, device)
+    calibrate()
+    cfg = LAYER
     line = {
         "metric": "prefill+decode tokens/s (8B-shape, C=8, 64K window); MFMA% and HBM GB/s vs peak",
-        "value": pre["tokens_per_s"],
+        "value": layer["tokens_per_s"],
         "unit": "tokens/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": pre["ms_per_step"],
+        "ms_per_step": layer["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "chunked prefill, one attention layer: B=2, 32q/8kv heads, head_dim 128, sink 64 + "
-                               "8 cascades x 2048 slots (full), 2048-token chunks, attention + score EMA + cache update"},
-        "roofline": pre["roofline"],
+        "config": {"workload": "one attention layer of the Llama-3.1-8B shape (B=1, 32q/8kv heads, head_dim 128, bf16) over "
+                               "sink 64 + 8 cascades x 8192 slots (64K window, full): per step one 4096-token prefill chunk "
+                               "and 8 single-token decode steps (the 131072 : 256 proportion of the full-model "
+                               "configuration), each = attention + score EMA + cache update",
+                   "tokens_per_step": cfg["B"] * (cfg["Q"] + cfg["decode_per_chunk"])},
+        "roofline": layer["roofline"],
         "cpu_baseline": cpu,
-        "prefill_stage_ms": pre["stage_ms"],
-        "prefill_attention_tflops_all_stages": pre["attention_tflops_all_stages"],
-        "decode": dec,
+        "cpu_config1": cpu1,
+        "prefill": layer["prefill"],
+        "decode": layer["decode"],
+        "update": layer["update"],
+        "cfg2_prefill": cfg2,
+        "cfg3_decode": cfg3,
     }
     print(json.dumps(line))
 

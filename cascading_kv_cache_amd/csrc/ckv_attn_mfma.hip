@@ -938,9 +938,12 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
     const int last_nrel = (int)(key_blk + 255 - p.Nc);
     const bool new_chunk = chunk_keys && p.new_mode;
     const bool pure_chunk = key_blk >= p.Nc;        // no cached key in the workgroup
-    if (new_chunk) {
+    // the weights of chunk keys by distance: a table in LDS, unless every entry is the same value (then the
+    // launch reserves no LDS for it, and two workgroups fit a compute unit whatever the chunk length)
+    if (new_chunk && !p.wnew_uniform) {
         for (int i = tid; i < Q; i += 256) wnew_lds[i] = p.w_new[i];
     }
+    auto wnew_at = [&](int i) -> float { return p.wnew_uniform ? p.wnew_value : wnew_lds[i]; };
     const int nmt = (Q - m_first + kQT2 - 1) / kQT2;  // query tiles per head
     const int n_steps = nmt * g_cnt;
 
@@ -1022,17 +1025,34 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
                 float ws[16];
                 load_weights(c - 1, ws);
                 __builtin_amdgcn_sched_barrier(0);
+                // an exponential is consumed one slot after it was issued, so no wavefront waits for the
+                // transcendental unit
+                float pe_prev[2] = {0.f, 0.f};
 #pragma unroll
                 for (int slot = 0; slot < 16; slot++) {
                     const int kk = slot >> 1, ks = slot & 1;
                     sq[c & 1][ks] = Mma<T>::mma(a1[kk], kreg[ks][kk], sq[c & 1][ks]);
+                    float pe[2];
 #pragma unroll
                     for (int r = 0; r < 2; r++) {
                         const int j = 2 * slot + r, ksv = j >> 4, v = j & 15;
-                        const float pe = __builtin_amdgcn_exp2f(sq[(c - 1) & 1][ksv][v]);
-                        acc[ksv] = fmaf(ws[v], pe, acc[ksv]);
+                        pe[r] = __builtin_amdgcn_exp2f(sq[(c - 1) & 1][ksv][v]);
                     }
+                    if (slot > 0) {
+#pragma unroll
+                        for (int r = 0; r < 2; r++) {
+                            const int j = 2 * (slot - 1) + r, ksv = j >> 4, v = j & 15;
+                            acc[ksv] = fmaf(ws[v], pe_prev[r], acc[ksv]);
+                        }
+                    }
+                    pe_prev[0] = pe[0];
+                    pe_prev[1] = pe[1];
                     __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int r = 0; r < 2; r++) {
+                    const int j = 30 + r, ksv = j >> 4, v = j & 15;
+                    acc[ksv] = fmaf(ws[v], pe_prev[r], acc[ksv]);
                 }
             }
             {
@@ -1050,15 +1070,14 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
         } else {
             // special cases, one 32-row subtile at a time
             const bool fast_new = !tail && !diag;   // new_chunk holds: every row is later than every key of the block
-            const float* wb[2] = {nullptr, nullptr};
             bool chunk_lane[2];
 #pragma unroll
-            for (int ks = 0; ks < 2; ks++) {
-                chunk_lane[ks] = nrel[ks] >= 0;
-                // a chunk key takes the weight of its distance m - n; a cached key (only in the block that
-                // straddles the chunk start) takes the row's EMA weight
-                wb[ks] = chunk_lane[ks] ? wnew_lds + (mt + 4 * half - nrel[ks]) : w_lds + 4 * half;
-            }
+            for (int ks = 0; ks < 2; ks++) chunk_lane[ks] = nrel[ks] >= 0;
+            // a chunk key takes the weight of its distance m - n; a cached key (only in the block that
+            // straddles the chunk start) takes the row's EMA weight
+            auto weight_of = [&](int ks, int r) -> float {
+                return chunk_lane[ks] ? wnew_at(mt + 4 * half - nrel[ks] + r) : w_lds[4 * half + r];
+            };
 #pragma unroll 1
             for (int c = 0; c < kCsSub; c++) {
                 f32x16 sacc[2];
@@ -1093,7 +1112,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
 #pragma unroll
                             for (int ks = 0; ks < 2; ks++) {
                                 const float pe = __builtin_amdgcn_exp2f(sacc[ks][4 * v4 + e]);
-                                const float w = wb[ks][r0 + e];
+                                const float w = weight_of(ks, r0 + e);
                                 if (pure_chunk) {
                                     acc[ks] += Mma<T>::round1(Mma<T>::round1(pe) * w);
                                 } else {
@@ -1118,7 +1137,7 @@ __global__ void __launch_bounds__(256, 2) colsum_mfma_kernel(ColsumParams p) {
                             pe = vis ? pe : 0.f;
                             if (is_chunk && p.new_mode) {
                                 // the eager path holds P and the products in the tensor dtype
-                                const float w = vis ? wnew_lds[m - nrel[ks]] : 0.f;
+                                const float w = vis ? wnew_at(m - nrel[ks]) : 0.f;
                                 acc[ks] += Mma<T>::round1(Mma<T>::round1(pe) * w);
                             } else {
                                 acc[ks] = fmaf(row_in ? we : 0.f, pe, acc[ks]);
@@ -1299,7 +1318,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         // pipeline start serve twice the work, and the units stay small enough for an even last round
         cp.gsplit = (G % 2 == 0 && G >= 4) ? G / 2 : G;
         const dim3 grid((unsigned)(cp.nkb * cp.nbkv * cp.gsplit));
-        const int lds = 2 * kCsStage + (int)mp.Q * 4;
+        const int lds = 2 * kCsStage + (cp.wnew_uniform ? 0 : (int)mp.Q * 4);
         if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(colsum_mfma_kernel<T>), lds)) return rc;
         hipLaunchKernelGGL(colsum_mfma_kernel<T>, grid, dim3(256), lds, stream, cp);
         CKV_HIP_TRY(hipGetLastError());
