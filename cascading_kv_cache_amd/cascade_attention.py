@@ -32,6 +32,20 @@ def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_p
     ``_stream``: raw stream handle when the caller already holds the device context."""
     _require_device(cache.key_cache[layer_idx], "the cache")
     dev = cache.key_cache[layer_idx].device
+    # Steady state of an eagerly filled cache: every token up to index S + num_sink was accepted by every
+    # cascade (cascading_cache.py:471-478), so from then on every slot holds a token, the largest position id
+    # is S - 1 plus the sink shift, and the chunk starts at S + num_sink whatever the stream does later.  The
+    # ids are then a constant vector, kept per length: no kernel, no device read.
+    S, NS = cache.max_seq_len[layer_idx], cache.num_sink_tokens
+    if not do_og_pos and cache.eager_fill and cache._seen_host[layer_idx] >= S + NS and S > 0:
+        memo = cache.__dict__.setdefault("_steady_q_pos", {})
+        key = (S + NS, q_len, dev)
+        ids = memo.get(key)
+        if ids is None:
+            if len(memo) > 16:
+                memo.clear()
+            ids = memo[key] = torch.arange(S + NS, S + NS + q_len, device=dev, dtype=torch.long)
+        return ids
     out = torch.empty(q_len, device=dev, dtype=torch.long)
     key_ptr, n_key, shift, sink_ptr, n_sink = None, 0, 0, None, 0
     if cache._seen_host[layer_idx] != 0:
@@ -183,6 +197,72 @@ def cascade_attention(query_states, key_states, value_states, cache: CascadingKV
         if update_cache:
             cache.update_state(key_states, value_states, L, score_states=new_scores, _stream=stream)
     return out, new_scores
+
+
+class DecodeStepGraph:
+    """Single-token steps of one layer replayed from a HIP graph.
+
+    A decode step is a chain of short kernels (query rotation, streaming attention, combine, scores, update plan,
+    update apply, the token counter); at batch 1 and small windows the host needs longer to launch them than the
+    device to run them.  The first ``step`` runs eagerly (it sets kernel attributes and sizes the scratch), the
+    second one records the same calls into a graph, and every later one copies the token's q, k, v into the
+    graph's fixed input buffers and replays it.  The cache is advanced exactly as by ``cascade_attention``; the
+    returned ``out`` / ``new_scores`` tensors are the graph's fixed outputs and are overwritten by the next step.
+
+    Recorded values that must not change between steps: the sink shift (the cache must already hold more than
+    ``num_sink_tokens`` tokens), shapes, dtype, head reduction, and the state tensors of the cache (``reset()``
+    or assigning a new tensor to ``score_cache[l]`` invalidates the graph: build a new one)."""
+
+    def __init__(self, cache: CascadingKVCache, layer_idx: int, inv_freq: torch.Tensor, num_heads: int,
+                 head_reduction: Optional[str] = None, homogeneous_heads: bool = False, do_og_pos: bool = False,
+                 scale: Optional[float] = None):
+        self.cache, self.layer_idx, self.inv_freq = cache, layer_idx, inv_freq
+        self.kw = dict(head_reduction=head_reduction, homogeneous_heads=homogeneous_heads, do_og_pos=do_og_pos,
+                       scale=scale)
+        kc = cache.key_cache[layer_idx]
+        B, KVH, _, D = kc.shape
+        self.q = torch.empty(B, num_heads, 1, D, dtype=kc.dtype, device=kc.device)
+        self.k = torch.empty(B, KVH, 1, D, dtype=kc.dtype, device=kc.device)
+        self.v = torch.empty(B, KVH, 1, D, dtype=kc.dtype, device=kc.device)
+        self.graph = None
+        self.out = self.new_scores = None
+        self._warm = False
+        self._state = None
+
+    def _run(self):
+        return cascade_attention(self.q, self.k, self.v, self.cache, self.layer_idx, self.inv_freq, **self.kw)
+
+    def step(self, q=None, k=None, v=None):
+        """One token: ``q (B, H, 1, D)``, ``k, v (B, KVH, 1, D)`` (or None when the caller has written them into
+        ``self.q / self.k / self.v`` already).  Returns ``(out, new_scores)``."""
+        cache, L = self.cache, self.layer_idx
+        if cache._seen_host[L] <= cache.num_sink_tokens:
+            raise _abi.CkvError("DecodeStepGraph needs a cache that already holds more than num_sink_tokens tokens")
+        if q is not None:
+            self.q.copy_(q)
+            self.k.copy_(k)
+            self.v.copy_(v)
+        if not self._warm:  # eager: kernel attributes, scratch sizes, argument blocks
+            self._warm = True
+            return self._run()
+        if self.graph is not None and self._state != cache._state_key(L):
+            raise _abi.CkvError("the cache's state tensors moved since the graph was recorded")
+        if self.graph is None:
+            if _abi.profile_enable(0) != 0:
+                raise _abi.CkvError("stage timing must be off while a step is recorded")
+            seen_host, seen_total = cache._seen_host[L], cache._seen_tokens
+            self._state = cache._state_key(L)
+            torch.cuda.synchronize(self.q.device)
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self.out, self.new_scores = self._run()
+            # recording ran no kernel: only the host-side counters moved, and the replay below is the step
+            cache._seen_host[L], cache._seen_tokens = seen_host, seen_total
+        self.graph.replay()
+        cache._seen_host[L] += 1
+        if L == 0:
+            cache._seen_tokens += 1
+        return self.out, self.new_scores
 
 
 class CascadeAttention(nn.Module):

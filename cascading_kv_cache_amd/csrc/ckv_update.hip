@@ -285,6 +285,96 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
     if (p.do_pos && tid == 0) p.pos_flag[bh] = cap > n_sink_new ? 1 : 0;
 }
 
+// The plan of a single incoming token (the decode step): one wavefront per (batch, kv head), no workgroup
+// barriers.  Lane i fetches what cascade i may need (trackers, period, the scores of its oldest and its newest
+// slot) so that all cascades' loads travel together; the walk over the cascades then runs on values handed
+// round by shuffles, identical in every lane, and lane 0 writes the chain.  Same semantics as the general
+// kernel (cascading_cache.py:381-726 for one token).
+__global__ void __launch_bounds__(CKV_WAVE) ckv_update_plan1_kernel(UpdateParams p) {
+    const ckv_update_args& A = p.a;
+    const int lane = threadIdx.x;
+    const int64_t bh = blockIdx.x;
+    const int64_t n = bh / A.H, h = bh % A.H;
+    const int C = A.cascades;
+    const int64_t W = A.window_size, S = A.max_seq_len, NS = A.num_sink;
+    int64_t* g_stored = A.stored_tokens + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+    int64_t* g_start = A.start_indices + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+    int64_t* g_sinks = A.stored_sinks + n * A.stored_sinks_stride[0] + h * A.stored_sinks_stride[1];
+    const int64_t cs_base = n * A.cache_s_stride[0] + h * A.cache_s_stride[1];
+    int32_t* first = p.first + bh * A.K + p.token_offset;
+    int32_t* next_of = p.next_of + bh * S;
+
+    const int64_t gidx = *A.real_token_idx + p.token_offset;  // 0-based global index of the token
+    const int64_t sinks0 = *g_sinks;
+    const float tok_score = load_as_float(A.s, n * A.s_stride[0] + h * A.s_stride[1] + p.token_offset * A.s_stride[2], A.dtype);
+    // lane i: cascade i
+    int32_t st = 0, sx = 0;
+    int64_t per = 1;
+    float oldest = 0.f, newest = 0.f;
+    if (lane < C) {
+        st = (int32_t)g_stored[lane * A.tracker_stride[2]];
+        sx = (int32_t)g_start[lane * A.tracker_stride[2]];
+        per = A.do_cache_every_n[lane];
+        const int64_t l = (int64_t)lane * W;
+        if (st > 0) {
+            oldest = load_as_float(A.cache_s, cs_base + (l + sx) * A.cache_s_stride[2], A.dtype);
+            newest = load_as_float(A.cache_s, cs_base + (l + (sx - 1 + st) % st) * A.cache_s_stride[2], A.dtype);
+        }
+    }
+    if (sinks0 < NS) {  // the token is a sink (cascading_cache.py:399-431): no position pass
+        if (lane == 0) {
+            first[0] = (int32_t)(S + sinks0);
+            *g_sinks = sinks0 + 1;
+            if (p.do_pos) p.pos_flag[bh] = 0;
+        }
+        return;
+    }
+    int carry_src = -1;          // -1 - token index, or the slot whose old content is carried
+    float carry_score = tok_score;
+    int32_t first_val = -1;      // where the token lands (-1: dropped)
+    const int64_t rel = gidx - NS;
+    const bool eager = A.eager_fill && gidx <= S + NS;
+    for (int i = 0; i < C; i++) {
+        const int32_t st_i = __shfl(st, i), sx_i = __shfl(sx, i);
+        const int64_t per_i = __shfl(per, i);
+        const int l = (int)((int64_t)i * W);
+        const bool acc = eager || (rel % per_i) == 0;
+        if (acc || st_i == 0) {
+            const int phys = l + (int)(((int64_t)sx_i + st_i) % W);
+            if (st_i < (int32_t)W) {  // append (or the first entry of an empty cascade)
+                if (lane == 0) {
+                    next_of[phys] = -1;
+                    if (carry_src < 0) first_val = phys; else next_of[carry_src] = phys;
+                    g_stored[i * A.tracker_stride[2]] = st_i + 1;
+                }
+                break;
+            }
+            // full: the oldest entry (at the ring start) leaves for the next cascade, or is dropped
+            if (lane == 0) {
+                next_of[phys] = -1;
+                if (carry_src < 0) first_val = phys; else next_of[carry_src] = phys;
+                g_start[i * A.tracker_stride[2]] = (int64_t)((sx_i + 1) % (int32_t)W);
+            }
+            carry_src = phys;
+            carry_score = __shfl(oldest, i);
+            continue;
+        }
+        // not accepted: the newest slot keeps its token unless the arrival's score is at least as large
+        if (carry_score >= __shfl(newest, i)) {
+            const int p_lead = l + (sx_i - 1 + st_i) % st_i;
+            if (lane == 0) {
+                next_of[p_lead] = -1;
+                if (carry_src < 0) first_val = p_lead; else next_of[carry_src] = p_lead;
+            }
+        }
+        break;
+    }
+    if (lane == 0) {
+        first[0] = first_val;
+        if (p.do_pos) p.pos_flag[bh] = 1;
+    }
+}
+
 // Position pass (cascading_cache.py:728-774, 129-142) after the plan kernel has updated the trackers:
 // slot j of cascade i gets ((j + seg - start) mod seg) + ub - seg, where seg is the number of stored
 // tokens and ub the ids still to hand out (all stored tokens, less a window per earlier cascade).
@@ -405,48 +495,67 @@ __global__ void ckv_update_apply_vec_kernel(UpdateParams p) {
     int64_t* og = A.og_pos + n * A.og_pos_stride[0] + h * A.og_pos_stride[1];
     uint8_t* mask = A.mask + n * A.mask_stride[0] + h * A.mask_stride[1];
 
-    // The successor of the next slot is requested together with the displaced row, so a hop costs one
-    // trip to memory, not two.
-    int nd = next_of[d];
-    for (int hop = 0; hop <= A.cascades; hop++) {  // a chain visits each cascade at most once
-        RowPiece old;
-        uint32_t o_score = 0;
-        int64_t o_og = 0;
-        int nnd = -1;
-        uint4* kd = reinterpret_cast<uint4*>(ck + (int64_t)d * row_bytes);
-        uint4* vd = reinterpret_cast<uint4*>(cv + (int64_t)d * row_bytes);
-        const int64_t sidx = cs_base + (int64_t)d * A.cache_s_stride[2];
-        if (nd >= 0) {  // the displaced row lives on elsewhere: pick it up before overwriting
-            nnd = next_of[nd];
+    // A chain is walked kHops slots at a time.  First only its slot numbers (4-byte loads that depend on
+    // each other, served by the L2 the plan kernel has just written them to); then every displaced row of
+    // the stretch is requested at once, so the rows cost one trip to memory instead of one per hop; then
+    // the stretch is written: slot 0 takes the carried row, slot j the row displaced from slot j - 1.
+    constexpr int kHops = 8;
+    for (int round = 0; round * kHops <= A.cascades; round++) {  // a chain visits each cascade at most once
+        int sl[kHops];
+        int nx = d;
+#pragma unroll
+        for (int j = 0; j < kHops; j++) {
+            sl[j] = nx;
+            nx = nx >= 0 ? next_of[nx] : -1;
+        }
+        RowPiece old[kHops];
+        uint32_t o_score[kHops];
+        int64_t o_og[kHops];
+#pragma unroll
+        for (int j = 0; j < kHops; j++) {
+            const int succ = j + 1 < kHops ? sl[j + 1] : nx;
+            old[j].k = old[j].v = make_uint4(0, 0, 0, 0);
+            o_score[j] = 0;
+            o_og[j] = 0;
+            if (sl[j] >= 0 && succ >= 0) {  // the displaced row lives on elsewhere: pick it up
+                if (active) {
+                    old[j].k = reinterpret_cast<const uint4*>(ck + (int64_t)sl[j] * row_bytes)[lane];
+                    old[j].v = reinterpret_cast<const uint4*>(cv + (int64_t)sl[j] * row_bytes)[lane];
+                }
+                if (lane == 0) {
+                    const int64_t sidx = cs_base + (int64_t)sl[j] * A.cache_s_stride[2];
+                    o_score[j] = es == 4 ? reinterpret_cast<const uint32_t*>(A.cache_s)[sidx]
+                                         : reinterpret_cast<const uint16_t*>(A.cache_s)[sidx];
+                    o_og[j] = og[(int64_t)sl[j] * A.og_pos_stride[2]];
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kHops; j++) {
+            if (sl[j] < 0) continue;
+            const RowPiece& src = j == 0 ? carry : old[j - 1];
+            const uint32_t w_score = j == 0 ? c_score : o_score[j - 1];
+            const int64_t w_og = j == 0 ? c_og : o_og[j - 1];
             if (active) {
-                old.k = kd[lane];
-                old.v = vd[lane];
+                reinterpret_cast<uint4*>(ck + (int64_t)sl[j] * row_bytes)[lane] = src.k;
+                reinterpret_cast<uint4*>(cv + (int64_t)sl[j] * row_bytes)[lane] = src.v;
             }
             if (lane == 0) {
-                o_score = es == 4 ? reinterpret_cast<const uint32_t*>(A.cache_s)[sidx]
-                                  : reinterpret_cast<const uint16_t*>(A.cache_s)[sidx];
-                o_og = og[(int64_t)d * A.og_pos_stride[2]];
+                const int64_t sidx = cs_base + (int64_t)sl[j] * A.cache_s_stride[2];
+                if (es == 4) {
+                    reinterpret_cast<uint32_t*>(A.cache_s)[sidx] = w_score;
+                } else {
+                    reinterpret_cast<uint16_t*>(A.cache_s)[sidx] = (uint16_t)w_score;
+                }
+                og[(int64_t)sl[j] * A.og_pos_stride[2]] = w_og;
+                mask[(int64_t)sl[j] * A.mask_stride[2]] = 0;
             }
         }
-        if (active) {
-            kd[lane] = carry.k;
-            vd[lane] = carry.v;
-        }
-        if (lane == 0) {
-            if (es == 4) {
-                reinterpret_cast<uint32_t*>(A.cache_s)[sidx] = c_score;
-            } else {
-                reinterpret_cast<uint16_t*>(A.cache_s)[sidx] = (uint16_t)c_score;
-            }
-            og[(int64_t)d * A.og_pos_stride[2]] = c_og;
-            mask[(int64_t)d * A.mask_stride[2]] = 0;
-        }
-        if (nd < 0) break;
-        carry = old;
-        c_score = o_score;
-        c_og = o_og;
-        d = nd;
-        nd = nnd;
+        if (nx < 0) break;
+        carry = old[kHops - 1];
+        c_score = o_score[kHops - 1];
+        c_og = o_og[kHops - 1];
+        d = nx;
     }
 }
 
@@ -629,10 +738,13 @@ int run_update(const ckv_update_args& A, void* workspace, hipStream_t stream) {
         p.token_offset = off;
         p.k_sub = ksub;
         p.do_pos = (off + ksub == A.K) ? 1 : 0;
-        const int T = ksub <= 256 ? 256 : 1024;  // few tokens: a small block plans them
-        const size_t lds = plan_lds_bytes(ksub);
-        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(ckv_update_plan_kernel), (int)lds)) return rc;
-        {
+        if (ksub == 1) {  // the decode step: one wavefront per unit
+            StageScope sc(CKV_STAGE_PLAN, stream);
+            hipLaunchKernelGGL(ckv_update_plan1_kernel, dim3((unsigned)(A.N * A.H)), dim3(CKV_WAVE), 0, stream, p);
+        } else {
+            const int T = ksub <= 256 ? 256 : 1024;  // few tokens: a small block plans them
+            const size_t lds = plan_lds_bytes(ksub);
+            if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(ckv_update_plan_kernel), (int)lds)) return rc;
             StageScope sc(CKV_STAGE_PLAN, stream);
             hipLaunchKernelGGL(ckv_update_plan_kernel, dim3((unsigned)(A.N * A.H)), dim3(T), lds, stream, p);
         }
