@@ -150,8 +150,29 @@ def update_bytes(cache, cfg, k, v, new_scores, es=2):
     return float(total), dict(rows_in=B * KVH * q_len, rows_relocated=n_reloc, slots_rewritten=n_changed)
 
 
-def stage_table(stages):
-    return {k: (ms / n if n else 0.0) for k, (ms, n) in stages.items()}
+def update_kernel_ms(cache, k, v, new_scores, reps=20):
+    """Kernel time of one cache update: the durations of all its kernels (plan and apply launches), each timed by
+    events attached to its own dispatch, summed per call.  The calls advance the (steady-state) cache."""
+    from cascading_kv_cache_amd import _abi
+
+    for _ in range(3):
+        cache.update_state(k, v, 0, new_scores)
+    torch.cuda.synchronize()
+    _abi.profile_enable(3)
+    _abi.profile_read()
+    for _ in range(reps):
+        cache.update_state(k, v, 0, new_scores)
+    torch.cuda.synchronize()
+    st = _abi.profile_read()
+    _abi.profile_enable(0)
+    return (st["plan"][0] + st["apply"][0]) / reps, {"plan_ms": st["plan"][0] / reps, "apply_ms": st["apply"][0] / reps,
+                                                       "launches_per_call": (st["plan"][1] + st["apply"][1]) / reps}
+
+
+def stage_table(stages, calls=None):
+    """Milliseconds per stage: per launch of the stage, or, with `calls`, per call of the operator (a stage may
+    be several launches of one call: the update plans a long chunk in pieces)."""
+    return {k: (ms / (calls if calls else n) if n else 0.0) for k, (ms, n) in stages.items()}
 
 
 def run_layer(steps, warmup, dtype, device):
@@ -219,14 +240,15 @@ def run_layer(steps, warmup, dtype, device):
     token_graph_s = phase(one_token_graph, 64)
     _abi.profile_enable(1)
     _abi.profile_read()
-    for i in range(max(3, min(steps, 10))):
+    n_pre = max(3, min(steps, 10))
+    for i in range(n_pre):
         one_chunk(i)
     torch.cuda.synchronize()
-    pre_stages = stage_table(_abi.profile_read())
+    pre_stages = stage_table(_abi.profile_read(), n_pre)
     for i in range(32):
         one_token(i)
     torch.cuda.synchronize()
-    dec_stages = stage_table(_abi.profile_read())
+    dec_stages = stage_table(_abi.profile_read(), 32)
     _abi.profile_enable(0)
 
     B, Q = cfg["B"], cfg["Q"]
@@ -242,7 +264,8 @@ def run_layer(steps, warmup, dtype, device):
     q, k, v = pool[0]
     new_scores = torch.rand(B, cfg["KVH"], Q, device=device).mul_(1e-6).to(dtype)
     ubytes, ucount = update_bytes(cache, cfg, k, v, new_scores)
-    upd_ms = pre_stages["plan"] + pre_stages["apply"]
+    upd_ms, upd_parts = update_kernel_ms(cache, k, v, new_scores)
+    ucount.update(upd_parts)
     res = dict(
         ms_per_step=dt / steps * 1e3,
         tokens_per_s=B * (Q + n_dec) * steps / dt,
@@ -296,7 +319,7 @@ def run_cfg2(steps, warmup, dtype, device):
     for i in range(min(steps, 10)):
         cascade_attention(*pool[i % len(pool)], cache, 0, inv_freq)
     torch.cuda.synchronize()
-    stages = stage_table(_abi.profile_read())
+    stages = stage_table(_abi.profile_read(), min(steps, 10))
     _abi.profile_enable(0)
     B, H, Q = cfg["B"], cfg["H"], cfg["Q"]
     flops = prefill_flops(cfg)
@@ -306,7 +329,8 @@ def run_cfg2(steps, warmup, dtype, device):
     q, k, v = pool[0]
     new_scores = torch.rand(B, cfg["KVH"], Q, device=device).mul_(1e-6).to(dtype)
     ubytes, ucount = update_bytes(cache, cfg, k, v, new_scores)
-    upd_ms = stages["plan"] + stages["apply"]
+    upd_ms, upd_parts = update_kernel_ms(cache, k, v, new_scores)
+    ucount.update(upd_parts)
     return dict(
         workload="chunked prefill: B=2, 32q/8kv heads, head_dim 128, sink 64 + 8 cascades x 2048 slots (full), 2048-token chunks",
         ms_per_step=dt / steps * 1e3, tokens_per_s=B * Q * steps / dt,
@@ -373,7 +397,7 @@ def run_cfg3(steps, warmup, dtype, device):
     for i in range(min(steps, 10)):
         cascade_attention(*pool[i % len(pool)], cache, 0, inv_freq)
     torch.cuda.synchronize()
-    stages = stage_table(_abi.profile_read())
+    stages = stage_table(_abi.profile_read(), min(steps, 10))
     _abi.profile_enable(0)
     B = cfg["B"]
     algo = decode_bytes(cfg)
@@ -382,7 +406,8 @@ def run_cfg3(steps, warmup, dtype, device):
     q, k, v = pool[0]
     new_scores = torch.rand(B, cfg["KVH"], 1, device=device).mul_(1e-6).to(dtype)
     ubytes, ucount = update_bytes(cache, cfg, k, v, new_scores)
-    upd_ms = stages["plan"] + stages["apply"]
+    upd_ms, upd_parts = update_kernel_ms(cache, k, v, new_scores)
+    ucount.update(upd_parts)
     return dict(
         workload="decode: B=16, 32q/8kv heads, head_dim 128, sink 64 + 4 cascades x 8192 slots (full), q=1",
         ms_per_step=dt / steps * 1e3, tokens_per_s=B * steps / dt, ms_per_step_graph_replay=dt_graph / steps * 1e3,

@@ -56,13 +56,16 @@ int ensure_dynamic_lds(const void* func, int bytes) {
     return CKV_OK;
 }
 
-static bool prof_wanted(int stage) {
-    return g_prof_level == 1 || (g_prof_level == 2 && (stage == CKV_STAGE_FWD || stage == CKV_STAGE_DECODE));
+// level 2: the attention main kernels; level 3: the kernels of the cache update.  Both time single kernels by
+// events attached to their dispatch.
+static bool dispatch_timed(int stage) {
+    return (g_prof_level == 2 && (stage == CKV_STAGE_FWD || stage == CKV_STAGE_DECODE)) ||
+           (g_prof_level == 3 && (stage == CKV_STAGE_PLAN || stage == CKV_STAGE_APPLY));
 }
 
-bool prof_kernel_events_wanted(int stage) {
-    return g_prof_level == 2 && (stage == CKV_STAGE_FWD || stage == CKV_STAGE_DECODE);
-}
+static bool prof_wanted(int stage) { return g_prof_level == 1 || dispatch_timed(stage); }
+
+bool prof_kernel_events_wanted(int stage) { return dispatch_timed(stage); }
 
 void prof_kernel_events(int stage, hipEvent_t* start, hipEvent_t* stop) {
     *start = *stop = nullptr;
@@ -103,7 +106,7 @@ void prof_end(int stage, hipStream_t stream) {
 
 extern "C" int ckv_profile_enable(int on) {
     const int prev = ckv::g_prof_level;
-    ckv::g_prof_level = on < 0 || on > 2 ? 1 : on;
+    ckv::g_prof_level = on < 0 || on > 3 ? 1 : on;
     return prev;
 }
 

@@ -41,6 +41,8 @@ struct UpdateParams {
     int32_t* first;        // [N*H][K]
     int32_t* next_of;      // [N*H][S]
     int32_t* pos_flag;     // [N*H]: the call put a token into the cascades, so the position ids change
+    int32_t* mode;         // [N*H]: 1 = planned by the steady-state kernel: the new ring starts wait in start_new
+    int32_t* start_new;    // [N*H][cascades]: ring starts after the call, committed by the apply kernel
     int32_t apply_blocks;  // blocks along x that move rows; the blocks behind them write position ids
 };
 
@@ -78,13 +80,14 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
     const ckv_update_args& A = p.a;
     const int tid = threadIdx.x, T = blockDim.x;
     const int64_t bh = blockIdx.x;
+    if (p.mode[bh]) return;  // the steady-state kernel has planned this unit
     const int64_t n = bh / A.H, h = bh % A.H;
     const int cap = p.k_sub;
     const int C = A.cascades;
     const int64_t W = A.window_size, S = A.max_seq_len, NS = A.num_sink;
 
     int32_t* a_src[2];
-    int32_t* a_trig[2];
+    uint16_t* a_trig[2];   // index of the token whose arrival set the entry moving: below kPlanMaxTokens
     float* a_score[2];
     unsigned char* ptr = smem;
     // per cascade, fetched once up front so that no cascade waits for global memory on their account:
@@ -93,7 +96,6 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
     float* lead_l = reinterpret_cast<float*>(ptr); ptr += 4 * kMaxCascades;
     for (int i = 0; i < 2; i++) {
         a_src[i] = reinterpret_cast<int32_t*>(ptr); ptr += 4 * (size_t)cap;
-        a_trig[i] = reinterpret_cast<int32_t*>(ptr); ptr += 4 * (size_t)cap;
         a_score[i] = reinterpret_cast<float*>(ptr); ptr += 4 * (size_t)cap;
     }
     uint32_t* eflag = reinterpret_cast<uint32_t*>(ptr); ptr += 4 * (size_t)cap;
@@ -102,7 +104,10 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
     float* w_score = reinterpret_cast<float*>(ptr); ptr += 4 * (size_t)(cap + 1);
     int32_t* st_l = reinterpret_cast<int32_t*>(ptr); ptr += 4 * kMaxCascades;
     int32_t* sx_l = reinterpret_cast<int32_t*>(ptr); ptr += 4 * kMaxCascades;
-    int* wave_tot = reinterpret_cast<int*>(ptr);
+    int* wave_tot = reinterpret_cast<int*>(ptr); ptr += 64 * sizeof(int);
+    for (int i = 0; i < 2; i++) {
+        a_trig[i] = reinterpret_cast<uint16_t*>(ptr); ptr += 2 * (size_t)((cap + 1) & ~1);
+    }
 
     int64_t* g_stored = A.stored_tokens + n * A.tracker_stride[0] + h * A.tracker_stride[1];
     int64_t* g_start = A.start_indices + n * A.tracker_stride[0] + h * A.tracker_stride[1];
@@ -136,7 +141,7 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
             first[t] = -1;
             const int a = t - n_sink_new;
             a_src[0][a] = -1 - t;
-            a_trig[0][a] = t;
+            a_trig[0][a] = (uint16_t)t;
             a_score[0][a] = load_as_float(
                 A.s, n * A.s_stride[0] + h * A.s_stride[1] + (p.token_offset + t) * A.s_stride[2], A.dtype);
         }
@@ -163,7 +168,7 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
         const bool per_small = small && per > 0 && per < (1ll << 31);
         const bool per_pow2 = per > 0 && (per & (per - 1)) == 0;
         const int32_t* Asrc = a_src[cur];
-        const int32_t* Atrig = a_trig[cur];
+        const uint16_t* Atrig = a_trig[cur];
         const float* Ascore = a_score[cur];
 
         // Scores of the ring entries this call can evict (the oldest ones, at most one per arrival beyond
@@ -237,7 +242,7 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
         const int room_i = (int)W - stored0;          // inserts that still append
         const bool has_next = (i + 1 < C);
         int32_t* Bsrc = a_src[cur ^ 1];
-        int32_t* Btrig = a_trig[cur ^ 1];
+        uint16_t* Btrig = a_trig[cur ^ 1];
         float* Bscore = a_score[cur ^ 1];
         for (int a = tid; a < nA; a += T) {
             const uint32_t ef = eflag[a];
@@ -285,6 +290,217 @@ __global__ void ckv_update_plan_kernel(UpdateParams p) {
     if (p.do_pos && tid == 0) p.pos_flag[bh] = cap > n_sink_new ? 1 : 0;
 }
 
+// Steady-state plan: every cascade of the unit is full, no token of the call is accepted by the eager-fill rule,
+// and every acceptance period divides the next one (the power schedules).  Then which arrivals a cascade sees,
+// which of them are inserted and where, is a closed form of the token counter: the arrivals of cascade i are
+// the tokens whose index is a multiple of period i-1, every (period i / period i-1)-th of them is inserted,
+// the n-th insert lands n slots behind the ring start and pushes the n-th oldest entry on to cascade i+1.
+// As long as a cascade evicts only entries the call has not touched, its arrivals can be read straight from
+// the cache as it was before the call, so every cascade is planned by workgroups of its own, side by side:
+// one thread per insert folds the arrivals up to the next insert into the group's winner ("later wins iff
+// score >=", cascading_cache.py:699) and writes where every member of the group ends up.  Every chain entry
+// has one writer: the workgroups of cascade i own the pointers of cascade i's arrivals.  The ring starts after
+// the call go to scratch (the neighbours still read the old ones); the apply kernel commits them.
+// A unit that does not meet the conditions is left to the general kernel (mode 0).
+constexpr int kSteadyParts = 4;   // workgroups per cascade and unit
+constexpr int kSteadyThreads = 256;
+
+struct SteadyCascade {
+    int64_t per_prev, r;   // period of the cascade before, inserts every r-th arrival
+    int64_t a0;            // first token of the call that arrives at this cascade
+    int32_t nA, kf, E;     // arrivals, index of the first inserted arrival, inserts
+    int32_t sx;            // ring start before the call
+};
+
+__global__ void __launch_bounds__(kSteadyThreads) ckv_update_plan_steady_kernel(UpdateParams p) {
+    __shared__ SteadyCascade sc[kMaxCascades];
+    __shared__ int64_t st_s[kMaxCascades], sx_s[kMaxCascades], per_s[kMaxCascades], seen_s, sinks_s;
+    __shared__ int fast_s;
+    const ckv_update_args& A = p.a;
+    const int tid = threadIdx.x;
+    const int64_t bh = blockIdx.y;
+    const int i = blockIdx.x / kSteadyParts, part = blockIdx.x % kSteadyParts;
+    const int64_t n = bh / A.H, h = bh % A.H;
+    const int C = A.cascades;
+    const int64_t W = A.window_size, S = A.max_seq_len, NS = A.num_sink;
+    const int cap = (int)A.K;  // the whole call is planned at once
+    const int64_t* g_stored = A.stored_tokens + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+    const int64_t* g_start = A.start_indices + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+    // the trackers of all cascades travel together; one thread then works out the closed forms
+    if (tid < C) {
+        st_s[tid] = g_stored[tid * A.tracker_stride[2]];
+        sx_s[tid] = g_start[tid * A.tracker_stride[2]];
+        per_s[tid] = A.do_cache_every_n[tid];
+    } else if (tid == kMaxCascades) {
+        seen_s = *A.real_token_idx;
+    } else if (tid == kMaxCascades + 1) {
+        sinks_s = A.stored_sinks[n * A.stored_sinks_stride[0] + h * A.stored_sinks_stride[1]];
+    }
+    __syncthreads();
+    // one thread per cascade works out that cascade's closed forms (they depend on the token counter and the
+    // periods only); 32-bit division when everything fits, which it does outside pathological streams
+    __shared__ int ok_s[kMaxCascades];
+    if (tid < C) {
+        const int j = tid;
+        const int64_t seen = seen_s, sinks0 = sinks_s;
+        const int64_t rel0 = seen - NS;
+        const int64_t per = per_s[j], per_prev = j == 0 ? 1 : per_s[j - 1];
+        const int64_t st = st_s[j], sx = sx_s[j];
+        bool ok = sinks0 >= NS && rel0 >= 0 && !(A.eager_fill && seen <= S + NS) && W >= 2 && W < (1ll << 30) &&
+                  cap < (1 << 30) && per > 0 && per_prev > 0 && st == W && sx >= 0 && sx < W;
+        SteadyCascade c;
+        c.per_prev = per_prev;
+        c.r = 1;
+        c.nA = c.kf = c.E = 0;
+        c.sx = (int32_t)sx;
+        c.a0 = 0;
+        if (ok) {
+            const bool small = rel0 < (1ll << 31) && per < (1ll << 31);
+            auto mod = [&](int64_t x, int64_t y) -> int64_t { return small ? (int64_t)((uint32_t)x % (uint32_t)y) : x % y; };
+            auto div = [&](int64_t x, int64_t y) -> int64_t { return small ? (int64_t)((uint32_t)x / (uint32_t)y) : x / y; };
+            ok = mod(per, per_prev) == 0;
+            if (ok) {
+                c.r = div(per, per_prev);
+                const int64_t a0 = mod(per_prev - mod(rel0, per_prev), per_prev);   // first token that arrives here
+                c.a0 = a0;
+                c.nA = a0 < cap ? (int32_t)div(cap - a0 + per_prev - 1, per_prev) : 0;
+                const int64_t q0 = div(rel0 + a0, per_prev);                       // arrival k is inserted iff (q0 + k) % r == 0
+                c.kf = (int32_t)mod(c.r - mod(q0, c.r), c.r);
+                c.E = c.nA > c.kf ? (int32_t)div((int64_t)c.nA - c.kf + c.r - 1, c.r) : 0;
+                // what the cascade evicts must be entries the call has not touched: at most all but the newest
+                // old entry; or all of them when no arrival challenges that entry before the first insert; cascade
+                // 0 with period 1 has no challengers at all, and what it evicts beyond its old entries are the
+                // call's own tokens in order
+                const bool untouched = c.E <= W - 1 || (c.E <= W && c.kf == 0) || (j == 0 && per == 1);
+                ok = j + 1 < C ? untouched : (c.E <= W || (j == 0 && per == 1));
+            }
+        }
+        sc[j] = c;
+        ok_s[j] = ok ? 1 : 0;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        bool ok = true;
+        for (int j = 0; j < C; j++) {
+            ok = ok && ok_s[j];
+            if (j >= 1 && sc[j - 1].E != sc[j].nA) ok = false;  // evictions of a full cascade = its inserts
+        }
+        fast_s = ok ? 1 : 0;
+    }
+    __syncthreads();
+    const bool fast = fast_s != 0;
+    if (blockIdx.x == 0 && tid == 0) {
+        p.mode[bh] = fast ? 1 : 0;
+        if (fast) p.pos_flag[bh] = 1;
+    }
+    if (!fast) return;
+    const SteadyCascade c = sc[i];
+    const int64_t cs_base = n * A.cache_s_stride[0] + h * A.cache_s_stride[1];
+    int32_t* first = p.first + bh * A.K;
+    int32_t* next_of = p.next_of + bh * S;
+    const int l = (int)((int64_t)i * W);
+    const int Wi = (int)W;
+    const bool prev_passes_tokens = i == 1 && sc[0].per_prev == 1 && sc[0].r == 1;  // cascade 0 has period 1
+    const int sx_prev = i >= 1 ? sc[i - 1].sx : 0;
+    // arrival k of this cascade: where it comes from (-1 - token, or the slot of the cascade before) and its score
+    auto arrival = [&](int k, int& src, float& score) {
+        if (i == 0) {
+            const int64_t t = c.a0 + (int64_t)k * c.per_prev;
+            src = -1 - (int)t;
+            score = load_as_float(A.s, n * A.s_stride[0] + h * A.s_stride[1] + t * A.s_stride[2], A.dtype);
+        } else if (prev_passes_tokens && k >= Wi) {
+            const int t = k - Wi;  // evicted by cascade 0 after it had been placed there in this call
+            src = -1 - t;
+            score = load_as_float(A.s, n * A.s_stride[0] + h * A.s_stride[1] + (int64_t)t * A.s_stride[2], A.dtype);
+        } else {
+            int ring = sx_prev + k;
+            if (ring >= Wi) ring -= Wi;
+            src = l - Wi + ring;
+            score = load_as_float(A.cache_s, cs_base + (int64_t)src * A.cache_s_stride[2], A.dtype);
+        }
+    };
+    auto point = [&](int src, int dst) {  // the arrival that came from `src` ends up in slot dst (-1: nowhere)
+        if (src < 0) first[-1 - src] = dst;
+        else next_of[src] = dst;
+    };
+    if (part == 0 && tid == 0) {
+        int sx_new = c.sx + (int)(c.E % Wi);
+        if (sx_new >= Wi) sx_new -= Wi;
+        p.start_new[bh * C + i] = sx_new;
+        // arrivals before the first insert challenge the newest entry earlier calls left
+        const int lead_n = c.kf < c.nA ? c.kf : c.nA;
+        if (lead_n > 0) {
+            const int p_lead = l + (c.sx == 0 ? Wi - 1 : c.sx - 1);
+            int ws = p_lead;
+            float wv = load_as_float(A.cache_s, cs_base + (int64_t)p_lead * A.cache_s_stride[2], A.dtype);
+            bool held = true;  // the old entry still holds the slot
+            for (int k = 0; k < lead_n; k++) {
+                int src;
+                float score;
+                arrival(k, src, score);
+                if (score >= wv) {
+                    if (!held) point(ws, -1);
+                    held = false;
+                    ws = src;
+                    wv = score;
+                } else {
+                    point(src, -1);
+                }
+            }
+            // with W inserts in the call the slot is taken again by the last of them (only behind the last
+            // cascade: elsewhere such a call is left to the general kernel), and the group's winner is dropped
+            const bool survives = c.E <= Wi - 1;
+            if (!held) {
+                if (survives) {
+                    point(ws, p_lead);
+                    next_of[p_lead] = -1;  // the old entry is dropped
+                } else {
+                    point(ws, -1);
+                }
+            }
+        }
+    }
+    const int drop_before = c.E > Wi ? c.E - Wi : 0;  // inserts whose slot is taken again later in the call
+    for (int g = part * kSteadyThreads + tid; g < c.E; g += kSteadyParts * kSteadyThreads) {
+        const int k0 = c.kf + (int)((int64_t)g * c.r);
+        int k1 = k0 + (int)c.r;
+        if (k1 > c.nA) k1 = c.nA;
+        if (g < drop_before) {
+            // placed and pushed out again within the call: cascade 1 owns the pointer (it sees the token as an
+            // arrival of its own); behind the last cascade the members are dropped
+            if (i + 1 >= C) {
+                for (int k = k0; k < k1; k++) {
+                    int src;
+                    float score;
+                    arrival(k, src, score);
+                    point(src, -1);
+                }
+            }
+            continue;
+        }
+        int ring = c.sx + (g % Wi);
+        if (ring >= Wi) ring -= Wi;
+        const int phys = l + ring;
+        int ws;
+        float wv;
+        arrival(k0, ws, wv);
+        for (int k = k0 + 1; k < k1; k++) {
+            int src;
+            float score;
+            arrival(k, src, score);
+            if (score >= wv) {
+                point(ws, -1);
+                ws = src;
+                wv = score;
+            } else {
+                point(src, -1);
+            }
+        }
+        point(ws, phys);
+        if (i + 1 >= C) next_of[phys] = -1;  // what the last cascade evicts is dropped
+    }
+}
+
 // The plan of a single incoming token (the decode step): one wavefront per (batch, kv head), no workgroup
 // barriers.  Lane i fetches what cascade i may need (trackers, period, the scores of its oldest and its newest
 // slot) so that all cascades' loads travel together; the walk over the cascades then runs on values handed
@@ -321,6 +537,7 @@ __global__ void __launch_bounds__(CKV_WAVE) ckv_update_plan1_kernel(UpdateParams
             newest = load_as_float(A.cache_s, cs_base + (l + (sx - 1 + st) % st) * A.cache_s_stride[2], A.dtype);
         }
     }
+    if (lane == 0) p.mode[bh] = 0;  // the trackers are written here, not left in scratch
     if (sinks0 < NS) {  // the token is a sink (cascading_cache.py:399-431): no position pass
         if (lane == 0) {
             first[0] = (int32_t)(S + sinks0);
@@ -393,18 +610,22 @@ __device__ inline void update_positions_block(const UpdateParams& p, int blk) {
     const int i = blk / per_c, j0 = (blk % per_c) * kPosChunk;
     const int64_t* g_stored = A.stored_tokens + n * A.tracker_stride[0] + h * A.tracker_stride[1];
     const int64_t* g_start = A.start_indices + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+    // a unit planned by the steady-state kernel: every cascade is full, and the ring starts after the call are
+    // still in scratch (this launch commits them, so the trackers themselves are not read here)
+    const bool steady = p.mode[bh] != 0;
     int64_t ub = 0;
-    for (int c = 0; c < C; c++) ub += g_stored[c * A.tracker_stride[2]];
+    for (int c = 0; c < C; c++) ub += steady ? (int64_t)W : g_stored[c * A.tracker_stride[2]];
     // cascade i is written only if every earlier one holds tokens and ids are left
     for (int c = 0; c < i; c++) {
-        if (g_stored[c * A.tracker_stride[2]] <= 0) return;
+        if (!steady && g_stored[c * A.tracker_stride[2]] <= 0) return;
         ub -= W;
         if (ub <= 0) return;
     }
-    const int64_t st = g_stored[i * A.tracker_stride[2]];
+    const int64_t st = steady ? (int64_t)W : g_stored[i * A.tracker_stride[2]];
     const uint32_t seg = (uint32_t)(st < W ? st : W);
     if (seg == 0) return;
-    const uint32_t add = seg - (uint32_t)g_start[i * A.tracker_stride[2]];  // start < seg or start == 0
+    const uint32_t sx_now = steady ? (uint32_t)p.start_new[bh * C + i] : (uint32_t)g_start[i * A.tracker_stride[2]];
+    const uint32_t add = seg - sx_now;  // start < seg or start == 0
     const int64_t base = ub - seg;
     auto id_of = [&](int j) -> int64_t {
         uint32_t x = (uint32_t)j + add;
@@ -434,6 +655,12 @@ template <int LANES>
 __global__ void ckv_update_apply_vec_kernel(UpdateParams p) {
     const ckv_update_args& A = p.a;
     constexpr int kGroups = 256 / LANES;
+    if (blockIdx.x == 0 && p.do_pos && p.mode[blockIdx.y] && (int)threadIdx.x < A.cascades) {
+        // commit the ring starts the steady-state plan left in scratch (nobody reads the trackers in this launch)
+        const int64_t bh_c = blockIdx.y;
+        A.start_indices[(bh_c / A.H) * A.tracker_stride[0] + (bh_c % A.H) * A.tracker_stride[1] +
+                        threadIdx.x * A.tracker_stride[2]] = p.start_new[bh_c * A.cascades + threadIdx.x];
+    }
     if ((int)blockIdx.x >= p.apply_blocks) {
         update_positions_block(p, (int)blockIdx.x - p.apply_blocks);
         return;
@@ -499,7 +726,7 @@ __global__ void ckv_update_apply_vec_kernel(UpdateParams p) {
     // each other, served by the L2 the plan kernel has just written them to); then every displaced row of
     // the stretch is requested at once, so the rows cost one trip to memory instead of one per hop; then
     // the stretch is written: slot 0 takes the carried row, slot j the row displaced from slot j - 1.
-    constexpr int kHops = 8;
+    constexpr int kHops = 4;
     for (int round = 0; round * kHops <= A.cascades; round++) {  // a chain visits each cascade at most once
         int sl[kHops];
         int nx = d;
@@ -565,6 +792,12 @@ template <typename U>
 __global__ void ckv_update_apply_elem_kernel(UpdateParams p) {
     const ckv_update_args& A = p.a;
     constexpr int kPerLane = 8;
+    if (blockIdx.x == 0 && p.do_pos && p.mode[blockIdx.y] && (int)threadIdx.x < A.cascades) {
+        // commit the ring starts the steady-state plan left in scratch (nobody reads the trackers in this launch)
+        const int64_t bh_c = blockIdx.y;
+        A.start_indices[(bh_c / A.H) * A.tracker_stride[0] + (bh_c % A.H) * A.tracker_stride[1] +
+                        threadIdx.x * A.tracker_stride[2]] = p.start_new[bh_c * A.cascades + threadIdx.x];
+    }
     if ((int)blockIdx.x >= p.apply_blocks) {
         update_positions_block(p, (int)blockIdx.x - p.apply_blocks);
         return;
@@ -662,7 +895,7 @@ __global__ void ckv_update_apply_elem_kernel(UpdateParams p) {
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline size_t plan_lds_bytes(int cap) {
-    return (size_t)cap * 32 + (size_t)(cap + 1) * 8 + kMaxCascades * 20 + 64 * sizeof(int) + 64;
+    return (size_t)cap * 24 + (size_t)(cap + 1) * 8 + (size_t)(cap + 2) * 4 + kMaxCascades * 20 + 64 * sizeof(int) + 64;
 }
 
 }  // namespace
@@ -670,10 +903,11 @@ inline size_t plan_lds_bytes(int cap) {
 
 extern "C" int64_t ckv_update_workspace_bytes(int64_t N, int64_t H, int64_t K, int64_t max_seq_len,
                                               int32_t cascades) {
-    (void)cascades;
-    if (N <= 0 || H <= 0 || K < 0 || max_seq_len <= 0) return 0;
+    if (N <= 0 || H <= 0 || K < 0 || max_seq_len <= 0 || cascades <= 0) return 0;
+    // move chains (first, next_of), then per unit: position flag, plan mode, ring starts after the call
     return ckv::align_up(N * H * (K + max_seq_len) * (int64_t)sizeof(int32_t), 256) +
-           ckv::align_up(N * H * (int64_t)sizeof(int32_t), 256) + 256;
+           2 * ckv::align_up(N * H * (int64_t)sizeof(int32_t), 256) +
+           ckv::align_up(N * H * cascades * (int64_t)sizeof(int32_t), 256) + 256;
 }
 
 // Scratch of the entry point that allocates nothing (ckv_update_static): one array per device, part of the
@@ -705,6 +939,17 @@ int static_scratch(void** out) {
     return CKV_OK;
 }
 
+// launch with the stage's timing: events attached to the dispatch when single kernels are timed, else the
+// stream bracket of StageScope
+template <typename Kernel>
+void launch_timed(int stage, Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const UpdateParams& p) {
+    StageScope sc(stage, stream, true);
+    hipEvent_t ev0, ev1;
+    prof_kernel_events(stage, &ev0, &ev1);
+    if (ev0) hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, stream, ev0, ev1, 0u, p);
+    else hipLaunchKernelGGL(kernel, grid, block, lds, stream, p);
+}
+
 int run_update(const ckv_update_args& A, void* workspace, hipStream_t stream) {
     const int es = (int)elem_bytes(A.dtype);
     const bool vec = A.kv_stride[3] == 1 && A.cache_stride[3] == 1 && (A.num_sink == 0 || A.sink_stride[3] == 1) &&
@@ -721,7 +966,7 @@ int run_update(const ckv_update_args& A, void* workspace, hipStream_t stream) {
     DeviceInfo di;
     if (int rc = current_device_info(&di)) return rc;
     const int lds_max = di.lds_max;
-    int qmax = (int)((lds_max - 4096) / 40);
+    int qmax = (int)((lds_max - 4096) / 36);
     qmax = qmax / 64 * 64;
     if (qmax > kPlanMaxTokens) qmax = kPlanMaxTokens;
     if (qmax < 64) return CKV_ERR_UNSUPPORTED;
@@ -732,24 +977,34 @@ int run_update(const ckv_update_args& A, void* workspace, hipStream_t stream) {
     p.next_of = p.first + A.N * A.H * A.K;
     p.pos_flag = reinterpret_cast<int32_t*>(reinterpret_cast<char*>(workspace) +
                                             align_up(A.N * A.H * (A.K + A.max_seq_len) * (int64_t)sizeof(int32_t), 256));
+    p.mode = p.pos_flag + align_up(A.N * A.H * (int64_t)sizeof(int32_t), 256) / 4;
+    p.start_new = p.mode + align_up(A.N * A.H * (int64_t)sizeof(int32_t), 256) / 4;
+    p.token_offset = 0;
+    p.k_sub = 0;
+    p.do_pos = 0;
+    p.apply_blocks = 0;
+    if (A.K >= 2) {
+        // every unit first gets the chance of the steady-state plan (whole call, all cascades side by side); it
+        // marks the units it has planned, the general kernel below takes the others
+        launch_timed(CKV_STAGE_PLAN, ckv_update_plan_steady_kernel,
+                     dim3((unsigned)(A.cascades * kSteadyParts), (unsigned)(A.N * A.H)), dim3(kSteadyThreads), 0, stream, p);
+        CKV_HIP_TRY(hipGetLastError());
+    }
 
     for (int64_t off = 0; off < A.K; off += qmax) {
         const int ksub = (int)((A.K - off < qmax) ? (A.K - off) : qmax);
         p.token_offset = off;
         p.k_sub = ksub;
         p.do_pos = (off + ksub == A.K) ? 1 : 0;
-        if (ksub == 1) {  // the decode step: one wavefront per unit
-            StageScope sc(CKV_STAGE_PLAN, stream);
-            hipLaunchKernelGGL(ckv_update_plan1_kernel, dim3((unsigned)(A.N * A.H)), dim3(CKV_WAVE), 0, stream, p);
+        if (A.K == 1) {  // the decode step: one wavefront per unit
+            launch_timed(CKV_STAGE_PLAN, ckv_update_plan1_kernel, dim3((unsigned)(A.N * A.H)), dim3(CKV_WAVE), 0, stream, p);
         } else {
             const int T = ksub <= 256 ? 256 : 1024;  // few tokens: a small block plans them
             const size_t lds = plan_lds_bytes(ksub);
             if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(ckv_update_plan_kernel), (int)lds)) return rc;
-            StageScope sc(CKV_STAGE_PLAN, stream);
-            hipLaunchKernelGGL(ckv_update_plan_kernel, dim3((unsigned)(A.N * A.H)), dim3(T), lds, stream, p);
+            launch_timed(CKV_STAGE_PLAN, ckv_update_plan_kernel, dim3((unsigned)(A.N * A.H)), dim3(T), lds, stream, p);
         }
         CKV_HIP_TRY(hipGetLastError());
-        StageScope sc_apply(CKV_STAGE_APPLY, stream);
         // the position ids of the last launch of a call are written by extra blocks of the apply grid
         const unsigned pos_blocks =
             p.do_pos ? (unsigned)(((A.window_size + kPosChunk - 1) / kPosChunk) * A.cascades) : 0u;
@@ -762,22 +1017,22 @@ int run_update(const ckv_update_args& A, void* workspace, hipStream_t stream) {
             p.apply_blocks = (ksub + 256 / lanes - 1) / (256 / lanes);
             const dim3 grid((unsigned)p.apply_blocks + pos_blocks, (unsigned)(A.N * A.H));
             switch (lanes) {
-                case 1: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<1>, grid, block, 0, stream, p); break;
-                case 2: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<2>, grid, block, 0, stream, p); break;
-                case 4: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<4>, grid, block, 0, stream, p); break;
-                case 8: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<8>, grid, block, 0, stream, p); break;
-                case 16: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<16>, grid, block, 0, stream, p); break;
-                case 32: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<32>, grid, block, 0, stream, p); break;
-                default: hipLaunchKernelGGL(ckv_update_apply_vec_kernel<64>, grid, block, 0, stream, p); break;
+                case 1: launch_timed(CKV_STAGE_APPLY, ckv_update_apply_vec_kernel<1>, grid, block, 0, stream, p); break;
+                case 2: launch_timed(CKV_STAGE_APPLY, ckv_update_apply_vec_kernel<2>, grid, block, 0, stream, p); break;
+                case 4: launch_timed(CKV_STAGE_APPLY, ckv_update_apply_vec_kernel<4>, grid, block, 0, stream, p); break;
+                case 8: launch_timed(CKV_STAGE_APPLY, ckv_update_apply_vec_kernel<8>, grid, block, 0, stream, p); break;
+                case 16: launch_timed(CKV_STAGE_APPLY, ckv_update_apply_vec_kernel<16>, grid, block, 0, stream, p); break;
+                case 32: launch_timed(CKV_STAGE_APPLY, ckv_update_apply_vec_kernel<32>, grid, block, 0, stream, p); break;
+                default: launch_timed(CKV_STAGE_APPLY, ckv_update_apply_vec_kernel<64>, grid, block, 0, stream, p); break;
             }
         } else {
             const dim3 block(256);
             p.apply_blocks = (ksub + 3) / 4;
             const dim3 grid((unsigned)p.apply_blocks + pos_blocks, (unsigned)(A.N * A.H));
             if (es == 4) {
-                hipLaunchKernelGGL(ckv_update_apply_elem_kernel<uint32_t>, grid, block, 0, stream, p);
+                launch_timed(CKV_STAGE_APPLY, ckv_update_apply_elem_kernel<uint32_t>, grid, block, 0, stream, p);
             } else {
-                hipLaunchKernelGGL(ckv_update_apply_elem_kernel<uint16_t>, grid, block, 0, stream, p);
+                launch_timed(CKV_STAGE_APPLY, ckv_update_apply_elem_kernel<uint16_t>, grid, block, 0, stream, p);
             }
         }
         CKV_HIP_TRY(hipGetLastError());

@@ -262,8 +262,10 @@ typedef enum ckv_stage {
     CKV_STAGE_COUNT = 8
 } ckv_stage;
 
-/* on: 0 = off, 1 = every stage, 2 = only the attention main kernels (CKV_STAGE_FWD, CKV_STAGE_DECODE):
- * two event records per call instead of a dozen, for timing inside a throughput measurement */
+/* on: 0 = off, 1 = every stage bracketed by event records in the stream, 2 = only the attention main kernels
+ * (CKV_STAGE_FWD, CKV_STAGE_DECODE), 3 = only the kernels of the cache update (CKV_STAGE_PLAN, CKV_STAGE_APPLY).
+ * Levels 2 and 3 attach the events to the kernels' own dispatches: nothing is put between a kernel and its
+ * neighbours, and the figures are kernel durations, fit for timing inside a throughput measurement. */
 int ckv_profile_enable(int on);                       /* returns the previous setting */
 int ckv_profile_read(double* ms, int64_t* launches);  /* both arrays CKV_STAGE_COUNT long */
 

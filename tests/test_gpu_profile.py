@@ -47,8 +47,20 @@ def test_every_stage():
     st = _run(1)
     assert st["fwd"][1] == 3 and st["scores"][1] == 3 and st["finish"][1] == 3
     assert st["decode"][1] == 4 and st["decode_tail"][1] == 4
-    assert st["prep"][1] == 7 and st["plan"][1] == 7 and st["apply"][1] == 7
+    # a chunk's update is planned by two launches (the steady-state kernel, then the general one for the units it
+    # left), a single token's by one
+    assert st["prep"][1] == 7 and st["plan"][1] == 3 * 2 + 4 and st["apply"][1] == 7
     assert all(ms > 0.0 for ms, n in st.values())
+
+
+def test_update_kernels_only():
+    """Level 3: the kernels of the cache update, each timed on its own dispatch, nothing else."""
+    st = _run(3)
+    assert st["plan"][1] == 3 * 2 + 4 and st["apply"][1] == 7
+    assert 0.0 < st["plan"][0] < 100.0 and 0.0 < st["apply"][0] < 100.0
+    for name, (ms, n) in st.items():
+        if name not in ("plan", "apply"):
+            assert n == 0 and ms == 0.0, name
 
 
 def test_off_records_nothing():
