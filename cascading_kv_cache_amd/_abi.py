@@ -84,6 +84,23 @@ class DenseArgs(C.Structure):
         ("beta", C.c_double),
         ("causal", C.c_int32), ("dtype", C.c_int32),
         ("workspace", VP), ("workspace_bytes", I64),
+        ("lse", VP),
+    ]
+
+
+class DenseBwdArgs(C.Structure):
+    _fields_ = [
+        ("q", VP), ("q_stride", I64 * 4),
+        ("k", VP), ("v", VP), ("kv_stride", I64 * 4),
+        ("mask", VP),
+        ("out", VP), ("out_stride", I64 * 4),
+        ("lse", VP),
+        ("dout", VP), ("dout_stride", I64 * 4),
+        ("dq", VP), ("dq_stride", I64 * 4),
+        ("dk", VP), ("dv", VP), ("dkv_stride", I64 * 4),
+        ("B", I64), ("H", I64), ("n_ctx", I64), ("n_kv", I64), ("D", I64),
+        ("scale", C.c_float), ("dtype", C.c_int32),
+        ("workspace", VP), ("workspace_bytes", I64),
     ]
 
 
@@ -219,6 +236,10 @@ def lib():
         L.ckv_attn_dense.restype = C.c_int
         L.ckv_dense_workspace_bytes.argtypes = [I64, I64, I64, I64, I64, C.c_int32]
         L.ckv_dense_workspace_bytes.restype = I64
+        L.ckv_attn_dense_bwd.argtypes = [C.POINTER(DenseBwdArgs), VP]
+        L.ckv_attn_dense_bwd.restype = C.c_int
+        L.ckv_dense_bwd_workspace_bytes.argtypes = [I64, I64, I64]
+        L.ckv_dense_bwd_workspace_bytes.restype = I64
         L.ckv_chunk_positions.argtypes = [C.c_void_p, I64, I64, C.c_void_p, I64, I64, C.c_void_p, C.c_void_p]
         L.ckv_chunk_positions.restype = C.c_int
         L.ckv_profile_enable.argtypes = [C.c_int]

@@ -218,3 +218,4 @@ extern "C" int ckv_abi_version(void) { return CKV_ABI_VERSION; }
 extern "C" int64_t ckv_sizeof_update_args(void) { return (int64_t)sizeof(ckv_update_args); }
 extern "C" int64_t ckv_sizeof_attn_args(void) { return (int64_t)sizeof(ckv_attn_args); }
 extern "C" int64_t ckv_sizeof_dense_args(void) { return (int64_t)sizeof(ckv_dense_args); }
+extern "C" int64_t ckv_sizeof_dense_bwd_args(void) { return (int64_t)sizeof(ckv_dense_bwd_args); }

@@ -240,10 +240,14 @@ extern "C" int ckv_attn_dense(const ckv_dense_args* args, void* stream_) {
             rc = launch_cast_scores(w.colsum, a.scores, a.scores_stride, a.B, a.H, a.n_kv, a.dtype, stream);
             if (rc) return rc;
         }
+        if (a.lse) {
+            CKV_HIP_TRY(hipMemcpyAsync(a.lse, w.lse, a.B * a.H * a.n_ctx * sizeof(float), hipMemcpyDeviceToDevice, stream));
+        }
         return CKV_OK;
     }
     Carver c(a.workspace);
     float* lse = (float*)c.take(a.B * a.H * a.n_ctx * 4);
+    if (a.lse) lse = a.lse;  // the forward kernel writes the caller's array directly
     float* colsum = (float*)c.take(a.B * a.H * a.n_kv * 4);
     float* w_ema = (float*)c.take((a.n_ctx + kColSlack) * 4);
     float* w_new = (float*)c.take(a.n_ctx * 4);

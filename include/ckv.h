@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define CKV_ABI_VERSION 1
+#define CKV_ABI_VERSION 2
 
 typedef enum ckv_dtype {
     CKV_F32 = 0,
@@ -225,12 +225,48 @@ typedef struct ckv_dense_args {
     int32_t dtype;
     void* workspace;
     int64_t workspace_bytes;
+    float* lse;                    /* optional (B, H, n_ctx) contiguous: natural-log row normalisers, what the
+                                      backward pass needs (the reference keeps M, flash_attention.py:272-276) */
 } ckv_dense_args;
 
 int64_t ckv_dense_workspace_bytes(int64_t B, int64_t H, int64_t n_ctx, int64_t n_kv, int64_t D,
                                   int32_t dtype);
 
 int ckv_attn_dense(const ckv_dense_args* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Backward of ckv_attn_dense: replaces _attention.backward -> _attn_bwd_preprocess / _attn_bwd
+ * (flash_attention.py:279-537, 654-710).  Given the forward's inputs, its output and row normalisers and the
+ * gradient of the output, writes dq, dk, dv (dtype and shapes of q, k, v); the scores carry no gradient, as
+ * in the reference.  Masked cached keys receive zero gradients.  head_dim up to 192.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct ckv_dense_bwd_args {
+    const void* q;                 /* (B, H, n_ctx, D) */
+    int64_t q_stride[4];
+    const void* k;                 /* (B, H, n_kv, D)  */
+    const void* v;
+    int64_t kv_stride[4];
+    const uint8_t* mask;           /* (n_kv - n_ctx,) bool, 1 = masked; may be NULL if that is 0 */
+    const void* out;               /* (B, H, n_ctx, D) forward output */
+    int64_t out_stride[4];
+    const float* lse;              /* (B, H, n_ctx) contiguous, from ckv_dense_args.lse */
+    const void* dout;              /* (B, H, n_ctx, D) gradient of out */
+    int64_t dout_stride[4];
+    void* dq;                      /* (B, H, n_ctx, D) */
+    int64_t dq_stride[4];
+    void* dk;                      /* (B, H, n_kv, D)  */
+    void* dv;
+    int64_t dkv_stride[4];
+    int64_t B, H, n_ctx, n_kv, D;
+    float scale;
+    int32_t dtype;
+    void* workspace;
+    int64_t workspace_bytes;
+} ckv_dense_bwd_args;
+
+int64_t ckv_dense_bwd_workspace_bytes(int64_t B, int64_t H, int64_t n_ctx);
+
+int ckv_attn_dense_bwd(const ckv_dense_bwd_args* args, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Position ids of an incoming chunk (cascade_attention.py:114-150): q_pos[i] = i on the first call

@@ -32,7 +32,8 @@ def test_header_declares_the_expected_entry_points():
     names = declared_functions()
     for must in ("ckv_update", "ckv_update_workspace_bytes", "ckv_attn", "ckv_attn_workspace_bytes", "ckv_attn_dense",
                  "ckv_dense_workspace_bytes", "ckv_strerror", "ckv_abi_version", "ckv_profile_enable",
-                 "ckv_profile_read", "ckv_chunk_positions"):
+                 "ckv_profile_read", "ckv_chunk_positions", "ckv_update_static", "ckv_attn_dense_bwd",
+                 "ckv_dense_bwd_workspace_bytes"):
         assert must in names
 
 
@@ -40,13 +41,13 @@ def test_library_exports_every_declared_symbol(lib):
     raw = C.CDLL(_abi.LIB_PATH)
     for name in declared_functions():
         assert hasattr(raw, name), f"{name} is declared in include/ckv.h but not exported"
-    assert lib.ckv_abi_version() == 1
+    assert lib.ckv_abi_version() == 2
 
 
 def test_ctypes_mirrors_match_struct_sizes(lib):
     raw = C.CDLL(_abi.LIB_PATH)
     for fn, struct in (("ckv_sizeof_update_args", _abi.UpdateArgs), ("ckv_sizeof_attn_args", _abi.AttnArgs),
-                       ("ckv_sizeof_dense_args", _abi.DenseArgs)):
+                       ("ckv_sizeof_dense_args", _abi.DenseArgs), ("ckv_sizeof_dense_bwd_args", _abi.DenseBwdArgs)):
         f = getattr(raw, fn)
         f.restype = C.c_int64
         assert f() == C.sizeof(struct), fn
@@ -105,6 +106,16 @@ def test_attention_argument_validation_needs_no_gpu(lib):
     d.dtype = _abi.CKV_F16
     d.B, d.H, d.n_ctx, d.n_kv, d.D = 1, 1, 16, 8, 64
     assert lib.ckv_attn_dense(C.byref(d), None) == -2
+    assert lib.ckv_attn_dense_bwd(None, None) == -1
+    g = _abi.DenseBwdArgs()
+    g.dtype = _abi.CKV_F16
+    g.B, g.H, g.n_ctx, g.n_kv, g.D = 1, 1, 16, 8, 64
+    assert lib.ckv_attn_dense_bwd(C.byref(g), None) == -2    # fewer keys than queries
+    g.n_kv, g.D = 32, 256
+    assert lib.ckv_attn_dense_bwd(C.byref(g), None) == -6    # head size beyond what the backward kernels tile
+    g.D = 64
+    assert lib.ckv_attn_dense_bwd(C.byref(g), None) == -1    # tensors missing
+    assert lib.ckv_dense_bwd_workspace_bytes(2, 4, 100) >= 2 * 4 * 100 * 4
 
 
 def test_fill_update_args_enforces_reference_preconditions():

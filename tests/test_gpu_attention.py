@@ -316,3 +316,54 @@ def test_attention_rejects_cpu_tensors():
     q = torch.zeros(1, 1, 16, 64)
     with pytest.raises(_abi.CkvError):
         attention(q, q, q, True, 1.0, torch.zeros(0, dtype=torch.bool), 0.9)
+
+
+@pytest.mark.parametrize("Z,H,N_CTX,N_KV,HEAD_DIM", [
+    (1, 2, 128, 128, 64), (1, 2, 256, 256, 64), (1, 2, 512, 512, 64), (1, 1, 128, 128 + 128, 64),
+    (1, 2, 1024, 16384 + 1024, 64), (2, 32, 1024, 16384 + 1024, 128), (1, 2, 512, 2560, 64),
+    (1, 2, 500, 2048 + 500, 64), (1, 2, 500, 2048 + 64 + 500, 64), (2, 3, 77, 300 + 77, 32),
+])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_dense_operator_backward(Z, H, N_CTX, N_KV, HEAD_DIM, dtype):
+    """The backward half of cascade/models/test.py:177-269: seed 20, N(0, 0.5) inputs, sm_scale 0.5, random cache
+    mask; dq, dk, dv of the operator against autograd through the dense formula (softmax in float32, then the
+    product with v in the tensor dtype), atol 1e-2 in float16 as in the reference's test, 1e-4 in float32, 2e-2 in
+    bfloat16 plus two units in the last place of the value (gradients of a key seen by hundreds of rows reach
+    magnitudes of 4 to 8, where neighbouring bfloat16 values are 3e-2 apart, and the reference formula rounds P
+    and the products to bfloat16 where the kernels round once)."""
+    from cascading_kv_cache_amd.flash_attention import attention
+
+    if dtype != torch.float16 and Z * H * N_KV > 300000:
+        pytest.skip("the largest shape runs in float16 only, like the reference's test")
+    torch.manual_seed(20)
+    q = torch.empty((Z, H, N_CTX, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
+    k = torch.empty((Z, H, N_KV, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
+    v = torch.empty((Z, H, N_KV, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
+    mask = torch.rand(N_KV - N_CTX, device="cuda") > 0.5
+    full = torch.cat((mask[None, :].expand(N_CTX, -1),
+                      torch.ones(N_CTX, N_CTX, dtype=torch.bool, device="cuda").triu(1)), dim=-1)
+    sm_scale = 0.5
+    dout = torch.randn_like(q)
+    p = torch.matmul(q, k.transpose(2, 3)) * sm_scale
+    p = p.masked_fill(full, float("-inf"))
+    p = torch.softmax(p.float(), dim=-1).to(dtype)
+    ref_out = torch.matmul(p, v).to(dtype)
+    ref_out.backward(dout)
+    ref_dv, v.grad = v.grad.clone(), None
+    ref_dk, k.grad = k.grad.clone(), None
+    ref_dq, q.grad = q.grad.clone(), None
+    del p
+    out, scores = attention(q, k, v, True, sm_scale, mask, 1.0)
+    assert not scores.requires_grad
+    atol = {torch.float32: 1e-4, torch.float16: 1e-2, torch.bfloat16: 2e-2}[dtype]
+    assert (out.float() - ref_out.float()).abs().max().item() <= atol
+    out.backward(dout, None)
+    for name, got, want in (("dv", v.grad, ref_dv), ("dk", k.grad, ref_dk), ("dq", q.grad, ref_dq)):
+        assert got.shape == want.shape and got.dtype == want.dtype
+        rtol = 2.0 ** -6 if dtype == torch.bfloat16 else 0.0
+        excess = ((got.float() - want.float()).abs() - rtol * want.float().abs()).max().item()
+        assert excess <= atol, f"{name}: error exceeds the relative allowance by {excess:.3e}"
+    # a masked slot receives no gradient at all
+    if int(mask.sum()) > 0:
+        assert k.grad[:, :, : N_KV - N_CTX][:, :, mask].abs().max().item() == 0.0
+        assert v.grad[:, :, : N_KV - N_CTX][:, :, mask].abs().max().item() == 0.0
