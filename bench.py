@@ -13,7 +13,9 @@ the dense bf16 MFMA peak from HIP-event timings of that kernel's own dispatch in
 sub-records carry their own roofline: `decode` (the single-token steps of the headline workload against HBM
 bandwidth), `update` (the cache update of the headline chunk against HBM bandwidth, bytes counted from the
 state difference), `cfg2_prefill` (B=2, 8 x 2048 slots, 2048-token chunks) and `cfg3_decode` (B=16,
-4 x 8192 slots, one token).  `cpu_baseline` times the CPU oracle (the reference's eager PyTorch path restated,
+4 x 8192 slots, one token) and `cfg4_full_model` (the whole 32-layer Llama-3.1-8B-shape decoder with random weights:
+131072 prompt tokens in 4096-token strides, then 256 greedy tokens; `--only cfg5` runs the Qwen2-7B-shape workload
+the same way).  `cpu_baseline` times the CPU oracle (the reference's eager PyTorch path restated,
 plus the serial update) on a bounded sample of the headline workload on the box's host cores.
 """
 import argparse
@@ -38,6 +40,9 @@ LAYER = dict(name="llama3.1-8b layer, 64K window", B=1, H=32, KVH=8, D=128, NS=6
              seed=4, decode_per_chunk=8)
 CFG2 = dict(name="cfg2", B=2, H=32, KVH=8, D=128, NS=64, S=16384, C=8, Q=2048, theta=5e5, seed=2)
 CFG3 = dict(name="cfg3", B=16, H=32, KVH=8, D=128, NS=64, S=32768, C=4, Q=1, theta=5e5, seed=3)
+# whole decoders with random weights: every layer through the library, everything else plain torch
+MODEL4 = dict(name="cfg4", preset="llama3.1-8b", B=1, prompt=131072, stride=4096, window=65536, cascades=8, new=256, seed=4)
+MODEL5 = dict(name="cfg5", preset="qwen2-7b", B=4, prompt=262144, stride=4096, window=32768, cascades=16, new=0, seed=5)
 
 STATE = ("key_cache", "value_cache", "score_cache", "sink_keys", "sink_values", "mask", "sink_mask", "pos", "og_pos",
          "sink_pos", "stored_tokens", "start_indices", "stored_sinks")
@@ -103,6 +108,13 @@ def fill_to_steady_state(cache, cfg, pool, inv_freq):
         i += 1
     torch.cuda.synchronize()
     assert int(cache.mask[0].sum()) == 0, "cache must be full before the timed region"
+
+
+def update_traffic(workload, single_token=False):
+    """Measured HBM bytes of one cache update: the sum over its launches (None when any figure is stale)."""
+    names = ["ckv_update_plan1_kernel"] if single_token else ["ckv_update_plan_steady_kernel", "ckv_update_plan_kernel"]
+    parts = [measured_traffic(k, workload) for k in names + ["ckv_update_apply_vec_kernel"]]
+    return None if any(x is None for x in parts) else sum(parts)
 
 
 def prefill_flops(cfg):
@@ -288,8 +300,10 @@ def run_layer(steps, warmup, dtype, device):
         update=dict(workload="cache update of one 4096-token chunk into the full headline cache",
                     roofline=dict(bound="hbm", achieved=ubytes / (upd_ms * 1e-3) / 1e9 if upd_ms else 0.0,
                                   peak=PEAK_HBM_GBPS, unit="GB/s",
-                                  frac=ubytes / (upd_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS if upd_ms else 0.0, traffic=None,
-                                  kernel="ckv_update_plan_kernel + ckv_update_apply_vec_kernel", kernel_ms=upd_ms,
+                                  frac=ubytes / (upd_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS if upd_ms else 0.0,
+                                  traffic=update_traffic("layer64k"),
+                                  kernel="ckv_update_plan_steady_kernel + ckv_update_plan_kernel + ckv_update_apply_vec_kernel",
+                                  kernel_ms=upd_ms,
                                   algorithmic_gb_per_launch=ubytes / 1e9), **ucount),
     )
     return res, cache, pool
@@ -342,7 +356,7 @@ def run_cfg2(steps, warmup, dtype, device):
         if attn_ms else None,
         update_roofline=dict(bound="hbm", achieved=ubytes / (upd_ms * 1e-3) / 1e9 if upd_ms else 0.0, peak=PEAK_HBM_GBPS,
                              unit="GB/s", frac=ubytes / (upd_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS if upd_ms else 0.0,
-                             traffic=None, kernel_ms=upd_ms, algorithmic_gb_per_launch=ubytes / 1e9, **ucount),
+                             traffic=update_traffic("cfg2"), kernel_ms=upd_ms, algorithmic_gb_per_launch=ubytes / 1e9, **ucount),
     )
 
 
@@ -417,8 +431,50 @@ def run_cfg3(steps, warmup, dtype, device):
         stage_ms=stages,
         update_roofline=dict(bound="hbm", achieved=ubytes / (upd_ms * 1e-3) / 1e9 if upd_ms else 0.0, peak=PEAK_HBM_GBPS,
                              unit="GB/s", frac=ubytes / (upd_ms * 1e-3) / 1e9 / PEAK_HBM_GBPS if upd_ms else 0.0,
-                             traffic=None, kernel_ms=upd_ms, algorithmic_gb_per_launch=ubytes / 1e9, **ucount),
+                             traffic=update_traffic("cfg3", single_token=True), kernel_ms=upd_ms, algorithmic_gb_per_launch=ubytes / 1e9, **ucount),
     )
+
+
+def run_model(cfg, device, dtype, prompt=None):
+    """The full-model workloads: a random-weight decoder of the named shape streams uniform random token ids through
+    in strides and then decodes greedily, every attention layer on its own layer of one cascading cache.  One short
+    untimed pass (two strides, two tokens) warms the BLAS library, then the cache is reset and the whole stream
+    is timed."""
+    from cascading_kv_cache_amd.decoder import PRESETS, CascadeDecoder
+    mcfg = PRESETS[cfg["preset"]]
+    prompt = prompt or cfg["prompt"]
+    model = CascadeDecoder(mcfg, dtype=dtype, device=device, seed=cfg["seed"], init_on_device=True)
+    g = torch.Generator().manual_seed(cfg["seed"])
+    ids = torch.randint(0, mcfg.vocab_size, (cfg["B"], prompt), generator=g).to(device)
+    cache = model.new_cache(cfg["window"], cfg["cascades"], batch=cfg["B"])
+    stride = cfg["stride"]
+
+    def stream(n_prompt, n_new):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = None
+        for i in range(0, n_prompt, stride):
+            logits = model(ids[:, i:i + stride], cache)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(n_new):
+            logits = model(torch.argmax(logits[:, -1, :], dim=-1)[:, None], cache)
+        torch.cuda.synchronize()
+        return t1 - t0, time.perf_counter() - t1
+
+    with torch.no_grad():
+        stream(2 * stride, 2)
+        cache.reset(verbose=False)
+        tp, td = stream(prompt, cfg["new"])
+    n_p, n_d = cfg["B"] * prompt, cfg["B"] * cfg["new"]
+    rec = {"workload": f"{cfg['preset']} shape, {mcfg.num_layers} layers, random weights, B={cfg['B']}: {prompt} uniform random "
+                       f"token ids per stream in {stride}-token strides through sink 64 + {cfg['cascades']} x "
+                       f"{cfg['window'] // cfg['cascades']} slots, then {cfg['new']} greedy tokens",
+           "tokens_per_s": (n_p + n_d) / (tp + td), "prefill_tokens_per_s": n_p / tp, "prefill_s": tp,
+           "decode_tokens_per_s": (n_d / td) if n_d else None, "decode_ms_per_token": (td / cfg["new"] * 1e3) if n_d else None}
+    del model, cache, ids
+    torch.cuda.empty_cache()
+    return rec
 
 
 def host_threads():
@@ -507,7 +563,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sub", action="store_true", help="skip the cfg2 / cfg3 sub-records")
-    ap.add_argument("--only", choices=["layer", "cfg2", "cfg3"], default=None,
+    ap.add_argument("--no-model", action="store_true", help="skip the full-model record (cfg4)")
+    ap.add_argument("--model-prompt", type=int, default=None, help="shorter prompt for the full-model records")
+    ap.add_argument("--only", choices=["layer", "cfg2", "cfg3", "cfg4", "cfg5"], default=None,
                     help="run one workload only (for profiler runs); the JSON line then carries that record alone")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 512 MiB device copy, the known-size reference that scales the "
@@ -531,6 +589,9 @@ def main():
             dst.copy_(src)
             torch.cuda.synchronize()
 
+    if args.only in ("cfg4", "cfg5"):
+        print(json.dumps({args.only: run_model(MODEL4 if args.only == "cfg4" else MODEL5, device, dtype, args.model_prompt)}))
+        return
     if args.only in ("cfg2", "cfg3"):
         rec = (run_cfg2 if args.only == "cfg2" else run_cfg3)(max(args.steps, 3), args.warmup, dtype, device)
         calibrate()
@@ -545,6 +606,8 @@ def main():
     cfg2 = None if sub else run_cfg2(max(args.steps, 20), args.warmup, dtype, device)
     torch.cuda.empty_cache()
     cfg3 = None if sub else run_cfg3(max(args.steps, 20), args.warmup, dtype, device)
+    torch.cuda.empty_cache()
+    cfg4 = None if (sub or args.no_model) else run_model(MODEL4, device, dtype, args.model_prompt)
     calibrate()
     cfg = LAYER
     line = {
@@ -573,6 +636,7 @@ def main():
         "update": layer["update"],
         "cfg2_prefill": cfg2,
         "cfg3_decode": cfg3,
+        "cfg4_full_model": cfg4,
     }
     print(json.dumps(line))
 

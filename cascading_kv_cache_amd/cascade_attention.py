@@ -32,19 +32,22 @@ def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_p
     ``_stream``: raw stream handle when the caller already holds the device context."""
     _require_device(cache.key_cache[layer_idx], "the cache")
     dev = cache.key_cache[layer_idx].device
-    # Steady state of an eagerly filled cache: every token up to index S + num_sink was accepted by every
-    # cascade (cascading_cache.py:471-478), so from then on every slot holds a token, the largest position id
-    # is S - 1 plus the sink shift, and the chunk starts at S + num_sink whatever the stream does later.  The
-    # ids are then a constant vector, kept per length: no kernel, no device read.
+    # An eagerly filled cache drops no token before it is full: every token up to index S + num_sink is accepted by
+    # every cascade (cascading_cache.py:471-478), so sinks and slots together hold min(seen, S + num_sink) tokens,
+    # their ids are 0 .. that - 1 (stale entries of slots not yet filled are never larger: the position pass hands
+    # out ids below the number of stored tokens, cascading_cache.py:112-142), and the chunk starts one past them
+    # whatever the stream does later.  The ids are then a function of the host-side token counter: no kernel, no
+    # device read.  (This holds for every state the update itself produces from an empty cache.)
     S, NS = cache.max_seq_len[layer_idx], cache.num_sink_tokens
-    if not do_og_pos and cache.eager_fill and cache._seen_host[layer_idx] >= S + NS and S > 0:
+    if not do_og_pos and cache.eager_fill and S > 0:
+        start = min(int(cache._seen_host[layer_idx]), S + NS)
         memo = cache.__dict__.setdefault("_steady_q_pos", {})
-        key = (S + NS, q_len, dev)
+        key = (start, q_len, dev)
         ids = memo.get(key)
         if ids is None:
             if len(memo) > 16:
                 memo.clear()
-            ids = memo[key] = torch.arange(S + NS, S + NS + q_len, device=dev, dtype=torch.long)
+            ids = memo[key] = torch.arange(start, start + q_len, device=dev, dtype=torch.long)
         return ids
     out = torch.empty(q_len, device=dev, dtype=torch.long)
     key_ptr, n_key, shift, sink_ptr, n_sink = None, 0, 0, None, 0

@@ -88,19 +88,24 @@ class DecoderLayer(nn.Module):
 class CascadeDecoder(nn.Module):
     """Decoder-only model whose every layer attends through one :class:`CascadingKVCache`."""
 
-    def __init__(self, cfg: DecoderConfig, dtype=torch.bfloat16, device="cuda:0", seed=0):
+    def __init__(self, cfg: DecoderConfig, dtype=torch.bfloat16, device="cuda:0", seed=0, init_on_device=False):
+        """Weights are N(0, 0.02) from ``seed``: drawn on the CPU (the same bits whatever the device, what the parity
+        tests need) or, with ``init_on_device``, by the device's generator (seconds instead of minutes at 8B)."""
         super().__init__()
         self.cfg, self.dtype, self.device = cfg, dtype, device
         self.embed_tokens = nn.Embedding(cfg.vocab_size, cfg.hidden_size, dtype=dtype, device=device)
         self.layers = nn.ModuleList(DecoderLayer(cfg, i, dtype, device) for i in range(cfg.num_layers))
         self.norm = RMSNorm(cfg.hidden_size, cfg.rms_eps, dtype, device)
         self.lm_head = nn.Linear(cfg.hidden_size, cfg.vocab_size, bias=False, dtype=dtype, device=device)
-        gen = torch.Generator(device="cpu").manual_seed(seed)
-        with torch.no_grad():  # N(0, 0.02), seeded, whatever the device
+        gen = torch.Generator(device=device if init_on_device else "cpu").manual_seed(seed)
+        with torch.no_grad():
             for name, prm in self.named_parameters():
                 if name.endswith("layernorm.weight") or name == "norm.weight":
                     continue
-                prm.copy_((torch.randn(prm.shape, generator=gen) * 0.02).to(dtype))
+                if init_on_device:
+                    prm.normal_(0.0, 0.02, generator=gen)
+                else:
+                    prm.copy_((torch.randn(prm.shape, generator=gen) * 0.02).to(dtype))
 
     def new_cache(self, window, cascades, batch=1, num_sink_tokens=64, **kw):
         return CascadingKVCache(window // cascades, num_sink_tokens=num_sink_tokens, max_batch_size=batch,

@@ -249,14 +249,16 @@ def test_original_position_mode(dtype, D, H, KVH, Q, q_last):
         assert led.flips == 0, led.summary()
 
 
+@pytest.mark.parametrize("eager", [False, True])
 @pytest.mark.parametrize("do_og_pos", [False, True])
-def test_chunk_positions_kernel(do_og_pos):
-    """ckv_chunk_positions against the rule of cascade_attention.py:114-150: 0.. on the first call,
-    then one past the largest position id among sinks and slots (stale entries included)."""
+def test_chunk_positions_kernel(do_og_pos, eager):
+    """Position ids of a chunk against the rule of cascade_attention.py:114-150: 0.. on the first call,
+    then one past the largest position id among sinks and slots (stale entries included).  ckv_chunk_positions
+    computes them on the device; with eager fill (and compact ids) the host derives them from its token counter."""
     from cascading_kv_cache_amd.cascade_attention import chunk_positions
 
     B, KVH, D, NS, W, C = 2, 2, 32, 4, 16, 4
-    gpu, cpu = make_pair(B, KVH, D, NS, W, C, torch.float32)
+    gpu, cpu = make_pair(B, KVH, D, NS, W, C, torch.float32, eager=eager)
     gen = torch.Generator().manual_seed(3)
     assert torch.equal(chunk_positions(gpu, 0, 7, do_og_pos).cpu(), torch.arange(7))
     for n in (3, 9, 40, 1, 100):

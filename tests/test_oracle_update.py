@@ -153,6 +153,35 @@ def test_eager_fill_fills_everything():
     assert sorted(c.og_pos.view(-1).tolist()) == list(range(4, 20))
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_eager_fill_query_positions_follow_the_token_counter(seed):
+    """With eager fill nothing is dropped before the cache is full, so the id the next chunk starts at (one past the
+    largest id among sinks and slots, stale entries included, cascade_attention.py:119-150) is min(seen, S + NSINK):
+    what the host side hands out without reading the device."""
+    rng = random.Random(100 + seed)
+    NS = rng.choice([0, 1, 4, 7])
+    W = rng.choice([1, 2, 3, 4, 8])
+    C = rng.choice([1, 2, 3, 4, 5])
+    func = rng.choice(CASCADE_FUNCS)
+    c = OracleCache(window_length=W, num_sink_tokens=NS, max_batch_size=1, heads=2, dim=1, max_seq_len=W * C,
+                    cascade_func=func, eager_fill=True)
+    n = rng.randint(1, 6 * W * C + NS)
+    k = token_stream(n, heads=2)
+    g = torch.Generator().manual_seed(seed)
+    scores = torch.rand(1, 2, n, generator=g)
+    done = 0
+    while done < n:
+        q = rng.randint(1, 2 * W + 3)
+        c.update(k[:, :, done:done + q].contiguous(), k[:, :, done:done + q].clone(), scores[:, :, done:done + q].contiguous())
+        done = min(done + q, n)
+        seen = int(c.seen_tokens)
+        shift = NS if seen > NS else 0
+        largest = int(c.pos[0, 0].amax()) + shift
+        if NS:
+            largest = max(largest, int(c.sink_pos[0, 0].amax()))
+        assert largest + 1 == min(seen, W * C + NS), (seen, largest)
+
+
 def test_eager_add_same_as_one_cascade():
     """cascade/models/test.py:423-497."""
     for S in (32, 64, 128):
