@@ -67,7 +67,7 @@ class AttnArgs(C.Structure):
         ("inv_freq", VP),
         ("beta", C.c_double),
         ("head_reduction", C.c_int32), ("homogeneous_heads", C.c_int32),
-        ("dtype", C.c_int32), ("reserved", C.c_int32),
+        ("dtype", C.c_int32), ("filled_slots", C.c_int32),
         ("workspace", VP), ("workspace_bytes", I64),
     ]
 

@@ -25,7 +25,7 @@ def default_inv_freq(head_dim: int, theta: float, device) -> torch.Tensor:
 
 
 def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_pos: bool = False,
-                    _stream: Optional[int] = None) -> torch.Tensor:
+                    _stream: Optional[int] = None, _replayable: bool = False) -> torch.Tensor:
     """Position ids of the incoming chunk (cascade_attention.py:119-150) without a host sync:
     0.. on the first call, otherwise one past the largest id among sinks and cache slots
     (stale and masked entries included, as in the reference).  One small kernel of the library.
@@ -38,8 +38,9 @@ def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_p
     # out ids below the number of stored tokens, cascading_cache.py:112-142), and the chunk starts one past them
     # whatever the stream does later.  The ids are then a function of the host-side token counter: no kernel, no
     # device read.  (This holds for every state the update itself produces from an empty cache.)
+    # (A caller that records the launches for replay gets the host value only once it no longer changes.)
     S, NS = cache.max_seq_len[layer_idx], cache.num_sink_tokens
-    if not do_og_pos and cache.eager_fill and S > 0:
+    if not do_og_pos and cache.eager_fill and S > 0 and (not _replayable or cache._seen_host[layer_idx] >= S + NS):
         start = min(int(cache._seen_host[layer_idx]), S + NS)
         memo = cache.__dict__.setdefault("_steady_q_pos", {})
         key = (start, q_len, dev)
@@ -148,12 +149,15 @@ def _describe_attention(query_states, key_states, value_states, cache, L, inv_fr
 def cascade_attention(query_states, key_states, value_states, cache: CascadingKVCache, layer_idx: int,
                       inv_freq: torch.Tensor, head_reduction: Optional[str] = None,
                       homogeneous_heads: bool = False, do_og_pos: bool = False, scale: Optional[float] = None,
-                      update_cache: bool = True):
+                      update_cache: bool = True, replayable: bool = False):
     """Attention of one chunk over [sink | cascades | chunk] plus the cache bookkeeping.
 
     query_states ``(B, H, q, D)``, key/value_states ``(B, KVH, q, D)``, all un-rotated.
     Returns ``out (B, H, q, D)``; mutates ``cache.score_cache[layer_idx]`` and, if
     ``update_cache``, scatters the chunk into the cache with its new scores.
+    ``replayable``: the launches are being recorded for replay (a HIP graph), so nothing that the host derives
+    from its token counter and that changes from call to call may go into them: position ids come from the device
+    unless the cache is full, and the library is not told how many slots are filled.
     """
     _require_device(query_states, "query_states")
     lib = _abi.lib()
@@ -170,7 +174,7 @@ def cascade_attention(query_states, key_states, value_states, cache: CascadingKV
 
     with torch.cuda.device(dev):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        q_pos = chunk_positions(cache, L, Q, do_og_pos, _stream=stream)
+        q_pos = chunk_positions(cache, L, Q, do_og_pos, _stream=stream, _replayable=replayable)
         out = torch.empty((B, H, Q, D), dtype=dtype, device=dev)
         new_scores = torch.empty((B, KVH, Q), dtype=dtype, device=dev)
 
@@ -192,6 +196,10 @@ def cascade_attention(query_states, key_states, value_states, cache: CascadingKV
         a.k_new, a.v_new = key_states.data_ptr(), value_states.data_ptr()
         a.q_pos = q_pos.data_ptr()
         a.pos_shift = 0 if do_og_pos else cache.pos_shift(L)
+        # the cache fills from slot 0 up and holds at most the tokens seen past the sinks: single-token steps skip
+        # the empty part of a cache that is still filling
+        filled = int(cache._seen_host[L]) - cache.num_sink_tokens
+        a.filled_slots = filled if not replayable and 0 < filled < cache.max_seq_len[L] else 0
         a.out = out.data_ptr()
         a.new_scores = new_scores.data_ptr()
         ws = workspace(dev, a._need, stream)
@@ -233,7 +241,8 @@ class DecodeStepGraph:
         self._state = None
 
     def _run(self):
-        return cascade_attention(self.q, self.k, self.v, self.cache, self.layer_idx, self.inv_freq, **self.kw)
+        return cascade_attention(self.q, self.k, self.v, self.cache, self.layer_idx, self.inv_freq, replayable=True,
+                                 **self.kw)
 
     def step(self, q=None, k=None, v=None):
         """One token: ``q (B, H, 1, D)``, ``k, v (B, KVH, 1, D)`` (or None when the caller has written them into

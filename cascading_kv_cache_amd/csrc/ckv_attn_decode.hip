@@ -21,6 +21,8 @@ namespace {
 constexpr int kD = 128;
 constexpr int kTK = 128;     // keys per workgroup tile
 constexpr int kSteps = 8;    // a wavefront covers 32 keys as 8 steps of 4 keys (16 lanes per key)
+constexpr int kStreamWaves = 8;          // streaming kernel: wavefronts per workgroup, 16 keys each
+constexpr int kSK = 16 * kStreamWaves;   // streaming kernel: keys per tile
 
 template <typename T>
 __device__ inline float round_t(float v) {
@@ -86,7 +88,18 @@ struct DecodeParams {
     int tiles;
     int shared_pos;
     float scale_log2;
+    // Streaming kernel: items exist only for tiles that can hold a visible key, numbered in tile order: the
+    // first `tiles_pre` tiles (sinks and the cache slots below the caller's `filled_slots` bound) and the tile
+    // of the new token (`tiles - 1`) when it is not one of them.  A cache that is still filling is mostly hidden.
+    int tiles_pre;
+    int n_vis;         // tiles_pre, or tiles_pre + 1
 };
+
+// the j-th tile with items; the rank of a tile among those (-1: the tile has no items, its keys are all hidden)
+__device__ inline int stream_tile_of(const DecodeParams& p, int j) { return j < p.tiles_pre ? j : p.tiles - 1; }
+__device__ inline int stream_rank_of(const DecodeParams& p, int tile) {
+    return tile < p.tiles_pre ? tile : (tile == p.tiles - 1 ? p.n_vis - 1 : -1);
+}
 
 // Items (tile-major: item = tile * B * KVH + b * KVH + kvh) are dealt out in equal contiguous runs:
 // workgroup w takes [total * w / wgs, total * (w + 1) / wgs).  Chunk index of an item.
@@ -610,8 +623,6 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
 // combination across wavefronts.  It is written out at the top of the next item, off the critical
 // path.
 // ---------------------------------------------------------------------------------------------
-constexpr int kStreamWaves = 8;                   // wavefronts per workgroup, 16 keys each
-constexpr int kSK = 16 * kStreamWaves;            // keys per tile
 constexpr int kStreamThreads = 64 * kStreamWaves;
 constexpr int kStreamWgPerCu = 8 / kStreamWaves;  // eight wavefronts per CU
 constexpr int kStreamDimBlocks = 8 / kStreamWaves;  // 16-dim blocks of the output a wavefront owns
@@ -666,7 +677,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
     const int key16 = lane & 15, kq = lane >> 4;  // logits: MFMA column (key) and k-quarter
     const int pg = lane & 3, kgrp = lane >> 2;    // softmax: head and group of kKpl keys
     constexpr int kKpl = kSK / 16, kDb = kStreamDimBlocks;
-    const int64_t nbh = a.B * a.KVH, total = (int64_t)p.tiles * nbh;
+    const int64_t nbh = a.B * a.KVH, total = (int64_t)p.n_vis * nbh;
     const int64_t item0 = total * blockIdx.x / gridDim.x, item1 = total * (blockIdx.x + 1) / gridDim.x;
     const int64_t NS = a.num_sink, S = a.S;
     const int KVH = (int)a.KVH;
@@ -701,9 +712,10 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
     unsigned char* p_wave = smem + kStreamP + wave * (4 * kStreamPPitch);                       // [4][kSK] 16-bit, padded rows
 
     for (int64_t item = item0; item < item1;) {
-        const int64_t tile = item / nbh, bh0 = item % nbh;
-        const int64_t bh1 = (tile + 1) * nbh > item1 ? item1 - tile * nbh : nbh;
-        item = tile * nbh + bh1;
+        const int64_t jt = item / nbh, bh0 = item % nbh;  // jt: the tile's rank among the visible ones
+        const int64_t tile = stream_tile_of(p, (int)jt);
+        const int64_t bh1 = (jt + 1) * nbh > item1 ? item1 - jt * nbh : nbh;
+        item = jt * nbh + bh1;
         const int64_t n_wave = tile * kSK + wave * 16;  // first key of this wavefront
 
         // ---- per-tile constants (the same for every (b, kvh): positions are shared)
@@ -816,7 +828,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
         // of them (two wavefronts one more each), and none before the first item of a run has results.
         auto flush = [&]() {
             if (!pending) return;
-            const int64_t pend_item = tile * nbh + (int64_t)pend_b * KVH + pend_kvh;
+            const int64_t pend_item = jt * nbh + (int64_t)pend_b * KVH + pend_kvh;
             const int64_t chunk_i = (pend_item - item0) * gridDim.x + blockIdx.x;
             unsigned char* chunk = p.chunks + chunk_i * (G * (kSK + kD) * 2);
             if (wave == kStreamProbWave && pg < G)  // every wavefront holds all of them: one stores, 16 bytes a lane
@@ -1002,9 +1014,9 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
     }
 }
 
-// one workgroup per (b, h): 4 quarters of 128 threads walk every 4th tile, then merge through LDS
-// AVG: the partials are per-tile averages in the tensor dtype (the streaming kernel) instead of fp32 sums
-template <typename T, bool AVG>
+// one workgroup per (b, h): 16 groups of 32 threads walk every 16th tile, eight tiles in flight, then merge
+// through LDS (the fp32 partial sums of the kernels that take a tile per workgroup)
+template <typename T>
 __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
     __shared__ float sh_m[8], sh_l[16];
     __shared__ float4 sh_o[16][32];
@@ -1012,13 +1024,8 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
     const int64_t row = blockIdx.x;  // b * H + h
     const int tid = threadIdx.x, d4 = tid & 31, grp = tid >> 5;  // 16 groups of 32 threads, 4 dims per thread
     const float* ml = p.part_ml + row * p.tiles * 2;
-    // streaming kernel: the row's results sit in the chunks of the items (tile, b, kvh)
-    const int64_t nbh_s = a.B * a.KVH, total_s = (int64_t)p.tiles * nbh_s;
-    const int G_s = (int)(a.H / a.KVH), g_s = (int)((row % a.H) % G_s);
-    const int64_t bh_s = (row / a.H) * a.KVH + (row % a.H) / G_s;
-    auto chunk_of = [&](int t) { return stream_chunk_of((int64_t)t * nbh_s + bh_s, total_s, p.stream_wgs); };
     float M = -INFINITY;
-    for (int t = tid; t < p.tiles; t += 512) M = fmaxf(M, AVG ? p.part_ml[(chunk_of(t) * G_s + g_s) * 2] : ml[2 * t]);
+    for (int t = tid; t < p.tiles; t += 512) M = fmaxf(M, ml[2 * t]);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
     if ((tid & 63) == 0) sh_m[tid >> 6] = M;
@@ -1031,45 +1038,21 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
     float L = 0.f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     const float4* po = reinterpret_cast<const float4*>(p.part_o + row * p.tiles * kD) + d4;
-    const int64_t chunk_bytes = (int64_t)G_s * (kSK + kD) * 2;
-    const int64_t in_chunk = ((int64_t)G_s * kSK + g_s * kD) * 2 + d4 * 8;
     constexpr int kBatch = 8;
     for (int t0 = grp; t0 < p.tiles; t0 += 16 * kBatch) {
         float4 v[kBatch];
         float2 w[kBatch];
-        // chunk of tile t0 + 16 u: worked out by lane u of the group (the division is the cost) and handed round
-        int64_t ck_mine = 0;
-        if constexpr (AVG) {
-            const int t = t0 + 16 * (d4 & (kBatch - 1));
-            if (t < p.tiles) ck_mine = chunk_of(t);
-        }
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
             const int t = t0 + 16 * u;
             const bool ok = t < p.tiles;
-            if constexpr (AVG) {
-                uint2 r = make_uint2(0u, 0u);
-                w[u] = make_float2(-INFINITY, 0.f);
-                const int64_t ck = __shfl(ck_mine, (tid & 32) + u);
-                if (ok) {
-                    r = *reinterpret_cast<const uint2*>(p.chunks + ck * chunk_bytes + in_chunk);
-                    w[u] = *reinterpret_cast<const float2*>(p.part_ml + (ck * G_s + g_s) * 2);
-                }
-                v[u] = make_float4(Mma16<T>::lo(r.x), Mma16<T>::hi(r.x), Mma16<T>::lo(r.y), Mma16<T>::hi(r.y));
-            } else {
-                v[u] = ok ? po[(int64_t)t * (kD / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
-                w[u] = ok ? *reinterpret_cast<const float2*>(ml + 2 * t) : make_float2(-INFINITY, 0.f);
-            }
+            v[u] = ok ? po[(int64_t)t * (kD / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
+            w[u] = ok ? *reinterpret_cast<const float2*>(ml + 2 * t) : make_float2(-INFINITY, 0.f);
         }
 #pragma unroll
         for (int u = 0; u < kBatch; u++) {
-            float sc = w[u].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w[u].x - M);
-            if constexpr (AVG) {
-                sc *= w[u].y;
-                L += sc;
-            } else {
-                L = fmaf(w[u].y, sc, L);
-            }
+            const float sc = w[u].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w[u].x - M);
+            L = fmaf(w[u].y, sc, L);
             o.x = fmaf(v[u].x, sc, o.x);
             o.y = fmaf(v[u].y, sc, o.y);
             o.z = fmaf(v[u].z, sc, o.z);
@@ -1093,6 +1076,99 @@ __global__ void __launch_bounds__(512) decode_tail_kernel(DecodeParams p) {
     out[d * a.out_stride[3]] = Elem<T>::from_float(od / L);
     if (d == 0) {
         const float l2 = M + __builtin_amdgcn_logf(L);
+        p.lse2[row] = l2;
+        if (a.lse) a.lse[row] = l2 * 0.6931471805599453f;
+    }
+}
+
+// The same for the streaming kernel's results (per-tile averages in the tensor dtype, one (max, sum) pair per head
+// and item) in as few trips to memory as the tiles allow: 32 groups of 16 lanes, a lane owns 8 dims (one 16-byte
+// piece of an average), a group walks every 32nd tile with kTailBatch tiles requested at once and keeps a running
+// (max, sum, weighted average) of its own, so no pass over the maxima comes first; the groups merge through LDS.
+// 513 tiles (a 64K cache) are two batches per group, 257 tiles one.
+constexpr int kTailBatch = 9;
+
+template <typename T>
+__global__ void __launch_bounds__(512) decode_tail_stream_kernel(DecodeParams p) {
+    __shared__ float sh_m[32], sh_l[32];
+    __shared__ float sh_o[32][kD];
+    const ckv_attn_args& a = p.a;
+    const int64_t row = blockIdx.x;  // b * H + h
+    const int tid = threadIdx.x, d8 = tid & 15, grp = tid >> 4;
+    const int n_vis = p.n_vis;  // the items are numbered over the tiles that can hold a visible key
+    const int64_t nbh = a.B * a.KVH, total = (int64_t)n_vis * nbh;
+    const int G = (int)(a.H / a.KVH), g = (int)((row % a.H) % G);
+    const int64_t bh = (row / a.H) * a.KVH + (row % a.H) / G;
+    const int64_t chunk_bytes = (int64_t)G * (kSK + kD) * 2;
+    const int64_t in_chunk = ((int64_t)G * kSK + g * kD) * 2 + d8 * 16;
+    float M = -INFINITY, L = 0.f;
+    float o[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = 0.f;
+    for (int t0 = grp; t0 < n_vis; t0 += 32 * kTailBatch) {
+        // chunk of tile t0 + 32 u: worked out by lane u of the group (two divisions) and handed round
+        int64_t ck_mine = 0;
+        {
+            const int t = t0 + 32 * d8;
+            if (d8 < kTailBatch && t < n_vis) ck_mine = stream_chunk_of((int64_t)t * nbh + bh, total, p.stream_wgs);
+        }
+        uint4 v[kTailBatch];
+        float2 w[kTailBatch];
+#pragma unroll
+        for (int u = 0; u < kTailBatch; u++) {
+            const int64_t ck = __shfl(ck_mine, (tid & 48) + u);
+            v[u] = make_uint4(0u, 0u, 0u, 0u);
+            w[u] = make_float2(-INFINITY, 0.f);
+            if (t0 + 32 * u < n_vis) {
+                v[u] = *reinterpret_cast<const uint4*>(p.chunks + ck * chunk_bytes + in_chunk);
+                w[u] = *reinterpret_cast<const float2*>(p.part_ml + (ck * G + g) * 2);
+            }
+        }
+        float bm = M;
+#pragma unroll
+        for (int u = 0; u < kTailBatch; u++) bm = fmaxf(bm, w[u].x);
+        if (bm == -INFINITY) continue;  // nothing visible so far
+        const float keep = M == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(M - bm);
+        M = bm;
+        L *= keep;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] *= keep;
+#pragma unroll
+        for (int u = 0; u < kTailBatch; u++) {
+            const float sc = w[u].x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(w[u].x - M) * w[u].y;
+            L += sc;
+            const uint32_t r[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                o[2 * e] = fmaf(Mma16<T>::lo(r[e]), sc, o[2 * e]);
+                o[2 * e + 1] = fmaf(Mma16<T>::hi(r[e]), sc, o[2 * e + 1]);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) sh_o[grp][d8 * 8 + e] = o[e];
+    if (d8 == 0) {
+        sh_m[grp] = M;
+        sh_l[grp] = L;
+    }
+    __syncthreads();
+    if (tid >= kD) return;
+    float Mx = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 32; k++) Mx = fmaxf(Mx, sh_m[k]);
+    float od = 0.f;
+    L = 0.f;
+#pragma unroll
+    for (int k = 0; k < 32; k++) {
+        const float f = sh_m[k] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sh_m[k] - Mx);
+        od = fmaf(sh_o[k][tid], f, od);
+        L = fmaf(sh_l[k], f, L);
+    }
+    const int64_t b = row / a.H, h = row % a.H;
+    T* out = (T*)a.out + b * a.out_stride[0] + h * a.out_stride[1];
+    out[tid * a.out_stride[3]] = Elem<T>::from_float(od / L);
+    if (tid == 0) {
+        const float l2 = Mx + __builtin_amdgcn_logf(L);
         p.lse2[row] = l2;
         if (a.lse) a.lse[row] = l2 * 0.6931471805599453f;
     }
@@ -1145,10 +1221,15 @@ __global__ void __launch_bounds__(256) decode_scores_kernel(DecodeParams p, floa
             const int64_t row = b * a.H + kv * G + g;
             float pt;
             if constexpr (PROBS) {  // 2^(logit - tile maximum) from the streaming kernel, and that maximum
-                const int64_t ck = stream_chunk_of((n / kSK) * (a.B * a.KVH) + b * a.KVH + kv, p.tiles * (a.B * a.KVH), p.stream_wgs);
-                const float e = (float)reinterpret_cast<const _Float16*>(p.chunks + ck * (G * (kSK + kD) * 2))[g * kSK + n % kSK];
-                const float m = p.part_ml[(ck * G + g) * 2];
-                pt = e == 0.f ? 0.f : round_t<T>(e * __builtin_amdgcn_exp2f(m - p.lse2[row]));
+                const int jt = stream_rank_of(p, (int)(n / kSK));  // -1: no key of the tile is visible
+                pt = 0.f;
+                if (jt >= 0) {
+                    const int64_t ck = stream_chunk_of((int64_t)jt * (a.B * a.KVH) + b * a.KVH + kv,
+                                                       (int64_t)p.n_vis * (a.B * a.KVH), p.stream_wgs);
+                    const float e = (float)reinterpret_cast<const _Float16*>(p.chunks + ck * (G * (kSK + kD) * 2))[g * kSK + n % kSK];
+                    const float m = p.part_ml[(ck * G + g) * 2];
+                    pt = e == 0.f ? 0.f : round_t<T>(e * __builtin_amdgcn_exp2f(m - p.lse2[row]));
+                }
             } else {
                 pt = round_t<T>(__builtin_amdgcn_exp2f(lg[g] - p.lse2[row]));
             }
@@ -1202,13 +1283,19 @@ __global__ void __launch_bounds__(256) decode_scores_probs_kernel(DecodeParams p
     const int64_t n0 = (idx % per) * 8, kvh = (idx / per) % a.KVH, b = idx / (per * a.KVH);
     if (n0 + 8 <= a.num_sink || n0 >= p.N) return;  // sinks keep no score; padding
     float pr[G][8];
-    const int64_t ck = stream_chunk_of((n0 / kSK) * (a.B * a.KVH) + b * a.KVH + kvh, p.tiles * (a.B * a.KVH), p.stream_wgs);
+    const int jt = stream_rank_of(p, (int)(n0 / kSK));  // -1: no key of the tile is visible, all probabilities are 0
+    const int64_t ck = jt < 0 ? 0 : stream_chunk_of((int64_t)jt * (a.B * a.KVH) + b * a.KVH + kvh,
+                                                    (int64_t)p.n_vis * (a.B * a.KVH), p.stream_wgs);
     const unsigned char* chunk = p.chunks + ck * (G * (kSK + kD) * 2);
 #pragma unroll
     for (int g = 0; g < G; g++) {
         const int64_t row = b * a.H + kvh * G + g;
-        const uint4 raw = *reinterpret_cast<const uint4*>(chunk + (g * kSK + n0 % kSK) * 2);
-        const float c = __builtin_amdgcn_exp2f(p.part_ml[(ck * G + g) * 2] - p.lse2[row]);
+        uint4 raw = make_uint4(0u, 0u, 0u, 0u);
+        float c = 0.f;
+        if (jt >= 0) {
+            raw = *reinterpret_cast<const uint4*>(chunk + (g * kSK + n0 % kSK) * 2);
+            c = __builtin_amdgcn_exp2f(p.part_ml[(ck * G + g) * 2] - p.lse2[row]);
+        }
         const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
         for (int k = 0; k < 8; k++) {
@@ -1284,7 +1371,14 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
     const ckv_attn_args& a = p.a;
     const bool use_stream =
         !std::is_same<T, float>::value && G <= 4 && p.shared_pos && stream_offsets_fit(a);
-    if (use_stream) p.tiles = (int)((p.N + kSK - 1) / kSK);  // the streaming kernel has its own tile size
+    if (use_stream) {
+        p.tiles = (int)((p.N + kSK - 1) / kSK);  // the streaming kernel has its own tile size
+        // keys that can be visible: the sinks, the leading `filled_slots` cache slots (all S when the caller gives
+        // no bound) and the new token
+        const int64_t filled = a.filled_slots > 0 && a.filled_slots < a.S ? a.filled_slots : a.S;
+        p.tiles_pre = (int)std::min<int64_t>((a.num_sink + filled + kSK - 1) / kSK, p.tiles);
+        p.n_vis = p.tiles_pre < p.tiles ? p.tiles_pre + 1 : p.tiles_pre;
+    }
     p.Np = (int64_t)p.tiles * kSK;
     {
         StageScope sc(CKV_STAGE_PREP, stream);
@@ -1312,7 +1406,7 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
                 if (int rc = current_device_info(&di)) return rc;
                 int64_t wgs = (di.cus > 0 ? di.cus : 256) * kStreamWgPerCu;
                 if (wgs > kStreamMaxWgs) wgs = kStreamMaxWgs;
-                if (wgs > p.tiles * nbh) wgs = p.tiles * nbh;
+                if (wgs > p.n_vis * nbh) wgs = p.n_vis * nbh;
                 p.stream_wgs = (int)wgs;
                 hipEvent_t ev0, ev1;
                 prof_kernel_events(CKV_STAGE_DECODE, &ev0, &ev1);
@@ -1334,11 +1428,11 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
         bool launched = false;
         if constexpr (G <= 4 && !std::is_same<T, float>::value) {
             if (use_stream) {
-                hipLaunchKernelGGL((decode_tail_kernel<T, true>), dim3((unsigned)(a.B * a.H)), dim3(512), 0, stream, p);
+                hipLaunchKernelGGL(decode_tail_stream_kernel<T>, dim3((unsigned)(a.B * a.H)), dim3(512), 0, stream, p);
                 launched = true;
             }
         }
-        if (!launched) hipLaunchKernelGGL((decode_tail_kernel<T, false>), dim3((unsigned)(a.B * a.H)), dim3(512), 0, stream, p);
+        if (!launched) hipLaunchKernelGGL(decode_tail_kernel<T>, dim3((unsigned)(a.B * a.H)), dim3(512), 0, stream, p);
         CKV_HIP_TRY(hipGetLastError());
         if (a.cache_s || a.new_scores) {
             // w_ema[0] == w_new[0] == (1 - beta) for a single query row; the new token's weight is
@@ -1426,6 +1520,8 @@ int launch_decode(const ckv_attn_args& a, hipStream_t stream) {
     p.logits = reinterpret_cast<float*>(w);
     p.chunks = reinterpret_cast<unsigned char*>(w);
     p.stream_wgs = 0;
+    p.tiles_pre = 0;
+    p.n_vis = 0;
     w += logits_area_bytes(a.B, a.H, a.KVH, p.N);
     const int64_t tiles_max = (p.N + kMinTile - 1) / kMinTile;
     p.part_ml = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * tiles_max * 2 * 4, 256);

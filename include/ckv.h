@@ -188,7 +188,10 @@ typedef struct ckv_attn_args {
     int32_t head_reduction;        /* ckv_head_reduction                                  */
     int32_t homogeneous_heads;     /* reduce over all H heads (cascade_attention.py:240-242) */
     int32_t dtype;                 /* ckv_dtype of every floating tensor above            */
-    int32_t reserved;
+    int32_t filled_slots;          /* optional bound: cache slots at or past this index are hidden whatever `mask`
+                                      says (the cache fills from slot 0 up, cascading_cache.py:381-726, so the
+                                      tokens stored so far bound it); 0 = no bound, every slot is looked at.  Lets
+                                      the single-token kernels skip the empty part of a cache that is still filling. */
 
     void* workspace;
     int64_t workspace_bytes;

@@ -17,8 +17,8 @@ def make_cache(B, KVH, D, NS, W, C, dtype, eager):
                             eager_fill=eager, verbose=False)
 
 
-@pytest.mark.parametrize("eager_fill,B,H,KVH", [(True, 1, 8, 2), (False, 2, 14, 2)])
-def test_graph_replayed_steps_equal_eager_steps(eager_fill, B, H, KVH):
+@pytest.mark.parametrize("eager_fill,B,H,KVH,chunks", [(True, 1, 8, 2, 5), (False, 2, 14, 2, 5), (True, 1, 8, 2, 4), (True, 2, 8, 2, 1)])
+def test_graph_replayed_steps_equal_eager_steps(eager_fill, B, H, KVH, chunks):
     from cascading_kv_cache_amd.cascade_attention import DecodeStepGraph, cascade_attention, default_inv_freq
 
     dtype, D, NS, W, C = torch.bfloat16, 128, 4, 64, 4
@@ -26,7 +26,9 @@ def test_graph_replayed_steps_equal_eager_steps(eager_fill, B, H, KVH):
     inv_freq = default_inv_freq(D, 5e5, "cuda:0")
     gen = torch.Generator().manual_seed(23)
     L = 1  # a layer other than the first: the graph must address that layer's state
-    for _ in range(5):  # past the window: the cascades evict
+    # 5 chunks: past the window, the cascades evict; 4: the cache fills up during the replayed steps; 1: it stays
+    # mostly empty, and the position ids and the filled part differ from step to step
+    for _ in range(chunks):
         q = (torch.randn(B, H, 60, D, generator=gen) * 0.7).to(dtype).cuda()
         k = (torch.randn(B, KVH, 60, D, generator=gen) * 0.7).to(dtype).cuda()
         v = (torch.randn(B, KVH, 60, D, generator=gen) * 0.7).to(dtype).cuda()
@@ -34,7 +36,7 @@ def test_graph_replayed_steps_equal_eager_steps(eager_fill, B, H, KVH):
             cascade_attention(q, k, v, c, L, inv_freq)
     graph = DecodeStepGraph(rep, L, inv_freq, H)
     scratch = torch.zeros(1 << 16, device="cuda:0")
-    for step in range(14):
+    for step in range(24):
         q = (torch.randn(B, H, 1, D, generator=gen) * 0.7).to(dtype).cuda()
         k = (torch.randn(B, KVH, 1, D, generator=gen) * 0.7).to(dtype).cuda()
         v = (torch.randn(B, KVH, 1, D, generator=gen) * 0.7).to(dtype).cuda()
