@@ -405,7 +405,7 @@ struct FwdParams {
     float* lse;       // (B*H, Q) natural log
     float* lse2;      // (B*H, Q) minus the log2-domain normaliser, consumed by the column pass
     int64_t B, H, KVH, Q, N, Nc, n_pad;
-    int G, QT;        // heads per kv head, positions per workgroup (G * QT <= 256)
+    int G;            // heads per kv head: a workgroup takes 256 consecutive rows of the kv head's (position, head) pairs, position-major
     float scale_log2; // softmax scale * log2(e)
     int n_qt, xcd_aware;  // query tiles per kv head; 1-D XCD-aware block order
 };
@@ -457,9 +457,11 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     qt_i = p.n_qt - 1 - qt_i;
     const int64_t bkv = bkv_i;
     const int64_t b = bkv / p.KVH, kvh = bkv % p.KVH;
-    const int m0 = qt_i * p.QT;
-
-    int m_hi = m0 + p.QT - 1;
+    // rows of a kv head are its (position, head) pairs, position-major: row rf = position * G + head.  A workgroup
+    // takes 256 consecutive ones whatever G is (7 heads per kv head: 36 4/7 positions), so every wavefront has
+    // 32 real rows and the number of workgroups is Q * G / 256, not Q / floor(256 / G).
+    const int m0 = qt_i * kRows / p.G;
+    int m_hi = (qt_i * kRows + kRows - 1) / p.G;
     if (m_hi > (int)p.Q - 1) m_hi = (int)p.Q - 1;
     const int n_tiles = (int)((p.Nc + m_hi) / kBN) + 1;
     const int tiles_cap = (int)(p.n_pad / kBN);
@@ -491,11 +493,11 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     int row_m;
     uint4 qreg[8];
     {
-        const int r = wave * 32 + col;
-        const int g = r / p.QT, mloc = r % p.QT;
-        row_m = m0 + mloc;
+        const int rf = qt_i * kRows + wave * 32 + col;
+        const int g = rf % p.G;
+        row_m = rf / p.G;
         const int64_t row_h = kvh * p.G + g;
-        const bool row_ok = g < p.G && row_m < p.Q;
+        const bool row_ok = row_m < p.Q;
         const T* qrow = (const T*)p.qr + ((b * p.H + row_h) * p.Q + row_m) * kD;
 #pragma unroll
         for (int kk = 0; kk < 8; kk++) {
@@ -785,9 +787,9 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
 
     // epilogue: lane owns d = 32dt + 8(v/4) + 4half + v%4 of its query row
     const float l_tot = l_run + __shfl_xor(l_run, 32);
-    const int g_row = (wave * 32 + col) / p.QT;
+    const int g_row = (qt_i * kRows + wave * 32 + col) % p.G;
     const int64_t row_h = kvh * p.G + g_row;
-    const bool row_ok = g_row < p.G && row_m < p.Q;
+    const bool row_ok = row_m < p.Q;
     const float inv = 1.f / l_tot;
     const bool rows16 = p.out_stride[3] == 1 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0 && p.out_stride[0] % 8 == 0 &&
                         p.out_stride[1] % 8 == 0 && p.out_stride[2] % 8 == 0;
@@ -813,9 +815,9 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
 #pragma unroll
         for (int pass = 0; pass < 8; pass++) {
             const int r = 4 * pass + (lane >> 4), piece = lane & 15;
-            const int rr = wave * 32 + r;
-            const int g_r = rr / p.QT, m_r = m0 + rr % p.QT;
-            if (g_r < p.G && m_r < p.Q) {
+            const int rr = qt_i * kRows + wave * 32 + r;
+            const int g_r = rr % p.G, m_r = rr / p.G;
+            if (m_r < p.Q) {
                 const uint4 v = *reinterpret_cast<const uint4*>(ow + r * kRowPitch + piece * 16);
                 T* dst = (T*)p.out + b * p.out_stride[0] + (kvh * p.G + g_r) * p.out_stride[1] + m_r * p.out_stride[2];
                 *reinterpret_cast<uint4*>(dst + piece * 8) = v;
@@ -1271,9 +1273,8 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         fp.lse2 = mp.lse2;
         fp.B = mp.B; fp.H = mp.H; fp.KVH = mp.KVH; fp.Q = mp.Q; fp.N = n; fp.Nc = n - mp.Q; fp.n_pad = n_pad;
         fp.G = G;
-        fp.QT = kRows / G;
         fp.scale_log2 = 1.f;  // already on the staged queries
-        const dim3 grid((unsigned)((mp.Q + fp.QT - 1) / fp.QT), (unsigned)(mp.B * mp.KVH));
+        const dim3 grid((unsigned)((mp.Q * G + kRows - 1) / kRows), (unsigned)(mp.B * mp.KVH));
         const int lds = pipe_lds_bytes(n_pad);
         if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fwd_pipe_kernel<T>), lds)) return rc;
         fp.n_qt = (int)grid.x;
