@@ -7,6 +7,11 @@
 //                 row with 8-byte pieces, K is rotated in registers, the G query heads of the
 //                 group share the row.  Outputs: raw logits (log2 domain) per key and head, and one
 //                 (max, sum, weighted V) partial per (head, tile).
+//   decode_stream 16-bit caches with shared positions and up to 8 query heads per kv head (the usual case): the
+//                 (128-key tile, batch x kv-head) items are dealt out in equal runs over one workgroup per
+//                 compute unit; rows travel global -> LDS as asynchronous copies one item ahead; logits and P.V
+//                 on the matrix pipe; per item one result chunk (fp16 probabilities relative to the tile
+//                 maximum, the tile's weighted V average, maximum and sum).  decode_stream_wide: 5 to 8 heads.
 //   decode_tail   combine the partials of a row: out, log-sum-exp.
 //   decode_scores P = exp2(logit - lse) exactly, head reduction, score EMA of every slot and the
 //                 new token's own score (cascade_attention.py:315-330 with q_len == 1).
@@ -1014,6 +1019,342 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The streaming kernel for 5 to 8 query heads per kv head (Qwen2-7B has 7).  The item stream, the row copies,
+// the waits and the result chunks are those of the kernel above; what differs: the query block of an item
+// (8 heads x 256 bytes) is one per workgroup and stage, copied by wavefronts 0 and 1 one item ahead and made
+// visible by that item's barrier; the logits of 8 heads go through LDS; and every wavefront normalises them
+// directly in the layout of the P.V operand (lane = (head, quarter) holds 32 keys of its head), so the
+// probabilities never go through LDS.  Wavefront w stores the 16 keys 16 w .. of every head's probabilities.
+// ---------------------------------------------------------------------------------------------
+constexpr int kWideQ = 2 * kStreamStage;            // two query blocks [8 heads][256 bytes]
+constexpr int kWideS = kWideQ + 2 * 2048;           // two [8 heads] logit planes, rows of kWidePitch floats
+constexpr int kWidePitch = kSK + 16;                // the pad spreads the heads over the banks
+constexpr int kWideLds = kWideS + 2 * 8 * kWidePitch * 4;
+
+__device__ inline void wait_vm(int n, bool lds_too) {  // s_waitcnt vmcnt(n) [lgkmcnt(0)]: the count is an immediate
+    if (lds_too) {
+        switch (n) {
+            case 4: __builtin_amdgcn_s_waitcnt(0x0074); break;
+            case 5: __builtin_amdgcn_s_waitcnt(0x0075); break;
+            case 6: __builtin_amdgcn_s_waitcnt(0x0076); break;
+            case 7: __builtin_amdgcn_s_waitcnt(0x0077); break;
+            default: __builtin_amdgcn_s_waitcnt(0x0070); break;
+        }
+    } else {
+        switch (n) {
+            case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+            case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
+            case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+            case 7: __builtin_amdgcn_s_waitcnt(0x0F77); break;
+            default: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+        }
+    }
+}
+
+template <typename T, int G>
+__global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_wide_kernel(DecodeParams p) {
+    static_assert(G > 4 && G <= 8, "the query block and the logit planes hold 8 heads");
+    extern __shared__ __align__(16) unsigned char smem[];
+    const uint32_t lds_base = lds_address(smem);
+    const ckv_attn_args& a = p.a;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int key16 = lane & 15, kq = lane >> 4;  // logits: MFMA column (key) and k-quarter; softmax and P.V: head and key quarter
+    constexpr int kPv = kSK / 16, kDb = kStreamDimBlocks;   // contraction steps of 16 keys
+    const int64_t nbh = a.B * a.KVH, total = (int64_t)p.n_vis * nbh;
+    const int64_t item0 = total * blockIdx.x / gridDim.x, item1 = total * (blockIdx.x + 1) / gridDim.x;
+    const int64_t NS = a.num_sink, S = a.S;
+    const int KVH = (int)a.KVH;
+    constexpr int kEs = (int)sizeof(T);
+
+    int kaddr[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) kaddr[ks] = (wave * 16 + key16) * 256 + (((4 * ks + kq) ^ key16) << 4);
+    int vt_addr[kDb];
+    {
+        const int r_l = lane & 15, key = 4 * (lane >> 4) + (r_l >> 2);
+#pragma unroll
+        for (int b2 = 0; b2 < kDb; b2++) {
+            vt_addr[b2] = kSK * 256 + key * 256 + 32 * ((kDb * wave + b2) ^ (key & 7)) + 16 * ((r_l & 3) >> 1) + 8 * (r_l & 1);
+        }
+    }
+    // query operand: head row key16 (rows past G read head 0, their results are not used), 16-byte piece
+    // 4 ks + kq kept in slot (4 ks + kq) ^ head
+    const int q_row = key16 < G ? key16 : 0;
+    int q_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) q_off[ks] = kWideQ + q_row * 256 + (((4 * ks + kq) ^ q_row) << 4);
+    float* s_all = reinterpret_cast<float*>(smem + kWideS);  // [2][8][kWidePitch]
+    const bool head_ok = key16 < G;
+
+    for (int64_t item = item0; item < item1;) {
+        const int64_t jt = item / nbh, bh0 = item % nbh;  // jt: the tile's rank among those with items
+        const int64_t tile = stream_tile_of(p, (int)jt);
+        const int64_t bh1 = (jt + 1) * nbh > item1 ? item1 - jt * nbh : nbh;
+        item = jt * nbh + bh1;
+        const int64_t n_wave = tile * kSK + wave * 16;  // first key of this wavefront
+
+        // ---- per-tile constants (the same for every (b, kvh): positions are shared)
+        bool vis1 = false;
+        float cs[2][8], sn[2][8];
+        {
+            const int64_t n = n_wave + key16;
+            int64_t pos = 0;
+            if (n < NS) { vis1 = a.sink_mask[n] == 0; pos = a.sink_pos[n]; }
+            else if (n < NS + S) { vis1 = a.mask[n - NS] == 0; pos = a.pos[n - NS] + a.pos_shift; }
+            else if (n < p.N) { vis1 = true; pos = a.q_pos[0]; }
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int f = 32 * ks + 8 * kq + e;
+                    const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
+                    fast_sincos(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
+                }
+        }
+        // rows of hidden slots are zeroed on the way into the P.V product (0 * NaN): masks of this lane's
+        // operand keys 16 ks + 4 kq .. + 3, two 16-bit values per word
+        uint32_t m01[kPv], m23[kPv];
+#pragma unroll
+        for (int half = 0; half < kSK / 64; half++) {
+            const int64_t n = tile * kSK + 64 * half + lane;
+            bool v = false;
+            if (n < NS) v = a.sink_mask[n] == 0;
+            else if (n < NS + S) v = a.mask[n - NS] == 0;
+            else if (n < p.N) v = true;
+            const unsigned long long vis64 = __builtin_amdgcn_ballot_w64(v);
+#pragma unroll
+            for (int k4 = 0; k4 < 4; k4++) {
+                const int ks = 4 * half + k4;
+                const uint32_t vk = (uint32_t)(vis64 >> (16 * k4 + 4 * kq)) & 0xfu;
+                m01[ks] = ((vk & 1u) ? 0x0000ffffu : 0u) | ((vk & 2u) ? 0xffff0000u : 0u);
+                m23[ks] = ((vk & 4u) ? 0x0000ffffu : 0u) | ((vk & 8u) ? 0xffff0000u : 0u);
+            }
+        }
+        // copies: block jb of a wavefront brings rows 4 jb .. 4 jb + 3 of its 16; seg: 0 sink, 1 cache, 2 the new token
+        int seg_c[4];
+        uint32_t relk[4], relv[4];
+        bool cache_only[4];
+#pragma unroll
+        for (int jb = 0; jb < 4; jb++) {
+            const int r = 4 * jb + (lane >> 4);
+            const int64_t n = n_wave + r;
+            int64_t row_off;
+            if (n < NS) { seg_c[jb] = 0; row_off = n * a.sink_stride[2]; }
+            else if (n < NS + S) { seg_c[jb] = 1; row_off = (n - NS) * a.cache_stride[2]; }
+            else { seg_c[jb] = 2; row_off = 0; }
+            relk[jb] = (uint32_t)(row_off * kEs) + ((((uint32_t)lane & 15u) ^ ((uint32_t)r & 15u)) << 4);
+            relv[jb] = (uint32_t)(row_off * kEs) + ((((uint32_t)lane & 15u) ^ (((uint32_t)r & 7u) << 1)) << 4);
+            cache_only[jb] = __builtin_amdgcn_ballot_w64(seg_c[jb] == 1) == ~0ull;
+        }
+        auto slabs = [&](int b, int kvh, const char* (&kb)[3], const char* (&vb)[3]) {
+            const int64_t o0 = ((int64_t)b * a.sink_stride[0] + (int64_t)kvh * a.sink_stride[1]) * kEs;
+            const int64_t o1 = ((int64_t)b * a.cache_stride[0] + (int64_t)kvh * a.cache_stride[1]) * kEs;
+            const int64_t o2 = ((int64_t)b * a.kv_new_stride[0] + (int64_t)kvh * a.kv_new_stride[1]) * kEs;
+            kb[0] = (const char*)a.sink_k + o0; vb[0] = (const char*)a.sink_v + o0;
+            kb[1] = (const char*)a.cache_k + o1; vb[1] = (const char*)a.cache_v + o1;
+            kb[2] = (const char*)a.k_new + o2; vb[2] = (const char*)a.v_new + o2;
+        };
+        auto copy_rows = [&](const char* (&base)[3], const uint32_t(&rel)[4], uint32_t dst) {  // four copies
+#pragma unroll
+            for (int jb = 0; jb < 4; jb++) {
+                if (cache_only[jb]) {
+                    async_copy16(base[1], rel[jb], dst + jb * 1024);
+                } else {
+#pragma unroll
+                    for (int sgm = 0; sgm < 3; sgm++)
+                        if (seg_c[jb] == sgm) async_copy16(base[sgm], rel[jb], dst + jb * 1024);
+                }
+            }
+        };
+        // the query block of (b, kvh) into stage `st` (wavefronts 0 and 1, four heads each: lane i fills slot
+        // i % 16 of head 4 wave + i / 16 with the piece that belongs there), then this wavefront's K rows.  The
+        // query copy goes first: whoever waits for the four K copies behind it has waited for it too.
+        auto copy_kq = [&](int b, int kvh, int st) {
+            if (wave < 2) {
+                const char* qsrc = (const char*)p.qrot_t + ((int64_t)b * a.H + (int64_t)kvh * G) * (kD * kEs);
+                const int h = 4 * wave + (lane >> 4);
+                if (h < G) async_copy16(qsrc, h * 256 + (((lane & 15) ^ h) << 4), lds_base + kWideQ + st * 2048 + wave * 1024);
+            }
+            const char *kb[3], *vb[3];
+            slabs(b, kvh, kb, vb);
+            copy_rows(kb, relk, lds_base + st * kStreamStage + wave * 4096);
+        };
+        auto copy_v = [&](int b, int kvh, int st) {
+            const char *kb[3], *vb[3];
+            slabs(b, kvh, kb, vb);
+            copy_rows(vb, relv, lds_base + st * kStreamStage + kSK * 256 + wave * 4096);
+        };
+
+        int b = (int)(bh0 / KVH), kvh = (int)(bh0 % KVH);
+        // results of the previous item, stored at the top of the next one
+        bool pending = false;
+        int pend_b = 0, pend_kvh = 0;
+        uint2 pend_o[kDb];
+        float pend_m = 0.f, pend_l = 0.f;
+        uint2 pend_e = make_uint2(0u, 0u);  // fp16 probabilities of head key16, keys 16 wave + 4 kq .. + 3
+#pragma unroll
+        for (int b2 = 0; b2 < kDb; b2++) pend_o[b2] = make_uint2(0u, 0u);
+        auto flush = [&]() {
+            if (!pending) return;
+            const int64_t pend_item = jt * nbh + (int64_t)pend_b * KVH + pend_kvh;
+            const int64_t chunk_i = (pend_item - item0) * gridDim.x + blockIdx.x;
+            unsigned char* chunk = p.chunks + chunk_i * (G * (kSK + kD) * 2);
+            if (head_ok) {
+                *reinterpret_cast<uint2*>(chunk + (key16 * kSK + 16 * wave + 4 * kq) * 2) = pend_e;
+#pragma unroll
+                for (int b2 = 0; b2 < kDb; b2++)
+                    *reinterpret_cast<uint2*>(chunk + (G * kSK + key16 * kD + 16 * (kDb * wave + b2) + 4 * kq) * 2) = pend_o[b2];
+            }
+            if (wave == 0 && kq == 0 && head_ok)  // maximum and sum: G pairs per chunk, in chunk order
+                *reinterpret_cast<float2*>(p.part_ml + (chunk_i * G + key16) * 2) = make_float2(pend_m, pend_l);
+        };
+        // Per item a wavefront issues, in this order: [the query copy of the next item,] four K copies of the
+        // next item, the stores of the previous item's results, and after the barrier four V copies of the next
+        // item.  Loads and stores retire in issue order.
+        const int my_stores = kDb + 1 + (wave == 0 ? 1 : 0);
+        int stored = 0;
+        copy_kq(b, kvh, 0);
+        copy_v(b, kvh, 0);
+        // the first query block of the run must have landed for every wavefront (younger: the four V copies)
+        __builtin_amdgcn_s_waitcnt(0x0F74);
+        __builtin_amdgcn_s_barrier();
+        int st = 0;
+        for (int64_t bh = bh0; bh < bh1; bh++) {
+            int b_nx = b, kvh_nx = kvh;
+            if (bh + 1 < bh1) {  // the last item of a run copies itself again: cheaper than a different path
+                kvh_nx = kvh + 1 == KVH ? 0 : kvh + 1;
+                b_nx = kvh + 1 == KVH ? b + 1 : b;
+            }
+            // this wavefront's K rows of the item are in LDS (younger: the stores issued after them and the four V
+            // copies of this item); its query block was complete before the previous barrier
+            wait_vm(4 + stored, false);
+            copy_kq(b_nx, kvh_nx, st ^ 1);
+            stored = pending ? my_stores : 0;
+            flush();
+            const unsigned char* stage = smem + st * kStreamStage;
+
+            // ---- rotate K in registers, logits by MFMA, shared through LDS
+            {
+                uint4 kraw[4], qop[4];
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) kraw[ks] = *reinterpret_cast<const uint4*>(stage + kaddr[ks]);
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) qop[ks] = *reinterpret_cast<const uint4*>(smem + q_off[ks] + st * 2048);
+                uint4 kop[4];
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    const uint32_t* w1 = reinterpret_cast<const uint32_t*>(&kraw[ks]);
+                    const uint32_t* w2 = reinterpret_cast<const uint32_t*>(&kraw[ks + 2]);
+                    uint32_t o1[4], o2[4];
+#pragma unroll
+                    for (int w = 0; w < 4; w++) {
+                        const float a0 = Mma16<T>::lo(w1[w]), a1 = Mma16<T>::hi(w1[w]);
+                        const float b0 = Mma16<T>::lo(w2[w]), b1 = Mma16<T>::hi(w2[w]);
+                        const float c0 = cs[ks][2 * w], s0 = sn[ks][2 * w];
+                        const float c1 = cs[ks][2 * w + 1], s1 = sn[ks][2 * w + 1];
+                        o1[w] = Mma16<T>::pack2(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
+                        o2[w] = Mma16<T>::pack2(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+                    }
+                    kop[ks] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+                    kop[ks + 2] = make_uint4(o2[0], o2[1], o2[2], o2[3]);
+                }
+                f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) sacc = Mma16<T>::mma(qop[ks], kop[ks], sacc);
+                // lane holds heads 4 kq + v of key key16
+                if (kq < 2) {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        if (4 * kq + v < G)
+                            s_all[(st * 8 + 4 * kq + v) * kWidePitch + wave * 16 + key16] = vis1 ? sacc[v] * p.scale_log2 : -INFINITY;
+                }
+            }
+            // this wavefront's V rows of the item and (wavefronts 0, 1) its part of the next query block have landed
+            // (younger: the four K copies of the next item and the stores of flush()); its logits are in LDS
+            wait_vm(4 + stored, true);
+            __builtin_amdgcn_s_barrier();
+            // every wavefront is past the previous item: its V stage can be refilled
+            copy_v(b_nx, kvh_nx, st ^ 1);
+
+            // ---- softmax of head key16 over the tile, by every wavefront, in the layout of the P.V operand:
+            //      this lane holds keys 16 ks + 4 kq .. + 3 (ks = 0 .. 7); lanes l, l ^ 16, l ^ 32, l ^ 48 share a head
+            float m_t, l_t;
+            uint2 pb[kPv];
+            uint2 e_mine = make_uint2(0u, 0u);
+            {
+                float x[kPv][4];
+                float mloc = -INFINITY;
+#pragma unroll
+                for (int ks = 0; ks < kPv; ks++) {
+                    float4 x4 = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+                    if (head_ok) x4 = *reinterpret_cast<const float4*>(s_all + (st * 8 + key16) * kWidePitch + 16 * ks + 4 * kq);
+                    x[ks][0] = x4.x; x[ks][1] = x4.y; x[ks][2] = x4.z; x[ks][3] = x4.w;
+                    mloc = fmaxf(fmaxf(mloc, fmaxf(x4.x, x4.y)), fmaxf(x4.z, x4.w));
+                }
+                const float m = rows4_max(mloc);
+                const float ms = m == -INFINITY ? 0.f : m;
+                float lloc = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < kPv; ks++) {
+                    const float e0 = __builtin_amdgcn_exp2f(x[ks][0] - ms), e1 = __builtin_amdgcn_exp2f(x[ks][1] - ms);
+                    const float e2 = __builtin_amdgcn_exp2f(x[ks][2] - ms), e3 = __builtin_amdgcn_exp2f(x[ks][3] - ms);
+                    lloc += (e0 + e1) + (e2 + e3);
+                    pb[ks] = make_uint2(Mma16<T>::pack2(e0, e1), Mma16<T>::pack2(e2, e3));  // hidden keys and idle rows: 0
+                    if (ks == wave) {  // the piece this wavefront hands to the score kernel, fp16 whatever the tensor dtype
+                        e_mine = make_uint2(Mma16<__half>::pack2(e0, e1), Mma16<__half>::pack2(e2, e3));
+                    }
+                }
+                m_t = m;
+                l_t = rows4_sum(lloc);
+            }
+            // ---- weighted V sum on the matrix pipe: this wavefront's dims over all keys of the tile.  Lane
+            //      16 q + g (g < G) ends up with dims 16 (kDb wave + b2) + 4 q .. + 3 of head g.
+            f32x4 acc[kDb];
+#pragma unroll
+            for (int b2 = 0; b2 < kDb; b2++) acc[b2] = f32x4{0.f, 0.f, 0.f, 0.f};
+            {
+                const uint32_t vbase = lds_base + st * kStreamStage;
+#pragma unroll
+                for (int ks = 0; ks < kPv; ks++) {
+#pragma unroll
+                    for (int b2 = 0; b2 < kDb; b2++) {
+                        const s16x4_t va = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                            (__attribute__((address_space(3))) s16x4_t*)(uintptr_t)(vbase + vt_addr[b2] + ks * 4096));
+                        uint2 av = __builtin_bit_cast(uint2, va);
+                        av.x &= m01[ks];
+                        av.y &= m23[ks];
+                        acc[b2] = Mma16<T>::mma_k16(av, pb[ks], acc[b2]);
+                    }
+                }
+            }
+            {
+                // lanes 16 q + g hold head g = key16: l_t is that head's sum (0: the tile is hidden)
+                const float inv_l = l_t > 0.f ? 1.0f / l_t : 0.f;
+#pragma unroll
+                for (int b2 = 0; b2 < kDb; b2++)
+                    pend_o[b2] = make_uint2(Mma16<T>::pack2(acc[b2][0] * inv_l, acc[b2][1] * inv_l),
+                                            Mma16<T>::pack2(acc[b2][2] * inv_l, acc[b2][3] * inv_l));
+            }
+            pend_m = m_t;
+            pend_l = l_t;
+            pend_e = e_mine;
+            pending = true;
+            pend_b = b;
+            pend_kvh = kvh;
+            b = b_nx;
+            kvh = kvh_nx;
+            st ^= 1;
+        }
+        flush();
+        // the repeated copies of the last item must land, and every wavefront be done with the stages,
+        // before the next run of items refills them
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __builtin_amdgcn_s_barrier();
+    }
+}
+
 // one workgroup per (b, h): 16 groups of 32 threads walk every 16th tile, eight tiles in flight, then merge
 // through LDS (the fp32 partial sums of the kernels that take a tile per workgroup)
 template <typename T>
@@ -1370,7 +1711,7 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
     DecodeParams p = p_in;
     const ckv_attn_args& a = p.a;
     const bool use_stream =
-        !std::is_same<T, float>::value && G <= 4 && p.shared_pos && stream_offsets_fit(a);
+        !std::is_same<T, float>::value && G <= 8 && p.shared_pos && stream_offsets_fit(a);
     if (use_stream) {
         p.tiles = (int)((p.N + kSK - 1) / kSK);  // the streaming kernel has its own tile size
         // keys that can be visible: the sinks, the leading `filled_slots` cache slots (all S when the caller gives
@@ -1399,9 +1740,12 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
                                stream, p);
         } else if (use_stream) {
             // streaming kernel: as many workgroups as run at once, items dealt out evenly
-            if constexpr (G <= 4) {
-                const int lds_s = kStreamLds;
-                if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(decode_stream_kernel<T, G>), lds_s)) return rc;
+            if constexpr (G <= 8) {
+                constexpr int lds_s = G <= 4 ? kStreamLds : kWideLds;
+                const void* kernel;
+                if constexpr (G <= 4) kernel = reinterpret_cast<const void*>(decode_stream_kernel<T, G>);
+                else kernel = reinterpret_cast<const void*>(decode_stream_wide_kernel<T, G>);
+                if (int rc = ensure_dynamic_lds(kernel, lds_s)) return rc;
                 DeviceInfo di;
                 if (int rc = current_device_info(&di)) return rc;
                 int64_t wgs = (di.cus > 0 ? di.cus : 256) * kStreamWgPerCu;
@@ -1410,11 +1754,20 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
                 p.stream_wgs = (int)wgs;
                 hipEvent_t ev0, ev1;
                 prof_kernel_events(CKV_STAGE_DECODE, &ev0, &ev1);
-                if (ev0)
-                    hipExtLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads),
-                                          (uint32_t)lds_s, stream, ev0, ev1, 0u, p);
-                else
-                    hipLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads), lds_s, stream, p);
+                if constexpr (G <= 4) {
+                    if (ev0)
+                        hipExtLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads),
+                                              (uint32_t)lds_s, stream, ev0, ev1, 0u, p);
+                    else
+                        hipLaunchKernelGGL((decode_stream_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads), lds_s, stream, p);
+                } else {
+                    if (ev0)
+                        hipExtLaunchKernelGGL((decode_stream_wide_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads),
+                                              (uint32_t)lds_s, stream, ev0, ev1, 0u, p);
+                    else
+                        hipLaunchKernelGGL((decode_stream_wide_kernel<T, G>), dim3((unsigned)wgs), dim3(kStreamThreads), lds_s,
+                                           stream, p);
+                }
             }
         } else {
             if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(decode_main_mfma_kernel<T, G>), lds)) return rc;
@@ -1426,7 +1779,7 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
     {
         StageScope sc(CKV_STAGE_DECODE_TAIL, stream);
         bool launched = false;
-        if constexpr (G <= 4 && !std::is_same<T, float>::value) {
+        if constexpr (G <= 8 && !std::is_same<T, float>::value) {
             if (use_stream) {
                 hipLaunchKernelGGL(decode_tail_stream_kernel<T>, dim3((unsigned)(a.B * a.H)), dim3(512), 0, stream, p);
                 launched = true;
@@ -1445,7 +1798,7 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
             else if (a.homogeneous_heads)
                 hipLaunchKernelGGL((decode_scores_kernel<T, G, true, false>), grid, dim3(256), 0, stream, p, w_one, (float)a.beta);
             else if (use_stream) {
-                if constexpr (G <= 4 && !std::is_same<T, float>::value) {
+                if constexpr (G <= 8 && !std::is_same<T, float>::value) {
                     const int64_t groups8 = a.B * a.KVH * (p.Np / 8);
                     hipLaunchKernelGGL((decode_scores_probs_kernel<T, G>), dim3((unsigned)((groups8 + 255) / 256)), dim3(256), 0,
                                        stream, p, w_one, (float)a.beta);
@@ -1502,9 +1855,15 @@ inline int64_t logits_area_bytes(int64_t B, int64_t H, int64_t KVH, int64_t N) {
     return align_up(std::max(B * H * N * 4, chunks * G * (kSK + kD) * 2), 256);
 }
 
+// (maximum, sum) pairs: one per head and tile, or per head and result chunk of the streaming kernels (up to one
+// chunk per workgroup more than there are items)
+inline int64_t ml_area_bytes(int64_t B, int64_t H, int64_t KVH, int64_t tiles) {
+    return align_up((B * H * tiles + std::min<int64_t>(tiles * B * KVH, kStreamMaxWgs) * (H / KVH)) * 2 * 4, 256);
+}
+
 int64_t decode_workspace_bytes(int64_t B, int64_t H, int64_t KVH, int64_t num_sink, int64_t S) {
     const int64_t N = num_sink + S + 1, tiles = (N + kMinTile - 1) / kMinTile;
-    return 2 * align_up(B * H * kD * 4, 256) + logits_area_bytes(B, H, KVH, N) + align_up(B * H * tiles * 2 * 4, 256) +
+    return 2 * align_up(B * H * kD * 4, 256) + logits_area_bytes(B, H, KVH, N) + ml_area_bytes(B, H, KVH, tiles) +
            align_up(B * H * tiles * kD * 4, 256) + align_up(B * H * 4, 256);
 }
 
@@ -1524,7 +1883,7 @@ int launch_decode(const ckv_attn_args& a, hipStream_t stream) {
     p.n_vis = 0;
     w += logits_area_bytes(a.B, a.H, a.KVH, p.N);
     const int64_t tiles_max = (p.N + kMinTile - 1) / kMinTile;
-    p.part_ml = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * tiles_max * 2 * 4, 256);
+    p.part_ml = reinterpret_cast<float*>(w); w += ml_area_bytes(a.B, a.H, a.KVH, tiles_max);
     p.part_o = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * tiles_max * kD * 4, 256);
     p.lse2 = reinterpret_cast<float*>(w);
     p.shared_pos = a.sink_pos_stride[0] == 0 && a.sink_pos_stride[1] == 0 && a.pos_stride[0] == 0 && a.pos_stride[1] == 0;

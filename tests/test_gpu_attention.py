@@ -166,7 +166,7 @@ def test_mfma_prefill_wide_range_of_logits(dtype, std):
 
 @pytest.mark.parametrize("H,KVH,W,C,NS,eager,dtype,reduction,homogeneous", [
     (8, 2, 64, 4, 8, True, torch.bfloat16, "mean", False),      # G = 4: the streaming kernel
-    (14, 2, 32, 4, 4, False, torch.bfloat16, "mean", False),    # G = 7: the tile-per-workgroup kernel
+    (14, 2, 32, 4, 4, False, torch.bfloat16, "mean", False),    # G = 7: the streaming kernel for 5 to 8 heads
     (4, 4, 32, 2, 4, True, torch.float16, "mean", False),       # G = 1
     (16, 2, 16, 8, 64, True, torch.bfloat16, "mean", False),    # G = 8
     (8, 4, 64, 2, 6, True, torch.float32, "mean", False),       # G = 2, float32
@@ -191,6 +191,9 @@ def test_decode_head128(H, KVH, W, C, NS, eager, dtype, reduction, homogeneous):
     (32, 8, torch.bfloat16, 6000),   # G = 4, cache full and evicting
     (16, 8, torch.float16, 2500),    # G = 2
     (8, 8, torch.bfloat16, 3500),    # G = 1
+    (56, 8, torch.bfloat16, 3000),   # G = 7 (the kernel for 5 to 8 heads per kv head), partly filled
+    (56, 8, torch.float16, 6000),    # G = 7, full and evicting
+    (64, 8, torch.bfloat16, 2500),   # G = 8
 ])
 def test_decode_streaming_many_items(H, KVH, dtype, fill):
     """Decode over a few thousand slots with 16 (batch, kv-head) units: more (tile, unit) items than
