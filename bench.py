@@ -112,8 +112,9 @@ def fill_to_steady_state(cache, cfg, pool, inv_freq):
 
 def update_traffic(workload, single_token=False):
     """Measured HBM bytes of one cache update: the sum over its launches (None when any figure is stale)."""
-    names = ["ckv_update_plan1_kernel"] if single_token else ["ckv_update_plan_steady_kernel", "ckv_update_plan_kernel"]
-    parts = [measured_traffic(k, workload) for k in names + ["ckv_update_apply_vec_kernel"]]
+    names = (["ckv_update_one_kernel"] if single_token else
+             ["ckv_update_plan_steady_kernel", "ckv_update_plan_kernel", "ckv_update_apply_vec_kernel"])
+    parts = [measured_traffic(k, workload) for k in names]
     return None if any(x is None for x in parts) else sum(parts)
 
 

@@ -786,6 +786,221 @@ __global__ void ckv_update_apply_vec_kernel(UpdateParams p) {
     }
 }
 
+// The whole update of a single incoming token (the decode step) in one launch.  One workgroup owns everything
+// of its (batch, kv head): wavefront 0 plans as the single-token plan kernel does (the chain of slots stays in
+// LDS: the token lands in chain[0], the old content of chain[j] in chain[j + 1], the last entry's old content is
+// dropped), writes the trackers and leaves their values after the call in LDS; then wavefront j moves the row
+// that ends in chain[j] (all rows are read before any is written) while every thread writes position ids from
+// the trackers in LDS.  No order between workgroups is needed, so plan, moves and position ids share a launch.
+// Same semantics as cascading_cache.py:381-774 for one token.  Needs 16-byte row pieces and at most kOneWaves
+// cascades.
+constexpr int kOneThreads = 1024, kOneWaves = kOneThreads / CKV_WAVE;
+// One workgroup writes all position ids of its unit, which takes as long with 8 units as with 128; the two-launch
+// path spreads them over the chip and is faster while the units are few (8 units of 64K slots: 9.4 + a launch gap
+// against 13.4 us; 128 units of 32K slots: 18 against 12.5 us).
+constexpr int kOneMinUnits = 32;
+
+__global__ void __launch_bounds__(kOneThreads) ckv_update_one_kernel(UpdateParams p) {
+    __shared__ int sh_chain[kOneWaves];
+    __shared__ int sh_n, sh_pos;
+    __shared__ int sh_stored[kOneWaves], sh_start[kOneWaves];
+    __shared__ int sh_write[kOneWaves];                     // position ids of the cascade are written
+    __shared__ unsigned sh_seg[kOneWaves], sh_add[kOneWaves];
+    __shared__ long long sh_base[kOneWaves];
+    const ckv_update_args& A = p.a;
+    const int tid = threadIdx.x, lane = tid % CKV_WAVE, wave = tid / CKV_WAVE;
+    const int64_t bh = blockIdx.x;
+    const int64_t n = bh / A.H, h = bh % A.H;
+    const int C = A.cascades;
+    const int64_t W = A.window_size, S = A.max_seq_len, NS = A.num_sink;
+    const int es = (int)elem_bytes(A.dtype);
+
+    if (wave == 0) {
+        int64_t* g_stored = A.stored_tokens + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+        int64_t* g_start = A.start_indices + n * A.tracker_stride[0] + h * A.tracker_stride[1];
+        int64_t* g_sinks = A.stored_sinks + n * A.stored_sinks_stride[0] + h * A.stored_sinks_stride[1];
+        const int64_t cs_base = n * A.cache_s_stride[0] + h * A.cache_s_stride[1];
+        const int64_t gidx = *A.real_token_idx;  // 0-based global index of the token
+        const int64_t sinks0 = *g_sinks;
+        const float tok_score = load_as_float(A.s, n * A.s_stride[0] + h * A.s_stride[1], A.dtype);
+        // lane i: cascade i; all cascades' loads travel together
+        int32_t st = 0, sx = 0;
+        int64_t per = 1;
+        float oldest = 0.f, newest = 0.f;
+        if (lane < C) {
+            st = (int32_t)g_stored[lane * A.tracker_stride[2]];
+            sx = (int32_t)g_start[lane * A.tracker_stride[2]];
+            per = A.do_cache_every_n[lane];
+            const int64_t l = (int64_t)lane * W;
+            if (st > 0) {
+                oldest = load_as_float(A.cache_s, cs_base + (l + sx) * A.cache_s_stride[2], A.dtype);
+                newest = load_as_float(A.cache_s, cs_base + (l + (sx - 1 + st) % st) * A.cache_s_stride[2], A.dtype);
+            }
+        }
+        int n_chain = 0, do_pos = 1;
+        int st_new = st, sx_new = sx;  // lane i: trackers of cascade i after the call
+        if (sinks0 < NS) {  // the token is a sink (cascading_cache.py:399-431): no position pass
+            if (lane == 0) {
+                sh_chain[0] = (int)(S + sinks0);
+                *g_sinks = sinks0 + 1;
+            }
+            n_chain = 1;
+            do_pos = 0;
+        } else {
+            float carry_score = tok_score;
+            const int64_t rel = gidx - NS;
+            const bool eager = A.eager_fill && gidx <= S + NS;
+            for (int i = 0; i < C; i++) {
+                const int32_t st_i = __shfl(st, i), sx_i = __shfl(sx, i);
+                const int64_t per_i = __shfl(per, i);
+                const int l = (int)((int64_t)i * W);
+                const bool acc = eager || (rel % per_i) == 0;
+                if (acc || st_i == 0) {
+                    const int phys = l + (int)(((int64_t)sx_i + st_i) % W);
+                    if (lane == 0) sh_chain[n_chain] = phys;
+                    n_chain++;
+                    if (st_i < (int32_t)W) {  // append (or the first entry of an empty cascade)
+                        if (lane == i) st_new = st_i + 1;
+                        if (lane == 0) g_stored[i * A.tracker_stride[2]] = st_i + 1;
+                        break;
+                    }
+                    // full: the oldest entry (at the ring start) leaves for the next cascade, or is dropped
+                    if (lane == i) sx_new = (sx_i + 1) % (int32_t)W;
+                    if (lane == 0) g_start[i * A.tracker_stride[2]] = (int64_t)((sx_i + 1) % (int32_t)W);
+                    carry_score = __shfl(oldest, i);
+                    continue;
+                }
+                // not accepted: the newest slot keeps its token unless the arrival's score is at least as large
+                if (carry_score >= __shfl(newest, i)) {
+                    if (lane == 0) sh_chain[n_chain] = l + (sx_i - 1 + st_i) % st_i;
+                    n_chain++;
+                }
+                break;
+            }
+        }
+        if (lane < C) {
+            sh_stored[lane] = st_new;
+            sh_start[lane] = sx_new;
+        }
+        if (lane == 0) {
+            sh_n = n_chain;
+            sh_pos = do_pos;
+        }
+    }
+    __syncthreads();
+    const int n_chain = sh_n;
+    const bool do_pos = sh_pos != 0;
+
+    // ---- position ids (cascading_cache.py:728-774, 129-142): per cascade the same closed form as the position
+    //      blocks of the apply kernel, from the trackers after the call
+    if (do_pos && tid < C) {
+        const int i = tid;
+        long long ub = 0;
+        for (int c = 0; c < C; c++) ub += sh_stored[c];
+        bool wr = true;
+        for (int c = 0; c < i; c++) {
+            if (sh_stored[c] <= 0) wr = false;
+            ub -= W;
+            if (ub <= 0) wr = false;
+        }
+        const long long stv = sh_stored[i];
+        const unsigned seg = (unsigned)(stv < W ? stv : W);
+        if (seg == 0) wr = false;
+        sh_write[i] = wr ? 1 : 0;
+        sh_seg[i] = seg;
+        sh_add[i] = seg - (unsigned)sh_start[i];  // start < seg or start == 0
+        sh_base[i] = ub - (long long)seg;
+    }
+
+    // ---- rows: wavefront j takes the row that ends in chain[j] (the token, or the old content of chain[j - 1])
+    const int chunks = (int)(A.HID * es / 16);
+    uint4 rk = make_uint4(0, 0, 0, 0), rv = make_uint4(0, 0, 0, 0);
+    uint32_t r_score = 0;
+    int64_t r_og = 0;
+    const bool mover = wave < n_chain;
+    const bool piece = lane < chunks;
+    char* ck = reinterpret_cast<char*>(A.cache_k) + (n * A.cache_stride[0] + h * A.cache_stride[1]) * es;
+    char* cv = reinterpret_cast<char*>(A.cache_v) + (n * A.cache_stride[0] + h * A.cache_stride[1]) * es;
+    const int64_t row_bytes = A.cache_stride[2] * es;
+    const int64_t cs_base = n * A.cache_s_stride[0] + h * A.cache_s_stride[1];
+    int64_t* og = A.og_pos + n * A.og_pos_stride[0] + h * A.og_pos_stride[1];
+    if (mover) {
+        if (wave == 0) {
+            const int64_t in_off = (n * A.kv_stride[0] + h * A.kv_stride[1]) * es;
+            if (piece) {
+                rk = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(A.k) + in_off)[lane];
+                rv = reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(A.v) + in_off)[lane];
+            }
+            if (lane == 0) {
+                const int64_t so = n * A.s_stride[0] + h * A.s_stride[1];
+                r_score = es == 4 ? reinterpret_cast<const uint32_t*>(A.s)[so] : reinterpret_cast<const uint16_t*>(A.s)[so];
+                r_og = *A.real_token_idx + 1;  // cascading_cache.py:388
+            }
+        } else {
+            const int src = sh_chain[wave - 1];
+            if (piece) {
+                rk = reinterpret_cast<const uint4*>(ck + (int64_t)src * row_bytes)[lane];
+                rv = reinterpret_cast<const uint4*>(cv + (int64_t)src * row_bytes)[lane];
+            }
+            if (lane == 0) {
+                const int64_t sidx = cs_base + (int64_t)src * A.cache_s_stride[2];
+                r_score = es == 4 ? reinterpret_cast<const uint32_t*>(A.cache_s)[sidx] : reinterpret_cast<const uint16_t*>(A.cache_s)[sidx];
+                r_og = og[(int64_t)src * A.og_pos_stride[2]];
+            }
+        }
+    }
+    __syncthreads();  // every displaced row is in registers, the position parameters are in LDS
+    if (mover) {
+        const int d = sh_chain[wave];
+        if (d >= S) {  // sink slot (cascading_cache.py:61-109); only the token itself gets here
+            const int64_t j = d - S;
+            const int64_t so = (n * A.sink_stride[0] + h * A.sink_stride[1] + j * A.sink_stride[2]) * es;
+            if (piece) {
+                reinterpret_cast<uint4*>(reinterpret_cast<char*>(A.sink_k) + so)[lane] = rk;
+                reinterpret_cast<uint4*>(reinterpret_cast<char*>(A.sink_v) + so)[lane] = rv;
+            }
+            if (lane == 0) {
+                A.sink_pos[n * A.sink_pos_stride[0] + h * A.sink_pos_stride[1] + j * A.sink_pos_stride[2]] = j;
+                A.sink_mask[n * A.sink_mask_stride[0] + h * A.sink_mask_stride[1] + j * A.sink_mask_stride[2]] = 0;
+            }
+        } else {
+            if (piece) {
+                reinterpret_cast<uint4*>(ck + (int64_t)d * row_bytes)[lane] = rk;
+                reinterpret_cast<uint4*>(cv + (int64_t)d * row_bytes)[lane] = rv;
+            }
+            if (lane == 0) {
+                const int64_t sidx = cs_base + (int64_t)d * A.cache_s_stride[2];
+                if (es == 4) reinterpret_cast<uint32_t*>(A.cache_s)[sidx] = r_score;
+                else reinterpret_cast<uint16_t*>(A.cache_s)[sidx] = (uint16_t)r_score;
+                og[(int64_t)d * A.og_pos_stride[2]] = r_og;
+                (A.mask + n * A.mask_stride[0] + h * A.mask_stride[1])[(int64_t)d * A.mask_stride[2]] = 0;
+            }
+        }
+    }
+    if (!do_pos) return;
+    int64_t* pos = A.pos + n * A.pos_stride[0] + h * A.pos_stride[1];
+    auto id_of = [&](int i, unsigned j) -> int64_t {
+        const unsigned seg = sh_seg[i];
+        unsigned x = j + sh_add[i];
+        if (x >= seg) x -= seg;
+        if (x >= seg) x %= seg;  // slots past the stored tokens of a cascade that is not full
+        return (int64_t)x + sh_base[i];
+    };
+    if (A.pos_stride[2] == 1 && (reinterpret_cast<uintptr_t>(pos) & 15u) == 0 && (W & 1) == 0) {
+        for (int i = 0; i < C; i++) {
+            if (!sh_write[i]) continue;
+            int64_t* pc = pos + (int64_t)i * W;
+            for (int64_t j = 2 * (int64_t)tid; j < W; j += 2 * kOneThreads)
+                *reinterpret_cast<longlong2*>(pc + j) = make_longlong2(id_of(i, (unsigned)j), id_of(i, (unsigned)j + 1));
+        }
+    } else {
+        for (int i = 0; i < C; i++) {
+            if (!sh_write[i]) continue;
+            for (int64_t j = tid; j < W; j += kOneThreads) pos[((int64_t)i * W + j) * A.pos_stride[2]] = id_of(i, (unsigned)j);
+        }
+    }
+}
+
 // Layouts the vector kernel cannot address (innermost stride != 1, rows not a multiple of 16
 // bytes, unaligned bases): one wavefront per token, one element at a time.
 template <typename U>
@@ -983,6 +1198,12 @@ int run_update(const ckv_update_args& A, void* workspace, hipStream_t stream) {
     p.k_sub = 0;
     p.do_pos = 0;
     p.apply_blocks = 0;
+    if (A.K == 1 && vec && A.cascades <= kOneWaves && A.HID * es / 16 <= CKV_WAVE && A.N * A.H >= kOneMinUnits) {
+        // the decode step of many streams: plan, moves and position ids of a unit by one workgroup, one launch
+        launch_timed(CKV_STAGE_APPLY, ckv_update_one_kernel, dim3((unsigned)(A.N * A.H)), dim3(kOneThreads), 0, stream, p);
+        CKV_HIP_TRY(hipGetLastError());
+        return CKV_OK;
+    }
     if (A.K >= 2) {
         // every unit first gets the chance of the steady-state plan (whole call, all cascades side by side); it
         // marks the units it has planned, the general kernel below takes the others

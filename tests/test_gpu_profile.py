@@ -48,7 +48,7 @@ def test_every_stage():
     assert st["fwd"][1] == 3 and st["scores"][1] == 3 and st["finish"][1] == 3
     assert st["decode"][1] == 4 and st["decode_tail"][1] == 4
     # a chunk's update is planned by two launches (the steady-state kernel, then the general one for the units it
-    # left), a single token's by one
+    # left), a single token's by one (with so few units)
     assert st["prep"][1] == 7 and st["plan"][1] == 3 * 2 + 4 and st["apply"][1] == 7
     assert all(ms > 0.0 for ms, n in st.values())
 

@@ -106,10 +106,23 @@ def test_chunk_longer_than_cascade_window():
     run_stream(gpu, cpu, 1500, lambda: 500, gen, torch.bfloat16, "rand")
 
 
-def test_single_token_calls():
-    gpu, cpu = make_pair(2, 4, 128, 4, 8, 4, torch.bfloat16)
+@pytest.mark.parametrize("B,H,D,NS,W,C,dtype,func,eager,mode", [
+    # 32 or more (batch, kv head) units: plan, row moves and position ids of a unit in one launch
+    (8, 4, 128, 4, 8, 4, torch.bfloat16, "pow2", True, "ties"),
+    (11, 3, 64, 7, 5, 3, torch.float32, "pow2", False, "rand"),     # odd window: position ids one by one
+    (16, 2, 128, 0, 16, 8, torch.float16, "pow2", False, "ties"),   # no sinks
+    (4, 8, 256, 2, 4, 16, torch.float32, "pow2", True, "zero"),     # 16 cascades, 64 row pieces: that kernel's limits
+    (4, 8, 16, 3, 4, 20, torch.bfloat16, "pow2", False, "ties"),    # more cascades than that: plan and apply launches
+    (4, 8, 5, 2, 4, 3, torch.float32, "pow2", True, "ties"),        # 20-byte rows: plan launch, elementwise apply kernel
+    (2, 4, 128, 4, 8, 4, torch.bfloat16, "pow2", True, "ties"),     # few units: plan and apply launches
+] + [(8, 4, 32, 4, 6, 4, torch.bfloat16, f, e, "ties") for f in CASCADE_FUNCS for e in (True, False)])
+def test_single_token_calls(B, H, D, NS, W, C, dtype, func, eager, mode):
+    """One token per call (the decode step): plan, row moves and position ids of a unit in one launch where the
+    layout allows it and the units are many, the two-launch path elsewhere; every acceptance schedule, with and
+    without eager fill."""
+    gpu, cpu = make_pair(B, H, D, NS, W, C, dtype, func, eager)
     gen = torch.Generator().manual_seed(6)
-    run_stream(gpu, cpu, 300, lambda: 1, gen, torch.bfloat16, "ties")
+    run_stream(gpu, cpu, NS + 3 * W * C + 40, lambda: 1, gen, dtype, mode)
 
 
 def test_call_larger_than_one_launch():
