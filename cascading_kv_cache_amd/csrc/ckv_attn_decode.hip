@@ -632,8 +632,8 @@ constexpr int kStreamThreads = 64 * kStreamWaves;
 constexpr int kStreamWgPerCu = 8 / kStreamWaves;  // eight wavefronts per CU
 constexpr int kStreamDimBlocks = 8 / kStreamWaves;  // 16-dim blocks of the output a wavefront owns
 constexpr int kStreamStage = 2 * kSK * 256;       // K rows then V rows of one tile (16-bit, 256 B per row)
-// two stages | per wavefront two 1 KiB query blocks | two [4 heads][kSK keys] logit planes | per wavefront [4][kSK] probabilities
-constexpr int kStreamQ = 2 * kStreamStage, kStreamS = kStreamQ + kStreamWaves * 2048, kStreamP = kStreamS + 2 * 4 * kSK * 4;
+// two stages | two 1 KiB query blocks | two [4 heads][kSK keys] logit planes | per wavefront [4][kSK] probabilities
+constexpr int kStreamQ = 2 * kStreamStage, kStreamS = kStreamQ + 2 * 1024, kStreamP = kStreamS + 2 * 4 * kSK * 4;
 constexpr int kStreamPPitch = kSK * 2 + 32;        // bytes per head row of the probabilities: the pad puts the four heads on different banks
 constexpr int kStreamLds = kStreamP + kStreamWaves * 4 * kStreamPPitch;
 
@@ -712,7 +712,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
     // query block of an item: head g at g * 256, its 16-byte piece c in slot c ^ g (the heads' rows would
     // otherwise sit on the same banks); lanes of idle MFMA rows read head 0 (their results are not used)
     const int q_row = key16 < G ? key16 : 0;
-    const int q_off = kStreamQ + wave * 2048 + q_row * 256 + ((kq ^ q_row) << 4);
+    const int q_off = kStreamQ + q_row * 256 + ((kq ^ q_row) << 4);
     float* s_all = reinterpret_cast<float*>(smem + kStreamS);                                   // [2][4][kSK]
     unsigned char* p_wave = smem + kStreamP + wave * (4 * kStreamPPitch);                       // [4][kSK] 16-bit, padded rows
 
@@ -801,16 +801,19 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                 }
             }
         };
-        // K rows and the query block of (b, kvh) into stage `st`: five copies
+        // the query block of (b, kvh) into stage `st` (one per workgroup, copied by wavefront 0: lane i fills slot
+        // i % 16 of head i / 16 with the piece that belongs there), then this wavefront's K rows.  The query copy
+        // goes first: whoever waits for the four K copies behind it has waited for it too, and the item's barrier
+        // makes it visible to the other wavefronts.
         auto copy_kq = [&](int b, int kvh, int st) {
+            if (wave == 0) {
+                const char* qsrc = (const char*)p.qrot_t + ((int64_t)b * a.H + (int64_t)kvh * G) * (kD * kEs);
+                if ((lane >> 4) < G)
+                    async_copy16(qsrc, (lane >> 4) * 256 + (((lane & 15) ^ (lane >> 4)) << 4), lds_base + kStreamQ + st * 1024);
+            }
             const char *kb[3], *vb[3];
             slabs(b, kvh, kb, vb);
             copy_rows(kb, relk, lds_base + st * kStreamStage + wave * 4096);
-            const char* qsrc = (const char*)p.qrot_t + ((int64_t)b * a.H + (int64_t)kvh * G) * (kD * kEs);
-            // lane i fills slot i % 16 of head i / 16 with the piece that belongs there
-            if ((lane >> 4) < G)
-                async_copy16(qsrc, (lane >> 4) * 256 + (((lane & 15) ^ (lane >> 4)) << 4),
-                             lds_base + kStreamQ + wave * 2048 + st * 1024);
         };
         // V rows: four copies
         auto copy_v = [&](int b, int kvh, int st) {
@@ -849,10 +852,13 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
 
         // Loads and stores retire in issue order, so "at most n operations outstanding" with n younger
         // ones issued after the wanted copies means the wanted ones are done.  Per item the order is
-        // K rows and queries of the next item (5), stores of the previous one (kDb, once there is one),
-        // V rows of the next item (4).
+        // [wavefront 0: the query block of the next item,] K rows of the next item (4), stores of the previous
+        // one (kDb and up, once there is one), V rows of the next item (4).
         copy_kq(b, kvh, 0);
         copy_v(b, kvh, 0);
+        // the first query block of the run must have landed for every wavefront (younger: the four V copies)
+        __builtin_amdgcn_s_waitcnt(0x0F74);
+        __builtin_amdgcn_s_barrier();
         int st = 0;
         // stores this wavefront issued in the latest flush(): kDb partial averages, the probabilities
         // from one wavefront, maximum and sum from another
@@ -861,6 +867,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
         auto wait_copies = [&](int younger, bool lds_too) {  // vmcnt(younger) [, lgkmcnt(0)]: the count is an immediate
             if (lds_too) {
                 switch (younger) {
+                    case 4: __builtin_amdgcn_s_waitcnt(0x0074); break;
                     case 5: __builtin_amdgcn_s_waitcnt(0x0075); break;
                     case 6: __builtin_amdgcn_s_waitcnt(0x0076); break;
                     case 7: __builtin_amdgcn_s_waitcnt(0x0077); break;
@@ -884,8 +891,8 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                 kvh_nx = kvh + 1 == KVH ? 0 : kvh + 1;
                 b_nx = kvh + 1 == KVH ? b + 1 : b;
             }
-            // K rows and queries of this item are in LDS: younger are the stores issued after them and the
-            // four V copies of this item
+            // this wavefront's K rows of the item are in LDS (younger: the stores issued after them and the four V
+            // copies of this item); the item's query block was complete before the previous barrier
             wait_copies(4 + stored, false);
             copy_kq(b_nx, kvh_nx, st ^ 1);
             stored = pending ? my_stores : 0;
@@ -927,9 +934,9 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                         s_all[(st * 4 + v) * kSK + wave * 16 + key16] = vis1 ? sacc[v] * p.scale_log2 : -INFINITY;
                 }
             }
-            // this wavefront's V rows of the item have landed (younger: the five copies of the next item's K
-            // rows and queries and the stores of flush()) and its logits are in LDS
-            wait_copies(5 + stored, true);
+            // this wavefront's V rows of the item and (wavefront 0) the next query block have landed (younger: the
+            // four K copies of the next item and the stores of flush()); its logits are in LDS
+            wait_copies(4 + stored, true);
             __builtin_amdgcn_s_barrier();
             // every wavefront is past the previous item: its V stage can be refilled
             copy_v(b_nx, kvh_nx, st ^ 1);
