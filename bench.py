@@ -444,7 +444,7 @@ def run_model(cfg, device, dtype, prompt=None):
     from cascading_kv_cache_amd.decoder import PRESETS, CascadeDecoder
     mcfg = PRESETS[cfg["preset"]]
     prompt = prompt or cfg["prompt"]
-    model = CascadeDecoder(mcfg, dtype=dtype, device=device, seed=cfg["seed"], init_on_device=True)
+    model = CascadeDecoder(mcfg, dtype=dtype, device=device, seed=cfg["seed"], init_on_device=True).fuse_projections()
     g = torch.Generator().manual_seed(cfg["seed"])
     ids = torch.randint(0, mcfg.vocab_size, (cfg["B"], prompt), generator=g).to(device)
     cache = model.new_cache(cfg["window"], cfg["cascades"], batch=cfg["B"])

@@ -50,8 +50,11 @@ class RMSNorm(nn.Module):
         super().__init__()
         self.weight = nn.Parameter(torch.ones(size, dtype=dtype, device=device))
         self.eps = eps
+        self.fused = False
 
     def forward(self, x):
+        if self.fused:  # one kernel; rounds once where the line below rounds twice
+            return nn.functional.rms_norm(x, (x.size(-1),), self.weight, self.eps)
         xf = x.float()
         xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)
         return self.weight * xf.to(x.dtype)
@@ -65,8 +68,21 @@ class GatedMLP(nn.Module):
         self.up_proj = nn.Linear(cfg.hidden_size, cfg.intermediate_size, **kw)
         self.down_proj = nn.Linear(cfg.intermediate_size, cfg.hidden_size, **kw)
 
+        self._w_gate_up = None
+
+    def fuse_projections(self):
+        """``gate_proj`` and ``up_proj`` as views of one buffer: one matrix product instead of two."""
+        with torch.no_grad():
+            w = torch.cat([self.gate_proj.weight, self.up_proj.weight], dim=0)
+            n = self.gate_proj.weight.size(0)
+            self.gate_proj.weight.data, self.up_proj.weight.data = w[:n], w[n:]
+            self._w_gate_up = w
+
     def forward(self, x):
-        return self.down_proj(nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+        if self._w_gate_up is None:
+            return self.down_proj(nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+        gate, up = nn.functional.linear(x, self._w_gate_up).chunk(2, dim=-1)
+        return self.down_proj(nn.functional.silu(gate) * up)
 
 
 class DecoderLayer(nn.Module):
@@ -106,6 +122,17 @@ class CascadeDecoder(nn.Module):
                     prm.normal_(0.0, 0.02, generator=gen)
                 else:
                     prm.copy_((torch.randn(prm.shape, generator=gen) * 0.02).to(dtype))
+
+    def fuse_projections(self):
+        """Fewer, larger launches outside attention (same weights, kept in shared buffers): q/k/v and gate/up
+        projections as one matrix product each, the norms as one kernel.  Off by default: the parity tests compare
+        the plain formulation with the CPU's."""
+        for layer in self.layers:
+            layer.self_attn.fuse_projections()
+            layer.mlp.fuse_projections()
+            layer.input_layernorm.fused = layer.post_attention_layernorm.fused = True
+        self.norm.fused = True
+        return self
 
     def new_cache(self, window, cascades, batch=1, num_sink_tokens=64, **kw):
         return CascadingKVCache(window // cascades, num_sink_tokens=num_sink_tokens, max_batch_size=batch,

@@ -40,6 +40,31 @@ class ProjectedCascadeAttention(CascadeAttention):
         self.k_proj = nn.Linear(hidden_size, num_key_value_heads * head_dim, bias=qkv_bias, **kw)
         self.v_proj = nn.Linear(hidden_size, num_key_value_heads * head_dim, bias=qkv_bias, **kw)
         self.o_proj = nn.Linear(num_heads * head_dim, hidden_size, bias=False, **kw)
+        self._w_qkv = self._b_qkv = None
+
+    def fuse_projections(self):
+        """Keep the three projection matrices in one buffer (``q_proj`` / ``k_proj`` / ``v_proj`` become views of
+        it), so that ``qkv`` is one matrix product instead of three: per token the projections are launch- and
+        bandwidth-bound, and the two small ones are the least efficient.  Same values, no extra memory."""
+        with torch.no_grad():
+            mods = (self.q_proj, self.k_proj, self.v_proj)
+            w = torch.cat([m.weight for m in mods], dim=0)
+            b = torch.cat([m.bias for m in mods], dim=0) if self.q_proj.bias is not None else None
+            at = 0
+            for m in mods:
+                n = m.weight.size(0)
+                m.weight.data = w[at:at + n]
+                if b is not None:
+                    m.bias.data = b[at:at + n]
+                at += n
+            self._w_qkv, self._b_qkv = w, b
+
+    def qkv(self, x, size, kv_size):
+        if self._w_qkv is None:
+            return super().qkv(x, size, kv_size)
+        n_q, n_kv = self.q_proj.weight.size(0), self.k_proj.weight.size(0)
+        q, k, v = nn.functional.linear(x, self._w_qkv, self._b_qkv).split((n_q, n_kv, n_kv), dim=-1)
+        return q.view(*size).transpose(1, 2), k.view(*kv_size).transpose(1, 2), v.view(*kv_size).transpose(1, 2)
 
 
 def stream_through(layer, cache, hidden, stride):

@@ -132,3 +132,30 @@ def test_generate_streams_past_the_window():
     # 500 prompt tokens + 11 fed-back tokens went through every layer (the last new token is never fed back)
     assert cache.seen_tokens_by_layer.cpu().tolist() == [511] * cfg.num_layers
     assert not bool(cache.mask[0].any()) and not bool(cache.mask[cfg.num_layers - 1].any())  # every slot holds a token
+
+
+@pytest.mark.parametrize("preset_bias", [False, True])
+def test_fused_projections_keep_the_decoder(preset_bias):
+    """q/k/v and gate/up projections as one product each (weights as views of shared buffers) and one-kernel norms:
+    the same decoder, prefill and single-token steps, up to the rounding of the norm."""
+    from dataclasses import replace
+
+    from cascading_kv_cache_amd.decoder import PRESETS, CascadeDecoder
+
+    cfg = replace(PRESETS["tiny"], qkv_bias=preset_bias)
+    dtype = torch.bfloat16
+    plain = CascadeDecoder(cfg, dtype=dtype, device="cuda:0", seed=5)
+    fused = CascadeDecoder(cfg, dtype=dtype, device="cuda:0", seed=5).fuse_projections()
+    for (n1, p1), (n2, p2) in zip(plain.named_parameters(), fused.named_parameters()):
+        assert n1 == n2 and torch.equal(p1, p2), n1
+    B, NS, W, C = 2, 4, 32, 2
+    ca, cb = (m.new_cache(W * C, C, batch=B, num_sink_tokens=NS) for m in (plain, fused))
+    ids = torch.randint(0, cfg.vocab_size, (B, 100), generator=torch.Generator().manual_seed(6)).cuda()
+    with torch.no_grad():
+        for chunk in [ids[:, 0:40], ids[:, 40:80]] + [ids[:, 80 + i:81 + i] for i in range(20)]:
+            la, lb = plain(chunk, ca).float(), fused(chunk, cb).float()
+            scale = la.abs().max().item()
+            assert (la - lb).abs().max().item() <= 2e-2 * scale + 1e-3
+    for name in ("mask", "sink_mask", "pos", "sink_pos", "stored_tokens", "start_indices", "stored_sinks"):
+        for i in range(cfg.num_layers):
+            assert torch.equal(getattr(ca, name)[i], getattr(cb, name)[i]), f"layer {i}: {name}"
