@@ -21,7 +21,7 @@ struct AttnWorkspace {
     void *qr, *kr, *vc;
     unsigned long long* tile_vis;
     uint8_t* kmasked;
-    float *lse, *lse2, *colsum, *w_ema, *w_new;
+    float *lse, *lse2, *colsum, *w_ema, *w_new, *part_o, *part_l2;
     int64_t bytes;
 };
 
@@ -40,6 +40,10 @@ AttnWorkspace carve_attn(void* base, int64_t B, int64_t H, int64_t KVH, int64_t 
     w.colsum = (float*)c.take(B * H * N * 4);
     w.w_ema = (float*)c.take((Q + kColSlack) * 4);
     w.w_new = (float*)c.take(Q * 4);
+    // shares of the forward kernel when few query rows would leave the chip idle
+    const int splits = mfma_supported(dtype, D, H, KVH, Q) && Q > 1 ? mfma_fwd_splits(B, H, KVH, Q, N) : 1;
+    w.part_o = splits > 1 ? (float*)c.take(splits * B * H * Q * D * 4) : nullptr;
+    w.part_l2 = splits > 1 ? (float*)c.take(splits * B * H * Q * 4) : nullptr;
     w.bytes = c.off;
     return w;
 }
@@ -114,6 +118,7 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
         mp.lse = w.lse;
         mp.lse2 = w.lse2;
         mp.colsum = want_scores ? w.colsum : nullptr;
+        mp.part_o = w.part_o; mp.part_l2 = w.part_l2;
         mp.w_ema = w.w_ema; mp.w_new = w.w_new;
         mp.beta = a.beta;
         mp.new_mode = 1;
@@ -228,6 +233,7 @@ extern "C" int ckv_attn_dense(const ckv_dense_args* args, void* stream_) {
         mp.lse = w.lse;
         mp.lse2 = w.lse2;
         mp.colsum = a.scores ? w.colsum : nullptr;
+        mp.part_o = w.part_o; mp.part_l2 = w.part_l2;
         mp.w_ema = w.w_ema; mp.w_new = w.w_new;
         mp.beta = a.beta;
         mp.new_mode = 0;  // every key is weighted by the query row alone (flash_attention.py:73-77)

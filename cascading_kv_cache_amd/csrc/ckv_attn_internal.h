@@ -94,6 +94,8 @@ struct MfmaProblem {
     float* lse;            // (B, H, Q) natural log
     float* lse2;           // (B*H*Q + kColSlack) scratch: minus the log2-domain normaliser, for the column pass
     float* colsum;         // (B, H, n) or null
+    float* part_o;         // (mfma_fwd_splits, B*H*Q, D) and
+    float* part_l2;        // (mfma_fwd_splits, B*H*Q): the forward kernel's shares, when it splits the keys
     const float* w_ema;
     const float* w_new;
     double beta;           // the EMA factor the weights were built from
@@ -105,6 +107,7 @@ struct MfmaProblem {
 
 bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH, int64_t Q);
 int64_t mfma_n_pad(int64_t n);
+int mfma_fwd_splits(int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t n);  // shares of the key tiles per query tile
 bool mfma_fits(int64_t n);  // the per-tile bookkeeping of n keys fits in LDS
 int launch_mfma(const MfmaProblem& p, hipStream_t stream);
 

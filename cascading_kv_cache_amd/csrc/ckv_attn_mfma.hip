@@ -408,6 +408,12 @@ struct FwdParams {
     int G;            // heads per kv head: a workgroup takes 256 consecutive rows of the kv head's (position, head) pairs, position-major
     float scale_log2; // softmax scale * log2(e)
     int n_qt, xcd_aware;  // query tiles per kv head; 1-D XCD-aware block order
+    // Few query rows (short chunks, one stream) would leave most of the chip idle: the key tiles of a query tile
+    // are then dealt out over n_split workgroups, each of which leaves a partial result (its rows normalised by
+    // its own sums, fp32) and the log2-domain normaliser of its share; a small kernel merges them.
+    int n_split;
+    float* part_o;    // (n_split, B*H*Q, D)
+    float* part_l2;   // (n_split, B*H*Q): m_ref + log2(l) of the share, -inf when it holds no visible key
 };
 
 // LDS tile of 256-byte rows taken from a row-major matrix (the query tile of the column pass): unpadded
@@ -447,10 +453,12 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
     // head are put on one XCD, so its K / V^T stream is fetched from HBM into one L2 instead of eight
     // (same run time, a fifth of the HBM reads).
     if (p.xcd_aware) {
-        const int id = blockIdx.x, jq = id >> 3;
-        bkv_i = (id & 7) + 8 * (jq / p.n_qt);
-        qt_i = jq % p.n_qt;
+        const int id = blockIdx.x, jq = id >> 3, per = p.n_qt * p.n_split;
+        bkv_i = (id & 7) + 8 * (jq / per);
+        qt_i = jq % per;
     }
+    const int split_i = qt_i % p.n_split;   // this workgroup's share of the query tile's key tiles
+    qt_i /= p.n_split;
     // Later query tiles see more chunk keys, so they go first: the compute units that finish the light
     // tiles of one round early pick up the heavy tiles of the next (two rounds of workgroups then cost
     // light + heavy everywhere instead of heavy + heavy on the slowest unit).
@@ -487,7 +495,10 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
         if (lane == 0) list_lds[tiles_cap] = cnt;
     }
     __syncthreads();
-    const int n_work = __builtin_amdgcn_readfirstlane(list_lds[tiles_cap]);
+    const int n_work_all = __builtin_amdgcn_readfirstlane(list_lds[tiles_cap]);
+    const int j_first = n_work_all * split_i / p.n_split;
+    const int n_work = n_work_all * (split_i + 1) / p.n_split - j_first;
+    list_lds += j_first;
 
     // ---- the query row this lane owns as MFMA column `col`
     int row_m;
@@ -787,6 +798,26 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
 
     // epilogue: lane owns d = 32dt + 8(v/4) + 4half + v%4 of its query row
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (p.n_split > 1) {
+        // a share of the key tiles: the row normalised by the share's own sum, and the share's normaliser
+        const int rf_p = qt_i * kRows + wave * 32 + col;
+        const int64_t row_p = (b * p.H + kvh * p.G + rf_p % p.G) * p.Q + row_m;
+        if (row_m < p.Q) {
+            const bool any = l_tot > 0.f;
+            const float inv_p = any ? 1.f / l_tot : 0.f;
+            float* po = p.part_o + ((int64_t)split_i * p.B * p.H * p.Q + row_p) * kD;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int v4 = 0; v4 < 4; v4++)
+                    *reinterpret_cast<float4*>(po + 32 * dt + 8 * v4 + 4 * half) =
+                        make_float4(oacc[dt][4 * v4] * inv_p, oacc[dt][4 * v4 + 1] * inv_p, oacc[dt][4 * v4 + 2] * inv_p,
+                                    oacc[dt][4 * v4 + 3] * inv_p);
+            if (half == 0)
+                p.part_l2[(int64_t)split_i * p.B * p.H * p.Q + row_p] = any ? m_ref + __builtin_amdgcn_logf(l_tot) : -INFINITY;
+        }
+        return;
+    }
     const int g_row = (qt_i * kRows + wave * 32 + col) % p.G;
     const int64_t row_h = kvh * p.G + g_row;
     const bool row_ok = row_m < p.Q;
@@ -841,6 +872,39 @@ __global__ void __launch_bounds__(512) fwd_pipe_kernel(FwdParams p) {
             p.lse[(b * p.H + row_h) * p.Q + row_m] = l2 * 0.6931471805599453f;
             p.lse2[(b * p.H + row_h) * p.Q + row_m] = -l2;
         }
+    }
+}
+
+// Merge of the forward kernel's shares: one row per 32 lanes (4 dims each), 8 rows per workgroup.
+template <typename T>
+__global__ void __launch_bounds__(256) fwd_combine_kernel(FwdParams p) {
+    const int64_t rows = p.B * p.H * p.Q;
+    const int64_t row = (int64_t)blockIdx.x * 8 + threadIdx.x / 32;
+    if (row >= rows) return;
+    const int d4 = threadIdx.x % 32;
+    float M = -INFINITY;
+    for (int s_ = 0; s_ < p.n_split; s_++) M = fmaxf(M, p.part_l2[s_ * rows + row]);
+    float L = 0.f;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s_ = 0; s_ < p.n_split; s_++) {
+        const float l2 = p.part_l2[s_ * rows + row];
+        if (l2 == -INFINITY) continue;
+        const float w = __builtin_amdgcn_exp2f(l2 - M);
+        const float4 v = *reinterpret_cast<const float4*>(p.part_o + (s_ * rows + row) * kD + 4 * d4);
+        L += w;
+        o.x = fmaf(v.x, w, o.x); o.y = fmaf(v.y, w, o.y); o.z = fmaf(v.z, w, o.z); o.w = fmaf(v.w, w, o.w);
+    }
+    const float inv = 1.f / L;
+    const int64_t m = row % p.Q, h = (row / p.Q) % p.H, b = row / (p.Q * p.H);
+    T* dst = (T*)p.out + b * p.out_stride[0] + h * p.out_stride[1] + m * p.out_stride[2];
+    dst[(4 * d4) * p.out_stride[3]] = Elem<T>::from_float(o.x * inv);
+    dst[(4 * d4 + 1) * p.out_stride[3]] = Elem<T>::from_float(o.y * inv);
+    dst[(4 * d4 + 2) * p.out_stride[3]] = Elem<T>::from_float(o.z * inv);
+    dst[(4 * d4 + 3) * p.out_stride[3]] = Elem<T>::from_float(o.w * inv);
+    if (d4 == 0) {
+        const float l2 = M + __builtin_amdgcn_logf(L);  // v_log_f32 is log2
+        p.lse[row] = l2 * 0.6931471805599453f;
+        p.lse2[row] = -l2;
     }
 }
 
@@ -1274,10 +1338,14 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         fp.B = mp.B; fp.H = mp.H; fp.KVH = mp.KVH; fp.Q = mp.Q; fp.N = n; fp.Nc = n - mp.Q; fp.n_pad = n_pad;
         fp.G = G;
         fp.scale_log2 = 1.f;  // already on the staged queries
-        const dim3 grid((unsigned)((mp.Q * G + kRows - 1) / kRows), (unsigned)(mp.B * mp.KVH));
+        fp.n_qt = (int)((mp.Q * G + kRows - 1) / kRows);
+        fp.n_split = mfma_fwd_splits(mp.B, mp.H, mp.KVH, mp.Q, n);
+        fp.part_o = mp.part_o;
+        fp.part_l2 = mp.part_l2;
+        if (fp.n_split > 1 && (!fp.part_o || !fp.part_l2)) return CKV_ERR_WORKSPACE;
+        const dim3 grid((unsigned)(fp.n_qt * fp.n_split), (unsigned)(mp.B * mp.KVH));
         const int lds = pipe_lds_bytes(n_pad);
         if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fwd_pipe_kernel<T>), lds)) return rc;
-        fp.n_qt = (int)grid.x;
         fp.xcd_aware = grid.y % 8 == 0;
         hipEvent_t ev0, ev1;
         prof_kernel_events(CKV_STAGE_FWD, &ev0, &ev1);
@@ -1285,6 +1353,11 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         if (ev0) hipExtLaunchKernelGGL(fwd_pipe_kernel<T>, launch_grid, dim3(512), (uint32_t)lds, stream, ev0, ev1, 0u, fp);
         else hipLaunchKernelGGL(fwd_pipe_kernel<T>, launch_grid, dim3(512), lds, stream, fp);
         CKV_HIP_TRY(hipGetLastError());
+        if (fp.n_split > 1) {
+            const int64_t rows = mp.B * mp.H * mp.Q;
+            hipLaunchKernelGGL(fwd_combine_kernel<T>, dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, stream, fp);
+            CKV_HIP_TRY(hipGetLastError());
+        }
     }
     if (mp.colsum) {
         StageScope sc(CKV_STAGE_SCORES, stream);
@@ -1338,6 +1411,19 @@ bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH, int64_t Q) {
 }
 
 int64_t mfma_n_pad(int64_t n) { return align_up(n, 256); }
+
+// Shares of a query tile's key tiles (1: no splitting).  A function of the shapes alone, so that the workspace
+// can be sized for it: the chip is taken to hold 256 workgroups of the forward kernel at once; fewer than that
+// are topped up to about 512, with at least 16 key tiles per share and at most 8 shares.
+int mfma_fwd_splits(int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t n) {
+    const int64_t G = H / KVH;
+    const int64_t wgs = ((Q * G + kRows - 1) / kRows) * B * KVH, tiles = (n + kBN - 1) / kBN;
+    if (wgs >= 256) return 1;
+    int64_t s_ = 512 / wgs;
+    if (s_ > tiles / 16) s_ = tiles / 16;
+    if (s_ > 8) s_ = 8;
+    return s_ < 1 ? 1 : (int)s_;
+}
 
 // the forward kernel keeps per-tile bookkeeping of all N keys in LDS
 bool mfma_fits(int64_t n) { return pipe_lds_bytes(mfma_n_pad(n)) <= kLdsLimit; }

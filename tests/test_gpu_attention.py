@@ -136,6 +136,20 @@ def test_mfma_prefill_head128(H, KVH, Q, W, C, NS, eager, dtype, reduction, homo
     assert led.flips <= 0.05 * led.compared, led.summary()
 
 
+@pytest.mark.parametrize("H,KVH,Q,W,C,dtype,eager", [
+    (8, 2, 320, 1024, 4, torch.bfloat16, True),     # 10 workgroups' worth of rows against 4160 slots: 4 shares
+    (14, 2, 256, 512, 8, torch.float16, False),     # G = 7
+    (4, 4, 512, 2048, 2, torch.bfloat16, True),     # G = 1
+])
+def test_mfma_prefill_short_chunks_split_the_keys(H, KVH, Q, W, C, dtype, eager):
+    """Short chunks of one or two streams against a few thousand slots: too few query rows to fill the chip, so the
+    forward kernel deals the key tiles of a query tile out over several workgroups and a second kernel merges their
+    shares.  The stream runs from the empty cache (shares without a visible key) until the cascades evict."""
+    chunks = (64 + W * C) // Q + 3
+    led = run_teacher_forced(1, H, KVH, 128, 64, W, C, Q, chunks, dtype, seed=31, eager=eager, std=0.7, q_last=Q - 11)
+    assert led.flips <= 0.05 * led.compared, led.summary()
+
+
 @pytest.mark.parametrize("dtype,std", [(torch.bfloat16, 0.05), (torch.bfloat16, 1.0), (torch.bfloat16, 3.0),
                                        (torch.float16, 2.5), (torch.bfloat16, 6.0)])
 def test_mfma_prefill_wide_range_of_logits(dtype, std):
