@@ -86,6 +86,7 @@ def job_latency(window=16384, cascades=4, cascade_stride=4096, lengths=None, hea
     torch.manual_seed(seed)
     layer = ProjectedCascadeAttention(hidden_size, num_heads, num_key_value_heads, head_dim,
                                       head_reduction=head_reduction, dtype=dtype, device=device)
+    layer.fuse_projections()  # q, k, v as one product
     results = []
     with torch.no_grad():
         for length in lengths:
