@@ -136,6 +136,40 @@ def test_mfma_prefill_head128(H, KVH, Q, W, C, NS, eager, dtype, reduction, homo
     assert led.flips <= 0.05 * led.compared, led.summary()
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_head128_streams(seed):
+    """Random shapes on the matrix-core and single-token kernels: heads per kv head 1, 2, 4, 7 or 8, ragged
+    chunk lengths from one token to several hundred mixed in one stream, windows from a few tiles to a few
+    thousand slots, with and without eager fill, every head reduction."""
+    import random
+
+    rng = random.Random(1000 + seed)
+    G = rng.choice([1, 2, 4, 7, 8])
+    KVH = rng.choice([1, 2, 4])
+    B = rng.choice([1, 2])
+    W = rng.choice([16, 64, 200, 512, 1024])
+    C = rng.choice([1, 2, 4, 8])
+    NS = rng.choice([3, 4, 64])   # the reference's prologue needs at least one sink (cascade_attention.py:145-148)
+    dtype = rng.choice([torch.bfloat16, torch.float16])
+    eager = rng.random() < 0.6
+    reduction = rng.choice(["mean", "max", "median"])
+    homogeneous = rng.random() < 0.25
+    total = NS + W * C
+    steps, done = [], 0
+    while done < total + 2 * W and len(steps) < 24:
+        kind = rng.random()
+        q = 1 if kind < 0.35 else (rng.randint(2, 40) if kind < 0.5 else rng.randint(41, max(64, min(700, total // 2))))
+        steps.append(q)
+        done += q
+    big = steps.index(max(steps))   # the reference sizes its query positions by the first chunk (cascade_attention.py:120-123)
+    steps[0], steps[big] = steps[big], steps[0]
+    print(f"seed={seed} B={B} H={G * KVH} KVH={KVH} W={W} C={C} NS={NS} {dtype} eager={eager} {reduction} "
+          f"homogeneous={homogeneous} steps={steps}", flush=True)
+    led = run_teacher_forced(B, G * KVH, KVH, 128, NS, W, C, 0, 0, dtype, seed=seed, reduction=reduction,
+                             homogeneous=homogeneous, eager=eager, std=0.7, steps=steps)
+    assert led.flips <= 0.05 * led.compared, led.summary()
+
+
 @pytest.mark.parametrize("H,KVH,Q,W,C,dtype,eager", [
     (8, 2, 320, 1024, 4, torch.bfloat16, True),     # 10 workgroups' worth of rows against 4160 slots: 4 shares
     (14, 2, 256, 512, 8, torch.float16, False),     # G = 7
