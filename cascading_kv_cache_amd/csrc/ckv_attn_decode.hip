@@ -1713,6 +1713,86 @@ __global__ void __launch_bounds__(256) decode_scores_probs_kernel(DecodeParams p
     }
 }
 
+// All heads reduced together (cascade_attention.py:240-242) after a streaming kernel: one thread per (batch, key),
+// a workgroup per 128-key tile, so that the factor 2^(tile maximum - normaliser) of every head is worked out once
+// per workgroup.  The thread walks the H heads in order (kv head major, as repeat_kv lays them out), keeps a running
+// sum or maximum, or parks the H values in its LDS column and finds the lower median by counting, and writes the
+// result to the score row of every kv head.
+constexpr int kHomoMaxHeads = 64;
+
+template <typename T, int G>
+__global__ void __launch_bounds__(kSK) decode_scores_homo_kernel(DecodeParams p, float w_one, float beta_pow) {
+    __shared__ float sh_c[kHomoMaxHeads];
+    __shared__ int64_t sh_ck[kHomoMaxHeads / G + 1];
+    __shared__ float sh_v[kHomoMaxHeads][kSK];   // median only
+    const ckv_attn_args& a = p.a;
+    const int tile = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+    const int H = (int)a.H, KVH = (int)a.KVH;
+    const int64_t n = (int64_t)tile * kSK + tid;
+    const int jt = stream_rank_of(p, tile);  // -1: no key of the tile is visible, every probability is 0
+    if (tid < H) {
+        const int kv = tid / G, g = tid % G;
+        float c = 0.f;
+        if (jt >= 0) {
+            const int64_t ck = stream_chunk_of((int64_t)jt * (a.B * KVH) + (int64_t)b * KVH + kv, (int64_t)p.n_vis * (a.B * KVH),
+                                               p.stream_wgs);
+            c = __builtin_amdgcn_exp2f(p.part_ml[(ck * G + g) * 2] - p.lse2[(int64_t)b * H + tid]);
+            if (g == 0) sh_ck[kv] = ck;
+        }
+        sh_c[tid] = c;
+    }
+    __syncthreads();
+    if (n < a.num_sink || n >= p.N) return;  // sinks keep no score; padding of the last tile
+    const bool is_new = n == p.N - 1;
+    const float w = is_new ? round_t<T>(w_one) : w_one;  // the new token's weight is built in the tensor dtype
+    const int mode = a.head_reduction;
+    float acc = mode == CKV_REDUCE_MAX ? -INFINITY : 0.f;
+    for (int h = 0; h < H; h++) {
+        float pt = 0.f;
+        if (jt >= 0) {
+            const unsigned char* chunk = p.chunks + sh_ck[h / G] * (G * (kSK + kD) * 2);
+            const float e = (float)reinterpret_cast<const _Float16*>(chunk)[(h % G) * kSK + tid];
+            pt = e == 0.f ? 0.f : round_t<T>(e * sh_c[h]);
+        }
+        const float v = round_t<T>(__fmul_rn(pt, w));
+        if (mode == CKV_REDUCE_MAX) acc = h == 0 ? v : fmaxf(acc, v);
+        else if (mode == CKV_REDUCE_MEAN) acc = __fadd_rn(acc, v);
+        else sh_v[h][tid] = v;
+    }
+    float red;
+    if (mode == CKV_REDUCE_MAX) {
+        red = acc;
+    } else if (mode == CKV_REDUCE_MEAN) {
+        red = round_t<T>(acc / (float)H);
+    } else {  // lower median: the value with at most (H-1)/2 values below it and more than that below or equal
+        red = sh_v[0][tid];
+        const int k = (H - 1) / 2;
+        for (int i = 0; i < H; i++) {
+            const float x = sh_v[i][tid];
+            int below = 0, equal = 0;
+            for (int j = 0; j < H; j++) {
+                const float y = sh_v[j][tid];
+                below += y < x;
+                equal += y == x;
+            }
+            if (below <= k && k < below + equal) red = x;
+        }
+    }
+    if (is_new) {
+        if (a.new_scores)
+            for (int kv = 0; kv < KVH; kv++)
+                *((T*)a.new_scores + b * a.new_scores_stride[0] + kv * a.new_scores_stride[1]) = Elem<T>::from_float(red);
+    } else if (a.cache_s) {
+        const int rows = a.cache_s_stride[1] == 0 ? 1 : KVH;  // one shared row or one per kv head
+        const int64_t i = n - a.num_sink;
+        for (int kv = 0; kv < rows; kv++) {
+            T* cs = (T*)a.cache_s + b * a.cache_s_stride[0] + kv * a.cache_s_stride[1] + i * a.cache_s_stride[2];
+            const float decayed = round_t<T>(__fmul_rn(beta_pow, Elem<T>::to_float(*cs)));
+            *cs = Elem<T>::from_float(__fadd_rn(decayed, red));
+        }
+    }
+}
+
 template <typename T, int G>
 int run_decode(const DecodeParams& p_in, hipStream_t stream) {
     DecodeParams p = p_in;
@@ -1800,7 +1880,11 @@ int run_decode(const DecodeParams& p_in, hipStream_t stream) {
             const float w_one = (float)(1.0 - a.beta);
             const int64_t items = a.B * a.KVH * (a.S + 1);
             const dim3 grid((unsigned)((items + 255) / 256));
-            if (a.homogeneous_heads && use_stream)
+            if (a.homogeneous_heads && use_stream && a.H <= kHomoMaxHeads) {
+                if constexpr (G <= 8 && !std::is_same<T, float>::value)
+                    hipLaunchKernelGGL((decode_scores_homo_kernel<T, G>), dim3((unsigned)p.tiles, (unsigned)a.B), dim3(kSK), 0, stream,
+                                       p, w_one, (float)a.beta);
+            } else if (a.homogeneous_heads && use_stream)
                 hipLaunchKernelGGL((decode_scores_kernel<T, G, true, true>), grid, dim3(256), 0, stream, p, w_one, (float)a.beta);
             else if (a.homogeneous_heads)
                 hipLaunchKernelGGL((decode_scores_kernel<T, G, true, false>), grid, dim3(256), 0, stream, p, w_one, (float)a.beta);
