@@ -7,8 +7,9 @@
  *   _update_kv_cache_inner  cascade/models/cascading_cache.py:302-774
  *   _update_sink_cache      cascade/models/cascading_cache.py:22-109
  *   _update_positional_idx  cascade/models/cascading_cache.py:112-142
- * It takes the product's argument struct (include/ckv.h) with HOST pointers so a test can
- * hand the same description to both sides.
+ * It has an argument block of its own (`oracle_update_desc` below: one {pointer, strides} record
+ * per tensor, filled by oracle/update.py) and shares no header and no marshalling code with the
+ * library under test, so a wrong stride or field on the product's side cannot reach both sides.
  *
  * Pinned by tests/test_oracle_update.py (closed forms for sinks and metadata, the C=1
  * StreamingLLM special case, the eager-fill rule, split-call invariance, a restatement of the
@@ -18,15 +19,53 @@
 #include <stdint.h>
 #include <string.h>
 
-#include "../include/ckv.h"
+/* dtype codes and status values of the oracle (its own; the Python face maps torch dtypes to them) */
+enum { ORACLE_F32 = 0, ORACLE_F16 = 1, ORACLE_BF16 = 2 };
+enum { ORACLE_OK = 0, ORACLE_ERR_NULL = 1, ORACLE_ERR_DTYPE = 2, ORACLE_ERR_SHAPE = 3 };
+
+/* a host tensor: base pointer and element strides, outermost dimension first (unused entries 0) */
+typedef struct oracle_tensor {
+    void* ptr;
+    int64_t stride[4];
+} oracle_tensor;
+
+/* the arguments of sink_cache (cascading_cache.py:962-985) in the order of that signature */
+typedef struct oracle_update_desc {
+    oracle_tensor k, v, s;                         /* (N, H, K, HID) x2, (N, >=H, K)              */
+    oracle_tensor sink_k, sink_v;                  /* (N, H, num_sink, HID)                       */
+    oracle_tensor sink_mask, sink_pos;             /* (N, H, num_sink) bool / int64               */
+    oracle_tensor cache_k, cache_v, cache_s;       /* (N, H, S, HID) x2, (N, H, S)                */
+    oracle_tensor mask, pos, og_pos;               /* (N, H, S) bool / int64 / int64              */
+    oracle_tensor do_cache_every_n;                /* (cascades,) int64                           */
+    oracle_tensor stored_tokens, start_indices;    /* (N, H, cascades) int64                      */
+    oracle_tensor stored_sinks;                    /* (N, H) int64                                */
+    int64_t num_sink, window_size, real_token_idx, max_seq_len;
+    int64_t eager_fill;
+    int64_t n, h, k_len, hid, cascades;            /* sizes of k and of the trackers              */
+    int64_t dtype;                                 /* ORACLE_F32 / F16 / BF16                     */
+} oracle_update_desc;
+
+/* The body below is written against flat names; this view gives them from the per-tensor records. */
+typedef struct oracle_view {
+    const void *k, *v, *s;
+    void *sink_k, *sink_v, *cache_k, *cache_v, *cache_s;
+    uint8_t *sink_mask, *mask;
+    int64_t *sink_pos, *pos, *og_pos, *stored_sinks, *stored_tokens, *start_indices;
+    const int64_t* do_cache_every_n;
+    const int64_t *kv_stride, *s_stride, *sink_stride, *cache_stride, *cache_s_stride, *sink_mask_stride,
+        *mask_stride, *sink_pos_stride, *pos_stride, *og_pos_stride, *stored_sinks_stride, *tracker_stride;
+    int64_t every_n_stride;
+    int64_t N, H, K, HID, num_sink, window_size, max_seq_len, cascades, seen;
+    int eager_fill, dtype;
+} oracle_view;
 
 static float oracle_load_score(const void* base, int64_t idx, int dtype) {
-    if (dtype == CKV_F32) {
+    if (dtype == ORACLE_F32) {
         return ((const float*)base)[idx];
     }
     uint16_t h = ((const uint16_t*)base)[idx];
     uint32_t bits;
-    if (dtype == CKV_BF16) {
+    if (dtype == ORACLE_BF16) {
         bits = (uint32_t)h << 16;
     } else { /* IEEE binary16 -> binary32, exact */
         uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
@@ -54,7 +93,7 @@ static float oracle_load_score(const void* base, int64_t idx, int dtype) {
     return f;
 }
 
-static int64_t elem_size(int dtype) { return dtype == CKV_F32 ? 4 : 2; }
+static int64_t elem_size(int dtype) { return dtype == ORACLE_F32 ? 4 : 2; }
 
 /* one row of HID elements, arbitrary strides */
 static void copy_row(void* dst, int64_t dst_off, int64_t dst_sh, const void* src, int64_t src_off,
@@ -65,13 +104,36 @@ static void copy_row(void* dst, int64_t dst_off, int64_t dst_sh, const void* src
     }
 }
 
-int ckv_oracle_update(const ckv_update_args* a) {
-    if (!a) return CKV_ERR_NULL;
-    if (a->dtype != CKV_F32 && a->dtype != CKV_F16 && a->dtype != CKV_BF16) return CKV_ERR_DTYPE;
+int ckv_oracle_update(const oracle_update_desc* d) {
+    if (!d) return ORACLE_ERR_NULL;
+    oracle_view view;
+    view.k = d->k.ptr; view.v = d->v.ptr; view.s = d->s.ptr;
+    view.sink_k = d->sink_k.ptr; view.sink_v = d->sink_v.ptr;
+    view.cache_k = d->cache_k.ptr; view.cache_v = d->cache_v.ptr; view.cache_s = d->cache_s.ptr;
+    view.sink_mask = (uint8_t*)d->sink_mask.ptr; view.mask = (uint8_t*)d->mask.ptr;
+    view.sink_pos = (int64_t*)d->sink_pos.ptr; view.pos = (int64_t*)d->pos.ptr; view.og_pos = (int64_t*)d->og_pos.ptr;
+    view.stored_sinks = (int64_t*)d->stored_sinks.ptr;
+    view.stored_tokens = (int64_t*)d->stored_tokens.ptr; view.start_indices = (int64_t*)d->start_indices.ptr;
+    view.do_cache_every_n = (const int64_t*)d->do_cache_every_n.ptr;
+    view.every_n_stride = d->do_cache_every_n.stride[0];
+    /* k and v, the two sink tensors, the two cache tensors and the two trackers are each walked with one
+     * set of strides, as the reference kernel does (cascading_cache.py:846-891 passes k's, sink_k's,
+     * cache_k's and stored_tokens' strides only); the Python face refuses pairs that differ */
+    view.kv_stride = d->k.stride; view.s_stride = d->s.stride; view.sink_stride = d->sink_k.stride;
+    view.cache_stride = d->cache_k.stride; view.cache_s_stride = d->cache_s.stride;
+    view.sink_mask_stride = d->sink_mask.stride; view.mask_stride = d->mask.stride;
+    view.sink_pos_stride = d->sink_pos.stride; view.pos_stride = d->pos.stride; view.og_pos_stride = d->og_pos.stride;
+    view.stored_sinks_stride = d->stored_sinks.stride; view.tracker_stride = d->stored_tokens.stride;
+    view.N = d->n; view.H = d->h; view.K = d->k_len; view.HID = d->hid;
+    view.num_sink = d->num_sink; view.window_size = d->window_size; view.max_seq_len = d->max_seq_len;
+    view.cascades = d->cascades; view.seen = d->real_token_idx;
+    view.eager_fill = d->eager_fill != 0; view.dtype = (int)d->dtype;
+    const oracle_view* a = &view;
+    if (a->dtype != ORACLE_F32 && a->dtype != ORACLE_F16 && a->dtype != ORACLE_BF16) return ORACLE_ERR_DTYPE;
     const int64_t es = elem_size(a->dtype);
     const int64_t W = a->window_size, C = a->cascades, NS = a->num_sink, S = a->max_seq_len;
-    if (W <= 0 || C <= 0 || C * W != S || a->HID <= 0 || a->HID > 4096) return CKV_ERR_SHAPE;
-    const int64_t seen = *a->real_token_idx;
+    if (W <= 0 || C <= 0 || C * W != S || a->HID <= 0 || a->HID > 4096) return ORACLE_ERR_SHAPE;
+    const int64_t seen = a->seen;
 
     /* the carried row lives here between cascades (cascading_cache.py:589-593) */
     char ck[4096 * 4], cv[4096 * 4], tk[4096 * 4], tv[4096 * 4], cs[4], ts[4];
@@ -116,7 +178,7 @@ int ckv_oracle_update(const ckv_update_args* a) {
                     const int64_t l = i * W;
                     int accept = always;
                     if (!accept) { /* cascading_cache.py:474-478 */
-                        accept = ((rti - 1 - NS) % a->do_cache_every_n[i]) == 0;
+                        accept = ((rti - 1 - NS) % a->do_cache_every_n[i * a->every_n_stride]) == 0;
                     }
                     const int64_t st = stored[i * st_c], sx = start[i * st_c];
                     int64_t slot;
@@ -175,7 +237,7 @@ int ckv_oracle_update(const ckv_update_args* a) {
                 for (int64_t i = 0; i < C; i++) {
                     const int64_t st = stored[i * st_c], sx = start[i * st_c];
                     const int64_t seg = st < W ? st : W; /* :130 */
-                    if (seg <= 0) return CKV_ERR_SHAPE;   /* the reference would divide by zero */
+                    if (seg <= 0) return ORACLE_ERR_SHAPE;   /* the reference would divide by zero */
                     for (int64_t j = 0; j < W; j++) {     /* :132-142 */
                         a->pos[p_base + (i * W + j) * a->pos_stride[2]] = ((j + seg - sx) % seg) + ub - seg;
                     }
@@ -185,5 +247,8 @@ int ckv_oracle_update(const ckv_update_args* a) {
             }
         }
     }
-    return CKV_OK;
+    return ORACLE_OK;
 }
+
+/* lets the Python face check that its ctypes mirror of oracle_update_desc has the same size */
+int64_t ckv_oracle_sizeof_desc(void) { return (int64_t)sizeof(oracle_update_desc); }

@@ -13,11 +13,65 @@ import os
 
 import torch
 
-from cascading_kv_cache_amd._abi import UpdateArgs, fill_update_args
-
 from . import build as _build
 
 _LIB = None
+
+ORACLE_DTYPE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+class OracleTensor(C.Structure):
+    """``oracle_tensor`` of ckv_oracle_update.c: base pointer and element strides, outermost first."""
+    _fields_ = [("ptr", C.c_void_p), ("stride", C.c_int64 * 4)]
+
+
+_TENSOR_FIELDS = ("k", "v", "s", "sink_k", "sink_v", "sink_mask", "sink_pos", "cache_k", "cache_v", "cache_s",
+                  "mask", "pos", "og_pos", "do_cache_every_n", "stored_tokens", "start_indices", "stored_sinks")
+_SCALAR_FIELDS = ("num_sink", "window_size", "real_token_idx", "max_seq_len", "eager_fill", "n", "h", "k_len", "hid",
+                  "cascades", "dtype")
+
+
+class OracleUpdateDesc(C.Structure):
+    """``oracle_update_desc`` of ckv_oracle_update.c: the arguments of ``sink_cache`` in the order of its
+    signature (cascading_cache.py:962-985).  Deliberately not the library's argument struct: the oracle is
+    described by code of its own, so a marshalling mistake on the product's side cannot cancel out."""
+    _fields_ = [(name, OracleTensor) for name in _TENSOR_FIELDS] + [(name, C.c_int64) for name in _SCALAR_FIELDS]
+
+
+def describe_update(k, v, s, sink_k, sink_v, sink_mask, sink_pos, cache_k, cache_v, cache_s, mask, pos, og_pos,
+                    do_cache_every_n, stored_tokens, start_indices, stored_sinks, num_sink, window_size,
+                    real_token_idx, max_seq_len, eager_fill) -> OracleUpdateDesc:
+    """One record per tensor, taken from the tensor itself.  The reference kernel walks k and v, the two sink
+    tensors, the two cache tensors and the two trackers with one set of strides each
+    (cascading_cache.py:846-891), so pairs whose stepped strides differ are refused here."""
+    tensors = dict(k=k, v=v, s=s, sink_k=sink_k, sink_v=sink_v, sink_mask=sink_mask, sink_pos=sink_pos,
+                   cache_k=cache_k, cache_v=cache_v, cache_s=cache_s, mask=mask, pos=pos, og_pos=og_pos,
+                   do_cache_every_n=do_cache_every_n, stored_tokens=stored_tokens, start_indices=start_indices,
+                   stored_sinks=stored_sinks)
+    for a, b in (("k", "v"), ("sink_k", "sink_v"), ("cache_k", "cache_v"), ("stored_tokens", "start_indices")):
+        ta, tb = tensors[a], tensors[b]
+        assert ta.shape == tb.shape, (a, b)
+        for size, sa, sb in zip(ta.shape, ta.stride(), tb.stride()):
+            assert size <= 1 or sa == sb, f"{a} and {b} must share strides"
+    floating = ("k", "v", "s", "sink_k", "sink_v", "cache_k", "cache_v", "cache_s")
+    assert all(tensors[n].dtype == k.dtype for n in floating)
+    assert sink_mask.dtype == torch.bool and mask.dtype == torch.bool
+    integer = ("sink_pos", "pos", "og_pos", "do_cache_every_n", "stored_tokens", "start_indices", "stored_sinks")
+    assert all(tensors[n].dtype == torch.int64 for n in integer)
+    d = OracleUpdateDesc()
+    for name, t in tensors.items():
+        assert t.device.type == "cpu", "the oracle runs on host memory"
+        rec = getattr(d, name)
+        rec.ptr = t.data_ptr()
+        for i, st in enumerate(t.stride()):
+            rec.stride[i] = st
+    d.num_sink, d.window_size, d.max_seq_len = int(num_sink), int(window_size), int(max_seq_len)
+    d.real_token_idx = int(real_token_idx)
+    d.eager_fill = 1 if eager_fill else 0
+    d.n, d.h, d.k_len, d.hid = k.shape
+    d.cascades = stored_tokens.shape[-1]
+    d.dtype = ORACLE_DTYPE[k.dtype]
+    return d
 
 
 def _lib():
@@ -27,8 +81,11 @@ def _lib():
         if not os.path.exists(path):
             path = _build.build()
         L = C.CDLL(path)
-        L.ckv_oracle_update.argtypes = [C.POINTER(UpdateArgs)]
+        L.ckv_oracle_update.argtypes = [C.POINTER(OracleUpdateDesc)]
         L.ckv_oracle_update.restype = C.c_int
+        L.ckv_oracle_sizeof_desc.argtypes = []
+        L.ckv_oracle_sizeof_desc.restype = C.c_int64
+        assert L.ckv_oracle_sizeof_desc() == C.sizeof(OracleUpdateDesc)
         _LIB = L
     return _LIB
 
@@ -36,12 +93,10 @@ def _lib():
 def oracle_sink_cache(k, v, s, sink_k, sink_v, sink_mask, sink_pos, cache_k, cache_v, cache_s, mask, pos,
                       og_pos, do_cache, do_cache_every_n, stored_tokens, start_indices, stored_sinks,
                       num_sink, window_size, real_token_idx, max_seq_len, eager_fill):
-    for t in (k, cache_k, stored_tokens):
-        assert t.device.type == "cpu", "the oracle runs on host memory"
-    a = fill_update_args(k, v, s, sink_k, sink_v, sink_mask, sink_pos, cache_k, cache_v, cache_s, mask, pos,
-                         og_pos, do_cache_every_n, stored_tokens, start_indices, stored_sinks, num_sink,
-                         window_size, real_token_idx, max_seq_len, eager_fill)
-    rc = _lib().ckv_oracle_update(C.byref(a))
+    d = describe_update(k, v, s, sink_k, sink_v, sink_mask, sink_pos, cache_k, cache_v, cache_s, mask, pos,
+                        og_pos, do_cache_every_n, stored_tokens, start_indices, stored_sinks, num_sink,
+                        window_size, real_token_idx, max_seq_len, eager_fill)
+    rc = _lib().ckv_oracle_update(C.byref(d))
     if rc != 0:
         raise RuntimeError(f"ckv_oracle_update returned {rc}")
     return k, v

@@ -204,3 +204,99 @@ def test_chunk_is_checked_against_the_cache_before_any_pointer_leaves():
     k = torch.zeros(2, 2, 3, 8, dtype=torch.float16)
     with pytest.raises(ValueError):
         c._update_args(k, k.clone(), torch.zeros(2, 1, 3, dtype=torch.float16), 0)
+
+
+# ---------------------------------------------------------------------------------------------
+# The oracle describes its arguments with code of its own (oracle/update.py:describe_update), the
+# library with _abi.fill_update_args.  Both are fed deliberately odd layouts and must agree field
+# by field; the oracle must also give the same result on those layouts as on contiguous copies.
+# ---------------------------------------------------------------------------------------------
+def _odd_layout_state(seed=0, N=2, KVH=3, H=6, K=5, D=4, NS=3, W=4, Cc=2, dtype=torch.float32):
+    """Every tensor of one sink_cache call as a non-contiguous view: scores with H > KVH heads in a
+    transposed layout (the caller of cascade_attention.py:331-339 repeats and hands over (B, H, q)),
+    caches and trackers cut out of larger buffers, incoming rows with a padded last dimension."""
+    g = torch.Generator().manual_seed(seed)
+    S = W * Cc
+
+    def cut(*shape, dt=dtype, pad=2):
+        big = torch.zeros(*(s + pad for s in shape), dtype=dt)
+        return big[tuple(slice(1, 1 + s) for s in shape)]
+
+    t = {}
+    t["k"] = torch.randn(N, K, KVH, D + 3, generator=g).to(dtype).permute(0, 2, 1, 3)[..., 1:1 + D]
+    t["v"] = torch.randn(N, K, KVH, D + 3, generator=g).to(dtype).permute(0, 2, 1, 3)[..., 1:1 + D]
+    t["s"] = torch.rand(K, N, H, generator=g).to(dtype).permute(1, 2, 0)       # (N, H, K), K outermost in memory
+    t["sink_k"], t["sink_v"] = cut(N, KVH, NS, D), cut(N, KVH, NS, D)
+    t["cache_k"], t["cache_v"] = cut(N, KVH, S, D), cut(N, KVH, S, D)
+    t["cache_s"] = cut(N, KVH, S)
+    t["sink_mask"], t["mask"] = cut(N, KVH, NS, dt=torch.bool), cut(N, KVH, S, dt=torch.bool)
+    t["sink_mask"].fill_(True)
+    t["mask"].fill_(True)
+    t["sink_pos"], t["pos"], t["og_pos"] = (cut(N, KVH, NS, dt=torch.long), cut(N, KVH, S, dt=torch.long),
+                                            cut(N, KVH, S, dt=torch.long))
+    t["stored_tokens"], t["start_indices"] = cut(N, KVH, Cc, dt=torch.long), cut(N, KVH, Cc, dt=torch.long)
+    t["stored_sinks"] = cut(N, KVH, dt=torch.long)
+    t["do_cache_every_n"] = torch.tensor([1, 2][:Cc], dtype=torch.long)
+    return t, dict(num_sink=NS, window_size=W, max_seq_len=S)
+
+
+_ORDER = ("k", "v", "s", "sink_k", "sink_v", "sink_mask", "sink_pos", "cache_k", "cache_v", "cache_s", "mask", "pos",
+          "og_pos", "do_cache_every_n", "stored_tokens", "start_indices", "stored_sinks")
+
+
+def test_oracle_and_library_describe_odd_layouts_alike():
+    from oracle.update import describe_update
+
+    t, sc = _odd_layout_state()
+    seen = torch.tensor(0, dtype=torch.long)
+    args = [t[n] for n in _ORDER]
+    lib_a = _abi.fill_update_args(*args, sc["num_sink"], sc["window_size"], seen, sc["max_seq_len"], True)
+    ora = describe_update(*args, sc["num_sink"], sc["window_size"], seen, sc["max_seq_len"], True)
+    # which field of the library's struct carries the pointer / the strides of which tensor
+    pairs = {"k": ("k", "kv_stride"), "v": ("v", "kv_stride"), "s": ("s", "s_stride"),
+             "sink_k": ("sink_k", "sink_stride"), "sink_v": ("sink_v", "sink_stride"),
+             "cache_k": ("cache_k", "cache_stride"), "cache_v": ("cache_v", "cache_stride"),
+             "cache_s": ("cache_s", "cache_s_stride"), "sink_mask": ("sink_mask", "sink_mask_stride"),
+             "mask": ("mask", "mask_stride"), "sink_pos": ("sink_pos", "sink_pos_stride"), "pos": ("pos", "pos_stride"),
+             "og_pos": ("og_pos", "og_pos_stride"), "stored_sinks": ("stored_sinks", "stored_sinks_stride"),
+             "stored_tokens": ("stored_tokens", "tracker_stride"), "start_indices": ("start_indices", "tracker_stride"),
+             "do_cache_every_n": ("do_cache_every_n", None)}
+    for name, (ptr_field, stride_field) in pairs.items():
+        rec = getattr(ora, name)
+        assert getattr(lib_a, ptr_field) == rec.ptr == t[name].data_ptr(), name
+        if stride_field is None:
+            continue
+        got = list(getattr(lib_a, stride_field))
+        for dim, size in enumerate(t[name].shape):
+            if size > 1:  # the stride of a size-1 dimension is arbitrary
+                assert got[dim] == rec.stride[dim] == t[name].stride(dim), (name, dim)
+    assert (lib_a.N, lib_a.H, lib_a.K, lib_a.HID) == (ora.n, ora.h, ora.k_len, ora.hid) == tuple(t["k"].shape)
+    assert (lib_a.num_sink, lib_a.window_size, lib_a.max_seq_len, lib_a.cascades) == (
+        ora.num_sink, ora.window_size, ora.max_seq_len, ora.cascades)
+    assert lib_a.eager_fill == ora.eager_fill == 1
+    assert lib_a.dtype == _abi.CKV_F32 and ora.dtype == 0
+    # the scores really are laid out with the token index outermost, and with more heads than the cache has
+    assert t["s"].stride() == (6, 1, 12) and t["s"].size(1) > t["k"].size(1)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_oracle_result_does_not_depend_on_the_layout(dtype):
+    """Three calls on the odd layouts against the same calls on contiguous copies."""
+    from oracle.update import oracle_sink_cache
+
+    t, sc = _odd_layout_state(seed=3, dtype=dtype)
+    flat = {n: x.clone().contiguous() for n, x in t.items()}
+    seen = 0
+    g = torch.Generator().manual_seed(9)
+    for call in range(3):
+        for n in ("k", "v", "s"):
+            fresh = torch.rand(t[n].shape, generator=g).to(dtype)
+            t[n].copy_(fresh)
+            flat[n].copy_(fresh)
+        for side in (t, flat):
+            oracle_sink_cache(*[side[n] for n in _ORDER[:13]], None, *[side[n] for n in _ORDER[13:]],
+                              sc["num_sink"], sc["window_size"], torch.tensor(seen), sc["max_seq_len"], True)
+        seen += t["k"].size(2)
+        for n in _ORDER[3:]:
+            assert torch.equal(t[n], flat[n]), (call, n)
+    assert not t["mask"].all() and t["stored_sinks"].eq(sc["num_sink"]).all()
