@@ -8,6 +8,7 @@ the reference mixin so model code written against it keeps working.
 """
 import ctypes as C
 import math
+import os
 from typing import Optional
 
 import torch
@@ -15,6 +16,9 @@ from torch import nn
 
 from . import _abi
 from .cascading_cache import CascadingKVCache, _require_device, workspace
+
+
+_DEBUG_COUNTERS = os.environ.get("CKV_DEBUG_COUNTERS", "0") not in ("", "0")
 
 
 def default_inv_freq(head_dim: int, theta: float, device) -> torch.Tensor:
@@ -38,9 +42,10 @@ def chunk_positions(cache: CascadingKVCache, layer_idx: int, q_len: int, do_og_p
     # out ids below the number of stored tokens, cascading_cache.py:112-142), and the chunk starts one past them
     # whatever the stream does later.  The ids are then a function of the host-side token counter: no kernel, no
     # device read.  (This holds for every state the update itself produces from an empty cache.)
-    # (A caller that records the launches for replay gets the host value only once it no longer changes.)
+    # A caller that records the launches for replay always gets the ids from the device: a recorded launch keeps
+    # the raw pointer of this tensor, which must neither depend on the host counter nor be freed under it.
     S, NS = cache.max_seq_len[layer_idx], cache.num_sink_tokens
-    if not do_og_pos and cache.eager_fill and S > 0 and (not _replayable or cache._seen_host[layer_idx] >= S + NS):
+    if not do_og_pos and cache.eager_fill and S > 0 and not _replayable:
         start = min(int(cache._seen_host[layer_idx]), S + NS)
         memo = cache.__dict__.setdefault("_steady_q_pos", {})
         key = (start, q_len, dev)
@@ -161,6 +166,8 @@ def cascade_attention(query_states, key_states, value_states, cache: CascadingKV
     """
     _require_device(query_states, "query_states")
     lib = _abi.lib()
+    if _DEBUG_COUNTERS:
+        cache.check_host_counter(layer_idx)
     B, H, Q, D = query_states.shape
     KVH = key_states.size(1)
     assert key_states.shape == (B, KVH, Q, D) and value_states.shape == (B, KVH, Q, D)
@@ -221,8 +228,10 @@ class DecodeStepGraph:
     returned ``out`` / ``new_scores`` tensors are the graph's fixed outputs and are overwritten by the next step.
 
     Recorded values that must not change between steps: the sink shift (the cache must already hold more than
-    ``num_sink_tokens`` tokens), shapes, dtype, head reduction, and the state tensors of the cache (``reset()``
-    or assigning a new tensor to ``score_cache[l]`` invalidates the graph: build a new one)."""
+    ``num_sink_tokens`` tokens), shapes, dtype, head reduction, and the addresses of the cache's state tensors
+    (assigning a new tensor to ``score_cache[l]`` raises at the next step: build a new graph).  The position ids of
+    the token come from a kernel inside the graph, never from the host counter.  ``reset()`` / ``init_cache()`` of
+    the cache are noticed (the cache counts them): the next step runs eagerly and the one after records afresh."""
 
     def __init__(self, cache: CascadingKVCache, layer_idx: int, inv_freq: torch.Tensor, num_heads: int,
                  head_reduction: Optional[str] = None, homogeneous_heads: bool = False, do_og_pos: bool = False,
@@ -239,6 +248,7 @@ class DecodeStepGraph:
         self.out = self.new_scores = None
         self._warm = False
         self._state = None
+        self._generation = None
 
     def _run(self):
         return cascade_attention(self.q, self.k, self.v, self.cache, self.layer_idx, self.inv_freq, replayable=True,
@@ -254,6 +264,9 @@ class DecodeStepGraph:
             self.q.copy_(q)
             self.k.copy_(k)
             self.v.copy_(v)
+        if self._generation != cache._generation:  # first use, or the cache was reset / reallocated since
+            self._generation = cache._generation
+            self.graph, self._warm = None, False
         if not self._warm:  # eager: kernel attributes, scratch sizes, argument blocks
             self._warm = True
             return self._run()
@@ -275,6 +288,13 @@ class DecodeStepGraph:
         if L == 0:
             cache._seen_tokens += 1
         return self.out, self.new_scores
+
+
+def _rotate(x, cos, sin):
+    """``x * cos + rotate_half(x) * sin`` in ``x.dtype``, cos / sin ``(B or 1, n, D)`` broadcast over heads."""
+    half = x.size(-1) // 2
+    turned = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+    return x * cos[:, None] + turned * sin[:, None]
 
 
 class CascadeAttention(nn.Module):
@@ -317,6 +337,57 @@ class CascadeAttention(nn.Module):
         out = self.o_proj(out)
         return out, None, past_key_value
 
+    # -- the reference mixin's remaining surface -------------------------------------------------------------
+    # ``forward_cascade`` above never calls these (the fused operator rotates, concatenates and reduces inside
+    # the kernels); they exist so that model code written against the reference mixin, which calls
+    # ``self.rope(...)`` and ``self.cascade_attn_flash(...)`` / ``self.cascade_attn_eager(...)`` itself, keeps
+    # working.  Both attention arms run the library's dense operator, whose scores are exact.
+
+    def rope(self, x, pos, cos=None, sin=None):
+        """Rotary embedding of ``x (B, heads, n, D)`` at positions ``pos (B or 1, n)``; returns
+        ``(rotated, cos, sin)`` so the caller can reuse the tables (cascade_attention.py:343-353).  Angles are
+        fp32 ``pos * inv_freq``; cos / sin are cast to ``x.dtype`` before they are applied
+        (modeling_llama.py:205-220, 248-252)."""
+        if cos is None or sin is None:
+            if not hasattr(self, "_inv_freq") or self._inv_freq.device != x.device:
+                self._inv_freq = default_inv_freq(self.head_dim, self.rope_theta, x.device)
+            angles = pos.to(torch.float32)[..., None] * self._inv_freq       # (B, n, D/2)
+            angles = torch.cat((angles, angles), dim=-1)
+            cos, sin = angles.cos().to(x.dtype), angles.sin().to(x.dtype)
+        return _rotate(x, cos, sin), cos, sin
+
+    def cascade_attn_flash(self, query_states, key_states, value_states, key_states_pos, v_states, sink_key_states,
+                           sink_value_states, k_states, sink_mask, key_mask, first_it, past_key_value, scale, q_len,
+                           homogeneous_heads):
+        """cascade_attention.py:202-229 on the library's dense operator: the caller has rotated and head-expanded
+        everything except ``key_states`` / ``value_states`` (the chunk as it goes into the cache).  The sums of the
+        cached keys are taken aligned with their slots, as the eager arm does (cascade_attention.py:319); the
+        reference's flash arm hands ``calc_scores`` the first ``n_keys`` columns, sink columns included."""
+        from .flash_attention import attention
+
+        self.last_attn_called, self.last_q_size = "flash", query_states.size(2)
+        groups = query_states.size(1) // value_states.size(1)
+        chunk_values = value_states[:, :, None].expand(-1, -1, groups, -1, -1).reshape(
+            value_states.size(0), -1, value_states.size(2), value_states.size(3))       # repeat_kv
+        keys = torch.cat((sink_key_states, k_states, key_states_pos), dim=2)
+        values = torch.cat((sink_value_states, v_states, chunk_values), dim=2)
+        hidden = torch.cat((sink_mask[0, 0], key_mask[0, 0]))
+        out, scores = attention(query_states, keys, values, True, scale, hidden, past_key_value.beta)
+        # the dense operator's scores cover [sink | cache | chunk]; the cached part is what the EMA is for
+        n_sink = sink_key_states.size(2)
+        ema, new_scores = self.calc_scores(scores[:, :, n_sink:], homogeneous_heads, k_states.size(2), q_len)
+        L = self.layer_idx
+        past_key_value.score_cache[L] = (past_key_value.beta ** q_len) * past_key_value.score_cache[L] + ema
+        past_key_value.update(key_states, value_states, L, score_states=new_scores)
+        return out, past_key_value
+
+    def cascade_attn_eager(self, *args):
+        """cascade_attention.py:250-340.  There is no eager arm on the device: the dense operator already returns
+        the exact sums the eager path computes, so this is ``cascade_attn_flash`` under the other name."""
+        out, cache = self.cascade_attn_flash(*args)
+        self.last_attn_called = "eager"
+        return out, cache
+
     def calc_scores(self, scores, homogeneous_heads, n_keys, q_len):
         """Head reduction of per-head score sums ``(B, H, n)`` with the semantics of
         cascade_attention.py:231-248, for callers that hold per-head scores of their own (``attention``
@@ -341,3 +412,25 @@ class CascadeAttention(nn.Module):
         if homogeneous_heads:
             new_scores = new_scores.repeat(1, kvh, 1)
         return reduced[:, :, :n_keys], new_scores
+
+
+class LlamaCascadeAttention(CascadeAttention):
+    """cascade_attention.py:343-353: cos / sin computed from the position ids (the mixin's default ``rope``)."""
+
+
+class Qwen2CascadeAttention(CascadeAttention):
+    """cascade_attention.py:356-367: cos / sin looked up in a table of ``max_position_embeddings`` rows (the ids
+    of a cascade cache can exceed the length a Qwen2 rotary module was asked for, hence the fixed table)."""
+
+    def rope(self, x, pos, cos=None, sin=None):
+        if cos is None or sin is None:
+            if not hasattr(self, "_inv_freq") or self._inv_freq.device != x.device:
+                self._inv_freq = default_inv_freq(self.head_dim, self.rope_theta, x.device)
+            rows = torch.arange(self.max_position_embeddings, device=x.device, dtype=torch.float32)
+            angles = torch.outer(rows, self._inv_freq)
+            angles = torch.cat((angles, angles), dim=-1)
+            cos, sin = angles.cos().to(x.dtype), angles.sin().to(x.dtype)
+        ids = pos.reshape(-1)
+        picked_cos = cos[ids].reshape(1, pos.size(1), cos.size(-1))
+        picked_sin = sin[ids].reshape(1, pos.size(1), sin.size(-1))
+        return _rotate(x, picked_cos, picked_sin), cos, sin

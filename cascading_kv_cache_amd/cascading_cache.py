@@ -112,38 +112,36 @@ class CascadingKVCache:
         eager_fill: bool = True,
         verbose: bool = True,
     ) -> None:
-        if isinstance(max_seq_len, int) != isinstance(window_length, int):
-            raise ValueError(
-                f"max_seq_len must be same type as window length: {type(max_seq_len)=} {type(window_length)=}")
-        if isinstance(max_seq_len, int):
-            max_seq_len = [max_seq_len for _ in range(layers)]
-        if isinstance(window_length, int):
-            window_length = [window_length for _ in range(layers)]
+        # one size for every layer, or one per layer: both arguments in the same form (cascading_cache.py:1050-1057)
+        per_layer = [isinstance(x, (list, tuple)) for x in (window_length, max_seq_len)]
+        if per_layer[0] != per_layer[1]:
+            raise ValueError("window_length and max_seq_len must both be integers or both be per-layer lists, got "
+                             f"{type(window_length).__name__} and {type(max_seq_len).__name__}")
+        if per_layer[0]:
+            windows, lengths = [int(w) for w in window_length], [int(s) for s in max_seq_len]
+            if len(windows) != layers or len(lengths) != layers:
+                raise ValueError(f"per-layer sizes need {layers} entries, got {len(windows)} and {len(lengths)}")
+        else:
+            windows, lengths = [int(window_length)] * layers, [int(max_seq_len)] * layers
+        bad = [l for l in range(layers) if windows[l] <= 0 or lengths[l] % windows[l] != 0]
+        if bad:
+            raise ValueError(f"max_seq_len must be a whole number of windows in every layer; layers {bad} have "
+                             f"windows {[windows[l] for l in bad]} and lengths {[lengths[l] for l in bad]}")
 
-        self.verbose = verbose
-        self.max_seq_len = max_seq_len
-        self.max_batch_size = max_batch_size
-        self.heads = heads
-        self.dim = dim
-        self.device = device
-        self.dtype = dtype
-        self.window_length = window_length
+        self.window_length, self.max_seq_len = windows, lengths
+        self.cascades = [s // w for s, w in zip(lengths, windows)]
         self.num_sink_tokens = num_sink_tokens
-        self.cascade_func = cascade_func
-        self.head_reduction = head_reduction
-        self.layers = layers
-        self.eager_fill = eager_fill
-        self.bh = self.max_batch_size * self.heads
-
-        if not all((self.max_seq_len[l] % self.window_length[l]) == 0 for l in range(layers)):
-            raise ValueError(
-                f"window length must evenly divide max seq len: {self.window_length=} {self.max_seq_len=}")
-        self.cascades = [self.max_seq_len[l] // self.window_length[l] for l in range(layers)]
+        self.max_batch_size, self.heads, self.dim, self.layers = max_batch_size, heads, dim, layers
+        self.bh = max_batch_size * heads
+        self.device, self.dtype = device, dtype
+        self.cascade_func, self.head_reduction, self.eager_fill = cascade_func, head_reduction, eager_fill
+        self.verbose = verbose
         self._seen_tokens = 0
         self.init_cache(self.device)
 
     def __repr__(self):
-        return f"{self.max_seq_len=}, {self.cascades=} {self.max_batch_size=}, {self.layers=} {self.heads=}"
+        return (f"CascadingKVCache(layers={self.layers}, batch={self.max_batch_size}, heads={self.heads}, "
+                f"dim={self.dim}, sinks={self.num_sink_tokens}, cascades={self.cascades}, slots={self.max_seq_len})")
 
     def __getitem__(self, layer_idx: int):
         return self.get_vals(layer_idx)
@@ -198,6 +196,7 @@ class CascadingKVCache:
         if verbose:
             print(f"RESET HIP CACHE {self.cascade_func=}")
         self._seen_tokens = 0
+        self._generation += 1   # a step recorded into a graph before the reset no longer describes this cache
         self._seen_host = [0 for _ in range(self.layers)]
         self.seen_tokens_by_layer.zero_()
         for group in (self.stored_tokens, self.stored_sinks, self.start_indices, self.pos, self.sink_pos,
@@ -210,34 +209,65 @@ class CascadingKVCache:
                 t.fill_(True)
 
     def init_cache(self, device):
-        L, B, H, D = self.layers, self.max_batch_size, self.heads, self.dim
-        nsink, dev, dtp = self.num_sink_tokens, device, self.dtype
+        """Allocates the state of every layer with the shapes and dtypes of cascading_cache.py:1196-1276."""
         if self.verbose:
             print(f"INIT CLEAN HIP CACHE {self.cascade_func=}")
+        n_layers, sinks = self.layers, self.num_sink_tokens
+        per_head = (self.max_batch_size, self.heads)
         self._seen_tokens = 0
+        self._generation = getattr(self, "_generation", 0) + 1   # recorded graphs and memoised blocks are void
         self._update_memo, self._attn_memo = {}, {}  # argument blocks described once per input layout
         # host mirror of seen_tokens_by_layer: lets callers branch without a device sync
-        self._seen_host = [0 for _ in range(L)]
-        self.seen_tokens_by_layer = torch.zeros(L, dtype=torch.long, device=dev)
-        self.do_cache = [torch.ones(self.cascades[l], device=dev, dtype=torch.bool) for l in range(L)]
-        self.do_cache_every_n = [
-            torch.tensor(acceptance_periods(self.cascade_func, self.cascades[l]), device=dev, dtype=torch.long)
-            for l in range(L)]
+        self._seen_host = [0] * n_layers
         self.beta = 0.9999999  # cascading_cache.py:1247
 
-        self.stored_tokens = [torch.zeros(B, H, self.cascades[l], device=dev, dtype=torch.long) for l in range(L)]
-        self.stored_sinks = [torch.zeros(B, H, device=dev, dtype=torch.long) for _ in range(L)]
-        self.start_indices = [torch.zeros(B, H, self.cascades[l], device=dev, dtype=torch.long) for l in range(L)]
-        self.pos = [torch.zeros(B, H, self.max_seq_len[l], device=dev, dtype=torch.long) for l in range(L)]
-        self.og_pos = [torch.zeros(B, H, self.max_seq_len[l], device=dev, dtype=torch.long) for l in range(L)]
-        self.sink_pos = [torch.zeros(B, H, nsink, device=dev, dtype=torch.long) for _ in range(L)]
-        self.key_cache = [torch.zeros(B, H, self.max_seq_len[l], D, device=dev, dtype=dtp) for l in range(L)]
-        self.value_cache = [torch.zeros(B, H, self.max_seq_len[l], D, device=dev, dtype=dtp) for l in range(L)]
-        self.score_cache = [torch.zeros(B, H, self.max_seq_len[l], device=dev, dtype=dtp) for l in range(L)]
-        self.sink_keys = [torch.zeros(B, H, nsink, D, device=dev, dtype=dtp) for _ in range(L)]
-        self.sink_values = [torch.zeros(B, H, nsink, D, device=dev, dtype=dtp) for _ in range(L)]
-        self.mask = [torch.ones(B, H, self.max_seq_len[l], device=dev, dtype=torch.bool) for l in range(L)]
-        self.sink_mask = [torch.ones(B, H, nsink, device=dev, dtype=torch.bool) for _ in range(L)]
+        def per_layer(fill, dtype, *tail):
+            """One tensor per layer, (batch, heads, *tail(layer)), every element ``fill``."""
+            return [torch.full(per_head + tuple(t(l) if callable(t) else t for t in tail), fill, device=device,
+                               dtype=dtype) for l in range(n_layers)]
+
+        slots = lambda l: self.max_seq_len[l]    # noqa: E731
+        levels = lambda l: self.cascades[l]      # noqa: E731
+        self.seen_tokens_by_layer = torch.zeros(n_layers, dtype=torch.long, device=device)
+        self.do_cache = [torch.ones(self.cascades[l], device=device, dtype=torch.bool) for l in range(n_layers)]
+        self.do_cache_every_n = [
+            torch.tensor(acceptance_periods(self.cascade_func, self.cascades[l]), device=device, dtype=torch.long)
+            for l in range(n_layers)]
+        # trackers and position ids (int64), keys / values / scores (cache dtype), masks (True = empty)
+        self.stored_tokens = per_layer(0, torch.long, levels)
+        self.start_indices = per_layer(0, torch.long, levels)
+        self.stored_sinks = per_layer(0, torch.long)
+        self.pos = per_layer(0, torch.long, slots)
+        self.og_pos = per_layer(0, torch.long, slots)
+        self.sink_pos = per_layer(0, torch.long, sinks)
+        self.key_cache = per_layer(0, self.dtype, slots, self.dim)
+        self.value_cache = per_layer(0, self.dtype, slots, self.dim)
+        self.score_cache = per_layer(0, self.dtype, slots)
+        self.sink_keys = per_layer(0, self.dtype, sinks, self.dim)
+        self.sink_values = per_layer(0, self.dtype, sinks, self.dim)
+        self.mask = per_layer(True, torch.bool, slots)
+        self.sink_mask = per_layer(True, torch.bool, sinks)
+
+    def sync_host_counter(self) -> List[int]:
+        """Re-reads the host mirror of ``seen_tokens_by_layer`` from the device (one read-back).
+
+        The fused operator never reads the device counter: the sink shift, the chunk's position ids on an
+        eagerly filled cache and the bound on filled slots all come from the host mirror, which ``update`` /
+        ``update_state`` / ``reset`` keep in step.  Code that changes the state some other way (copies saved state
+        tensors into the cache, calls the module-level ``sink_cache`` and bumps ``seen_tokens_by_layer`` itself, as
+        the reference allows) must call this afterwards.  Setting the environment variable ``CKV_DEBUG_COUNTERS=1``
+        makes every fused call check the mirror against the device (a device read-back per call)."""
+        self._seen_host = [int(x) for x in self.seen_tokens_by_layer.tolist()]
+        self._seen_tokens = self._seen_host[0] if self._seen_host else 0
+        return list(self._seen_host)
+
+    def check_host_counter(self, layer_idx: int):
+        """Raises if the host mirror of a layer's token counter disagrees with the device (a read-back)."""
+        dev = int(self.seen_tokens_by_layer[layer_idx])
+        if dev != self._seen_host[layer_idx]:
+            raise _abi.CkvError(
+                f"layer {layer_idx}: the device counter says {dev} tokens, the host mirror {self._seen_host[layer_idx]}; "
+                "state was changed outside update()/reset(): call sync_host_counter()")
 
     def pos_shift(self, layer_idx: int) -> int:
         """The sink shift of get_vals (cascading_cache.py:1282-1283), from the host counter."""

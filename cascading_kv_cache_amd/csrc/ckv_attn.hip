@@ -41,7 +41,7 @@ AttnWorkspace carve_attn(void* base, int64_t B, int64_t H, int64_t KVH, int64_t 
     w.w_ema = (float*)c.take((Q + kColSlack) * 4);
     w.w_new = (float*)c.take(Q * 4);
     // shares of the forward kernel when few query rows would leave the chip idle
-    const int splits = mfma_supported(dtype, D, H, KVH, Q) && Q > 1 ? mfma_fwd_splits(B, H, KVH, Q, N) : 1;
+    const int splits = mfma_supported(dtype, D, H, KVH, Q) && Q > 1 ? mfma_fwd_splits_for_workspace(B, H, KVH, Q, N) : 1;
     w.part_o = splits > 1 ? (float*)c.take(splits * B * H * Q * D * 4) : nullptr;
     w.part_l2 = splits > 1 ? (float*)c.take(splits * B * H * Q * 4) : nullptr;
     w.bytes = c.off;

@@ -107,7 +107,10 @@ struct MfmaProblem {
 
 bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH, int64_t Q);
 int64_t mfma_n_pad(int64_t n);
-int mfma_fwd_splits(int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t n);  // shares of the key tiles per query tile
+// shares of the key tiles per query tile on a chip of `cus` compute units; what a workspace must hold
+int mfma_fwd_splits(int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t n, int cus);
+int mfma_fwd_splits_for_workspace(int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t n);
+int mfma_device_cus();  // compute units of the current device (256 where none can be asked)
 bool mfma_fits(int64_t n);  // the per-tile bookkeeping of n keys fits in LDS
 int launch_mfma(const MfmaProblem& p, hipStream_t stream);
 

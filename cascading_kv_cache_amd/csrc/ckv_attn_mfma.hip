@@ -1267,6 +1267,7 @@ template <typename T>
 int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
     const int64_t n = mp.n, n_pad = mp.n_pad;
     const float scale_log2 = mp.scale * 1.4426950408889634f;
+    const int cus = mfma_device_cus();
     {
         StageScope sc(CKV_STAGE_PREP, stream);
         StageParams sp;
@@ -1294,7 +1295,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         int64_t splits = nbh;
         if (mp.shared_pos) {  // about two workgroups per compute unit
             const int64_t tiles = n_pad / kBN;
-            splits = (512 + tiles - 1) / tiles;
+            splits = (2 * cus + tiles - 1) / tiles;
             if (splits < 2) splits = 2;
             if (splits > nbh) splits = nbh;
         }
@@ -1312,10 +1313,10 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         sq.vec = mp.q_stride[3] == 1 && reinterpret_cast<uintptr_t>(mp.q) % 16 == 0 && mp.q_stride[0] % 8 == 0 &&
                  mp.q_stride[1] % 8 == 0 && mp.q_stride[2] % 8 == 0;
         {
-            // about 1024 query blocks (64 positions each); the rest of batch x heads is looped over inside,
-            // sharing cos/sin
+            // about four query blocks (64 positions each) per compute unit; the rest of batch x heads is looped
+            // over inside, sharing cos/sin
             const int64_t bx = (mp.Q + 63) / 64, nbh_q = mp.B * mp.H;
-            int64_t by = (1024 + bx - 1) / bx;
+            int64_t by = (4 * cus + bx - 1) / bx;
             if (by > nbh_q) by = nbh_q;
             if (by < 1) by = 1;
             StageGrid g;
@@ -1339,7 +1340,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         fp.G = G;
         fp.scale_log2 = 1.f;  // already on the staged queries
         fp.n_qt = (int)((mp.Q * G + kRows - 1) / kRows);
-        fp.n_split = mfma_fwd_splits(mp.B, mp.H, mp.KVH, mp.Q, n);
+        fp.n_split = mfma_fwd_splits(mp.B, mp.H, mp.KVH, mp.Q, n, cus);
         fp.part_o = mp.part_o;
         fp.part_l2 = mp.part_l2;
         if (fp.n_split > 1 && (!fp.part_o || !fp.part_l2)) return CKV_ERR_WORKSPACE;
@@ -1412,17 +1413,33 @@ bool mfma_supported(int dtype, int64_t D, int64_t H, int64_t KVH, int64_t Q) {
 
 int64_t mfma_n_pad(int64_t n) { return align_up(n, 256); }
 
-// Shares of a query tile's key tiles (1: no splitting).  A function of the shapes alone, so that the workspace
-// can be sized for it: the chip is taken to hold 256 workgroups of the forward kernel at once; fewer than that
-// are topped up to about 512, with at least 16 key tiles per share and at most 8 shares.
-int mfma_fwd_splits(int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t n) {
+// Shares of a query tile's key tiles (1: no splitting) on a chip of `cus` compute units, each of which holds one
+// workgroup of the forward kernel at a time: launches with fewer workgroups than that are topped up to about two per
+// compute unit, with at least 16 key tiles per share and at most 8 shares.
+int mfma_fwd_splits(int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t n, int cus) {
     const int64_t G = H / KVH;
     const int64_t wgs = ((Q * G + kRows - 1) / kRows) * B * KVH, tiles = (n + kBN - 1) / kBN;
-    if (wgs >= 256) return 1;
-    int64_t s_ = 512 / wgs;
+    if (wgs >= cus) return 1;
+    int64_t s_ = 2 * (int64_t)cus / wgs;
     if (s_ > tiles / 16) s_ = tiles / 16;
     if (s_ > 8) s_ = 8;
     return s_ < 1 ? 1 : (int)s_;
+}
+
+// compute units of the current device; 256 (one MI355X) where no device can be asked, e.g. when a workspace is
+// sized on a host without one
+int mfma_device_cus() {
+    DeviceInfo di;
+    if (current_device_info(&di) != CKV_OK || di.cus <= 0) return 256;
+    return di.cus;
+}
+
+// what a workspace is sized for: the shares the current device would use, and never fewer than a 256-unit chip's,
+// so that a size computed where no device is visible also serves the launch
+int mfma_fwd_splits_for_workspace(int64_t B, int64_t H, int64_t KVH, int64_t Q, int64_t n) {
+    const int here = mfma_fwd_splits(B, H, KVH, Q, n, mfma_device_cus());
+    const int base = mfma_fwd_splits(B, H, KVH, Q, n, 256);
+    return here > base ? here : base;
 }
 
 // the forward kernel keeps per-tile bookkeeping of all N keys in LDS

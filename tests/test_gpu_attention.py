@@ -420,3 +420,70 @@ def test_dense_operator_backward(Z, H, N_CTX, N_KV, HEAD_DIM, dtype):
     if int(mask.sum()) > 0:
         assert k.grad[:, :, : N_KV - N_CTX][:, :, mask].abs().max().item() == 0.0
         assert v.grad[:, :, : N_KV - N_CTX][:, :, mask].abs().max().item() == 0.0
+
+
+@pytest.mark.parametrize("flavour", ["llama", "qwen2"])
+def test_reference_mixin_surface(flavour):
+    """A layer written the way the reference's model files use the mixin — ``get_vals``, ``self.rope`` on queries,
+    chunk keys, sinks and cached keys, ``repeat_kv``, then ``self.cascade_attn_flash`` / ``cascade_attn_eager``
+    (cascade_attention.py:103-200) — against the fused operator on a second cache: outputs within tolerance,
+    score cache within tolerance, cache metadata bit-exact, over chunks that fill the cache and evict."""
+    from types import SimpleNamespace
+
+    from cascading_kv_cache_amd.cascade_attention import (LlamaCascadeAttention, Qwen2CascadeAttention,
+                                                          cascade_attention, default_inv_freq)
+    from cascading_kv_cache_amd.cascading_cache import CascadingKVCache
+
+    B, H, KVH, D, NS, W, C, dtype = 2, 8, 2, 128, 4, 32, 2, torch.bfloat16
+    base = Qwen2CascadeAttention if flavour == "qwen2" else LlamaCascadeAttention
+
+    class Layer(base):
+        def __init__(self):
+            super().__init__()
+            self.num_heads, self.num_key_value_heads, self.head_dim, self.layer_idx = H, KVH, D, 0
+            self.num_key_value_groups = H // KVH
+            self.rope_theta, self.max_position_embeddings = 5e5, 512
+            self.config = SimpleNamespace(_head_reduction="mean", _homogeneous_heads=False, _do_og_pos=False)
+
+    def expand(x):  # repeat_kv
+        return x[:, :, None].expand(-1, -1, H // KVH, -1, -1).reshape(x.size(0), H, x.size(2), x.size(3))
+
+    layer = Layer()
+    caches = [CascadingKVCache(window_length=W, num_sink_tokens=NS, max_batch_size=B, heads=KVH, dim=D,
+                               max_seq_len=W * C, device="cuda:0", dtype=dtype, layers=1, verbose=False)
+              for _ in range(2)]
+    by_hand, fused = caches
+    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    gen = torch.Generator().manual_seed(77)
+    for c, qn in enumerate((24, 24, 24, 24, 1, 1)):
+        q = (torch.randn(B, H, qn, D, generator=gen) * 0.7).to(dtype).cuda()
+        k = (torch.randn(B, KVH, qn, D, generator=gen) * 0.7).to(dtype).cuda()
+        v = (torch.randn(B, KVH, qn, D, generator=gen) * 0.7).to(dtype).cuda()
+        # teacher forcing: the hand-driven cache restarts from the fused one's state
+        for name in STATE:
+            getattr(by_hand, name)[0].copy_(getattr(fused, name)[0])
+        by_hand.seen_tokens_by_layer.copy_(fused.seen_tokens_by_layer)
+        by_hand.sync_host_counter()
+        first = by_hand._seen_host[0] == 0
+        sink_k, sink_v, sink_pos, sink_mask, ck, cv, key_pos, key_mask, _ = by_hand.get_vals(0)
+        top = 0 if first else int(max(sink_pos.max(), key_pos.max())) + 1
+        q_pos = torch.arange(top, top + qn, device="cuda:0").view(1, -1)
+        q_rot, _, _ = layer.rope(q, q_pos)
+        k_rot, _, _ = layer.rope(k, q_pos)
+        sink_rot, _, _ = layer.rope(sink_k, sink_pos)
+        cache_rot, _, _ = layer.rope(ck, key_pos)
+        arm = layer.cascade_attn_flash if c % 2 == 0 else layer.cascade_attn_eager
+        out_h, _ = arm(q_rot, k, v, expand(k_rot), expand(cv), expand(sink_rot), expand(sink_v), expand(cache_rot),
+                       sink_mask, key_mask, first, by_hand, 1 / math.sqrt(D), qn, False)
+        assert layer.last_attn_called == ("flash" if c % 2 == 0 else "eager") and layer.last_q_size == qn
+        out_f, _ = cascade_attention(q, k, v, fused, 0, inv_freq)
+        torch.cuda.synchronize()
+        err = (out_h.float() - out_f.float()).abs().max().item()
+        assert err <= tol(dtype), f"chunk {c}: out differs by {err:.3e}"
+        for name in META:
+            assert torch.equal(getattr(by_hand, name)[0], getattr(fused, name)[0]), f"chunk {c}: {name}"
+        assert by_hand._seen_host == fused._seen_host
+        same = by_hand.og_pos[0] == fused.og_pos[0]
+        assert same.float().mean().item() >= 0.99, f"chunk {c}: {(~same).sum().item()} slots hold another token"
+        sh, sf = by_hand.score_cache[0].float(), fused.score_cache[0].float()
+        assert_scores_close(torch.where(same, sh, sf), sf, dtype, f"chunk {c}: score cache")

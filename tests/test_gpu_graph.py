@@ -72,3 +72,47 @@ def test_graph_refuses_a_cache_whose_state_moved():
     cache.score_cache[0] = cache.score_cache[0].clone()
     with pytest.raises(_abi.CkvError):
         graph.step(q, k, k)
+
+
+def test_graph_survives_a_reset_of_its_cache():
+    """A step recorded on a full, eagerly filled cache; then ``reset()`` (which zeroes every state tensor in
+    place, so no address changes) and a partial refill: later steps must equal eager steps bit for bit — the
+    position ids of the token must come from the cache as it is now, not from the time of the recording."""
+    from cascading_kv_cache_amd.cascade_attention import DecodeStepGraph, cascade_attention, default_inv_freq
+
+    dtype, B, H, KVH, D, NS, W, C = torch.bfloat16, 1, 8, 2, 128, 4, 32, 2
+    ref, rep = make_cache(B, KVH, D, NS, W, C, dtype, True), make_cache(B, KVH, D, NS, W, C, dtype, True)
+    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    gen = torch.Generator().manual_seed(5)
+
+    def chunk(n):
+        q = (torch.randn(B, H, n, D, generator=gen) * 0.7).to(dtype).cuda()
+        k = (torch.randn(B, KVH, n, D, generator=gen) * 0.7).to(dtype).cuda()
+        v = (torch.randn(B, KVH, n, D, generator=gen) * 0.7).to(dtype).cuda()
+        return q, k, v
+
+    def both_step(graph, what):
+        q, k, v = chunk(1)
+        out_e, new_e = cascade_attention(q, k, v, ref, 0, inv_freq)
+        out_g, new_g = graph.step(q, k, v)
+        torch.cuda.synchronize()
+        assert torch.equal(bits(out_g), bits(out_e)), f"{what}: out"
+        assert torch.equal(bits(new_g), bits(new_e)), f"{what}: new scores"
+        for name in STATE:
+            assert torch.equal(bits(getattr(rep, name)[0]), bits(getattr(ref, name)[0])), f"{what}: {name}"
+
+    q, k, v = chunk(W * C + NS + 10)       # more than the cache holds: full and evicting
+    for c in (ref, rep):
+        cascade_attention(q, k, v, c, 0, inv_freq)
+    graph = DecodeStepGraph(rep, 0, inv_freq, H)
+    for step in range(4):
+        both_step(graph, f"full cache, step {step}")
+    assert graph.graph is not None
+    for c in (ref, rep):
+        c.reset(verbose=False)
+    q, k, v = chunk(NS + 9)                # past the sinks, far from full
+    for c in (ref, rep):
+        cascade_attention(q, k, v, c, 0, inv_freq)
+    for step in range(6):
+        both_step(graph, f"after reset, step {step}")
+    assert graph.graph is not None          # recorded again after the reset

@@ -115,3 +115,65 @@ def test_default_inv_freq_is_the_hf_formula():
     assert inv.dtype == torch.float32 and inv.shape == (64,)
     assert inv[0].item() == 1.0
     assert abs(inv[32].item() - 5e5 ** -0.5) < 1e-9
+
+
+def test_state_loaded_from_elsewhere_needs_a_counter_sync():
+    """State copied into a cache behind ``update``'s back (a saved stream, the module-level operator plus a hand
+    bump of ``seen_tokens_by_layer``, which the reference allows): the host mirror is stale until
+    ``sync_host_counter`` re-reads the device counter; ``check_host_counter`` says so."""
+    c = make()
+    c.pos[0][0, 0, :3] = torch.tensor([0, 1, 2])
+    c.seen_tokens_by_layer[0] = 5            # what a loader would restore
+    c.seen_tokens_by_layer[1] = 5
+    assert c.pos_shift(0) == 0               # stale mirror: no sink shift yet
+    with pytest.raises(_abi.CkvError):
+        c.check_host_counter(0)
+    assert c.sync_host_counter() == [5, 5]
+    c.check_host_counter(0)
+    c.check_host_counter(1)
+    assert c.pos_shift(0) == c.num_sink_tokens and c.get_vals(0)[6][0, :3].tolist() == [2, 3, 4]
+    gen = c._generation
+    c.reset(verbose=False)
+    assert c._generation == gen + 1 and c.sync_host_counter() == [0, 0]
+
+
+def test_reference_mixin_names_are_present():
+    """cascade/models/cascade_attention.py:202-229, 250-340, 343-367."""
+    from cascading_kv_cache_amd.cascade_attention import LlamaCascadeAttention, Qwen2CascadeAttention
+
+    for cls in (CascadeAttention, LlamaCascadeAttention, Qwen2CascadeAttention):
+        for name in ("forward", "qkv", "forward_cascade", "calc_scores", "cascade_attn_flash", "cascade_attn_eager", "rope"):
+            assert callable(getattr(cls, name)), (cls.__name__, name)
+    names = list(inspect.signature(CascadeAttention.cascade_attn_flash).parameters)[1:]
+    assert names == ["query_states", "key_states", "value_states", "key_states_pos", "v_states", "sink_key_states",
+                     "sink_value_states", "k_states", "sink_mask", "key_mask", "first_it", "past_key_value", "scale",
+                     "q_len", "homogeneous_heads"]
+
+
+def test_rope_flavours_agree_and_match_the_complex_rotation():
+    """``rope`` on the CPU (plain torch): the table lookup of the Qwen2 flavour and the direct computation of the
+    Llama flavour give the same rotation, and both equal multiplication by e^{i pos theta_j} on (x_j, x_{j+D/2})."""
+    from types import SimpleNamespace
+
+    from cascading_kv_cache_amd.cascade_attention import LlamaCascadeAttention, Qwen2CascadeAttention
+
+    D = 16
+    x = torch.randn(2, 3, 5, D, dtype=torch.float64, generator=torch.Generator().manual_seed(4))
+    pos = torch.tensor([[0, 1, 7, 30, 63]])
+    layers = []
+    for cls in (LlamaCascadeAttention, Qwen2CascadeAttention):
+        layer = cls()
+        layer.head_dim, layer.rope_theta, layer.max_position_embeddings = D, 1e4, 64
+        layer.config = SimpleNamespace()
+        layers.append(layer)
+    (a, cos_a, _), (b, cos_b, _) = layers[0].rope(x, pos), layers[1].rope(x, pos)
+    assert cos_a.shape == (1, 5, D) and cos_b.shape == (64, D)      # per position / whole table
+    assert torch.allclose(a, b, atol=1e-6)
+    inv = 1.0 / (1e4 ** (torch.arange(0, D, 2, dtype=torch.float64) / D))
+    z = torch.complex(x[..., :D // 2], x[..., D // 2:]) * torch.polar(torch.ones(5, D // 2, dtype=torch.float64),
+                                                                        pos[0, :, None].double() * inv)
+    want = torch.cat((z.real, z.imag), dim=-1)
+    assert torch.allclose(a, want, atol=1e-5)   # the angles are fp32 products, as in the reference
+    # tables handed back are reused
+    again, _, _ = layers[1].rope(x, pos, cos=cos_b, sin=layers[1].rope(x, pos)[2])
+    assert torch.equal(again, b)
