@@ -83,6 +83,7 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
     if (a.num_sink > 0 && (!a.sink_k || !a.sink_v || !a.sink_mask || !a.sink_pos)) return CKV_ERR_NULL;
     if (a.S > 0 && (!a.cache_k || !a.cache_v || !a.mask || !a.pos)) return CKV_ERR_NULL;
     if (!(a.beta > 0.0) || !(a.beta <= 1.0)) return CKV_ERR_SHAPE;
+    if (!(a.scale > 0.f)) return CKV_ERR_SHAPE;  // queries and keys are each multiplied by its square root
     if (!a.workspace || a.workspace_bytes < ckv_attn_workspace_bytes(a.B, a.H, a.KVH, a.Q, a.D, a.num_sink, a.S, a.dtype))
         return CKV_ERR_WORKSPACE;
     if (decode_supported(a)) return launch_decode(a, stream);
@@ -124,6 +125,7 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
         mp.new_mode = 1;
         mp.B = a.B; mp.H = a.H; mp.KVH = a.KVH; mp.Q = a.Q; mp.n = N; mp.n_pad = mfma_n_pad(N);
         mp.scale = a.scale;
+        mp.key_scale = sqrtf(a.scale);
         mp.dtype = a.dtype;
         rc = launch_mfma(mp, stream);
         if (rc) return rc;
@@ -147,7 +149,7 @@ extern "C" int ckv_attn(const ckv_attn_args* args, void* stream_) {
         cp.w_new = w.w_new;
         cp.new_mode = 1;
         cp.B = a.B; cp.H = a.H; cp.KVH = a.KVH; cp.Q = a.Q; cp.N = N; cp.D = a.D;
-        cp.scale = a.scale;
+        cp.scale = 1.f;  // the staged queries and keys each carry sqrt(scale), rounded in as the eager path does
         cp.dtype = a.dtype;
         rc = launch_core_generic(cp, stream);
         if (rc) return rc;
@@ -239,6 +241,7 @@ extern "C" int ckv_attn_dense(const ckv_dense_args* args, void* stream_) {
         mp.new_mode = 0;  // every key is weighted by the query row alone (flash_attention.py:73-77)
         mp.B = a.B; mp.H = a.H; mp.KVH = a.H; mp.Q = a.n_ctx; mp.n = a.n_kv; mp.n_pad = mfma_n_pad(a.n_kv);
         mp.scale = a.scale;
+        mp.key_scale = 1.f;
         mp.dtype = a.dtype;
         rc = launch_mfma(mp, stream);
         if (rc) return rc;

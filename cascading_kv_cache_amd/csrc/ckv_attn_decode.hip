@@ -34,6 +34,18 @@ __device__ inline float round_t(float v) {
     return Elem<T>::to_float(Elem<T>::from_float(v));
 }
 
+// One rotation pair with the roundings of the eager path, which evaluates x*cos + rotate_half(x)*sin in the tensor
+// dtype (cascade_attention.py:31-35; cos and sin cast to the dtype, modeling_llama.py:219-220) and then multiplies
+// queries and keys alike by sqrt(softmax scale) (cascade_attention.py:284-291): every product and every sum is
+// rounded on its own (no fused multiply-add), `c` and `s` arrive rounded, `post` is the sqrt(scale) factor.
+template <typename T>
+__device__ inline void rope_ref(float x1, float x2, float c, float s, float post, float& r1, float& r2) {
+    r1 = round_t<T>(__fadd_rn(round_t<T>(__fmul_rn(x1, c)), round_t<T>(__fmul_rn(-x2, s))));
+    r2 = round_t<T>(__fadd_rn(round_t<T>(__fmul_rn(x2, c)), round_t<T>(__fmul_rn(x1, s))));
+    r1 = round_t<T>(__fmul_rn(r1, post));
+    r2 = round_t<T>(__fmul_rn(r2, post));
+}
+
 // all-reduce (sum) inside each row of 16 lanes with DPP: quad xor 1, quad xor 2, half mirror, mirror
 __device__ inline float row16_sum(float x) {
     int v = __float_as_int(x);
@@ -92,7 +104,8 @@ struct DecodeParams {
     int64_t N;         // num_sink + S + 1
     int tiles;
     int shared_pos;
-    float scale_log2;
+    float key_scale;   // sqrt(softmax scale): rotated queries and keys both carry it, rounded in (see rope_ref)
+    float scale_log2;  // what the logits are still multiplied by: log2(e)
     // Streaming kernel: items exist only for tiles that can hold a visible key, numbered in tile order: the
     // first `tiles_pre` tiles (sinks and the cache slots below the caller's `filled_slots` bound) and the tile
     // of the new token (`tiles - 1`) when it is not one of them.  A cache that is still filling is mostly hidden.
@@ -131,8 +144,8 @@ __global__ void decode_q_kernel(DecodeParams p) {
     float sn, cs;
     sincosf(__fmul_rn((float)a.q_pos[0], f), &sn, &cs);
     const float x1 = Elem<T>::to_float(q[j * a.q_stride[3]]), x2 = Elem<T>::to_float(q[(j + 64) * a.q_stride[3]]);
-    // the eager path rotates in the tensor dtype (cascade_attention.py:31-35)
-    const float r1 = round_t<T>(x1 * cs - x2 * sn), r2 = round_t<T>(x2 * cs + x1 * sn);
+    float r1, r2;
+    rope_ref<T>(x1, x2, round_t<T>(cs), round_t<T>(sn), p.key_scale, r1, r2);
     p.qrot[row * kD + j] = r1 * p.scale_log2;
     p.qrot[row * kD + 64 + j] = r2 * p.scale_log2;
     ((T*)p.qrot_t)[row * kD + j] = Elem<T>::from_float(r1);
@@ -194,6 +207,8 @@ __global__ void __launch_bounds__(256) decode_main_kernel(DecodeParams p) {
                 const int f = 4 * j + e;
                 const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
                 sincosf(__fmul_rn((float)pos, fr), &sn[s][e], &cs[s][e]);
+                sn[s][e] = round_t<T>(sn[s][e]);
+                cs[s][e] = round_t<T>(cs[s][e]);
             }
         }
     }
@@ -246,9 +261,11 @@ __global__ void __launch_bounds__(256) decode_main_kernel(DecodeParams p) {
                     const int f = 4 * j + e;
                     const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
                     sincosf(__fmul_rn((float)posv[s], fr), &s_, &c_);
+                    s_ = round_t<T>(s_);
+                    c_ = round_t<T>(c_);
                 }
-                const float ra = ka[e] * c_ - kb[e] * s_;
-                const float rb = kb[e] * c_ + ka[e] * s_;
+                float ra, rb;
+                rope_ref<T>(ka[e], kb[e], c_, s_, p.key_scale, ra, rb);
 #pragma unroll
                 for (int g = 0; g < G; g++) acc[g] = fmaf(ra, qa[g][e], fmaf(rb, qb[g][e], acc[g]));
             }
@@ -383,6 +400,29 @@ struct Mma16<__half> {
     }
 };
 
+// rope_ref on packed words: w1 holds elements (j, j+1) of a key row, w2 their partners (j+64, j+65); c0/s0 and
+// c1/s1 are the rounded cos/sin of the two pairs.  Products of two 16-bit values and sums of two 16-bit values are
+// exact in fp32, so each packed conversion below is one of the reference's roundings.
+template <typename T>
+__device__ inline void rope_ref_words(uint32_t w1, uint32_t w2, float c0, float s0, float c1, float s1, float post,
+                                      uint32_t& o1, uint32_t& o2) {
+    const float a0 = Mma16<T>::lo(w1), a1 = Mma16<T>::hi(w1), b0 = Mma16<T>::lo(w2), b1 = Mma16<T>::hi(w2);
+    const uint32_t p0 = Mma16<T>::pack2(a0 * c0, b0 * s0), q0 = Mma16<T>::pack2(b0 * c0, a0 * s0);
+    const uint32_t p1 = Mma16<T>::pack2(a1 * c1, b1 * s1), q1 = Mma16<T>::pack2(b1 * c1, a1 * s1);
+    o1 = Mma16<T>::pack2(Mma16<T>::lo(p0) - Mma16<T>::hi(p0), Mma16<T>::lo(p1) - Mma16<T>::hi(p1));
+    o2 = Mma16<T>::pack2(Mma16<T>::lo(q0) + Mma16<T>::hi(q0), Mma16<T>::lo(q1) + Mma16<T>::hi(q1));
+    o1 = Mma16<T>::pack2(Mma16<T>::lo(o1) * post, Mma16<T>::hi(o1) * post);
+    o2 = Mma16<T>::pack2(Mma16<T>::lo(o2) * post, Mma16<T>::hi(o2) * post);
+}
+// cos / sin of an angle, rounded to the tensor dtype as the reference's rotary module hands them out
+template <typename T>
+__device__ inline void sincos_ref(float angle, float* sn, float* cs) {
+    float s_, c_;
+    fast_sincos(angle, &s_, &c_);
+    *sn = Mma16<T>::lo(Mma16<T>::pack2(s_, 0.f));
+    *cs = Mma16<T>::lo(Mma16<T>::pack2(c_, 0.f));
+}
+
 template <typename T, int G>
 __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p) {
     extern __shared__ __align__(16) float red[];  // [16][G][128] partials, [16][G] max, [16][G] sum, [4][32][8] logits
@@ -432,7 +472,7 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
                 for (int e = 0; e < 8; e++) {
                     const int f = 32 * ks + 8 * kq + e;
                     const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                    fast_sincos(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
+                    sincos_ref<T>(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
                 }
         }
     }
@@ -500,7 +540,7 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
                     for (int e = 0; e < 8; e++) {
                         const int f = 32 * ks + 8 * kq + e;
                         const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                        fast_sincos(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
+                        sincos_ref<T>(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
                     }
             }
             uint4 kop[4];
@@ -511,12 +551,7 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
                 uint32_t o1[4], o2[4];
 #pragma unroll
                 for (int w = 0; w < 4; w++) {
-                    const float a0 = Mma16<T>::lo(w1[w]), a1 = Mma16<T>::hi(w1[w]);
-                    const float b0 = Mma16<T>::lo(w2[w]), b1 = Mma16<T>::hi(w2[w]);
-                    const float c0 = cs[gi][ks][2 * w], s0 = sn[gi][ks][2 * w];
-                    const float c1 = cs[gi][ks][2 * w + 1], s1 = sn[gi][ks][2 * w + 1];
-                    o1[w] = Mma16<T>::pack2(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
-                    o2[w] = Mma16<T>::pack2(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+                    rope_ref_words<T>(w1[w], w2[w], cs[gi][ks][2 * w], sn[gi][ks][2 * w], cs[gi][ks][2 * w + 1], sn[gi][ks][2 * w + 1], p.key_scale, o1[w], o2[w]);
                 }
                 kop[ks] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
                 kop[ks + 2] = make_uint4(o2[0], o2[1], o2[2], o2[3]);
@@ -738,7 +773,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                 for (int e = 0; e < 8; e++) {
                     const int f = 32 * ks + 8 * kq + e;
                     const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                    fast_sincos(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
+                    sincos_ref<T>(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
                 }
         }
         // Rows of hidden slots may hold anything (their probability is zero, but 0 * NaN is not), so
@@ -914,12 +949,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                     uint32_t o1[4], o2[4];
 #pragma unroll
                     for (int w = 0; w < 4; w++) {
-                        const float a0 = Mma16<T>::lo(w1[w]), a1 = Mma16<T>::hi(w1[w]);
-                        const float b0 = Mma16<T>::lo(w2[w]), b1 = Mma16<T>::hi(w2[w]);
-                        const float c0 = cs[ks][2 * w], s0 = sn[ks][2 * w];
-                        const float c1 = cs[ks][2 * w + 1], s1 = sn[ks][2 * w + 1];
-                        o1[w] = Mma16<T>::pack2(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
-                        o2[w] = Mma16<T>::pack2(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+                        rope_ref_words<T>(w1[w], w2[w], cs[ks][2 * w], sn[ks][2 * w], cs[ks][2 * w + 1], sn[ks][2 * w + 1], p.key_scale, o1[w], o2[w]);
                     }
                     kop[ks] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
                     kop[ks + 2] = make_uint4(o2[0], o2[1], o2[2], o2[3]);
@@ -1117,7 +1147,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                 for (int e = 0; e < 8; e++) {
                     const int f = 32 * ks + 8 * kq + e;
                     const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                    fast_sincos(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
+                    sincos_ref<T>(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
                 }
         }
         // rows of hidden slots are zeroed on the way into the P.V product (0 * NaN): masks of this lane's
@@ -1257,12 +1287,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                     uint32_t o1[4], o2[4];
 #pragma unroll
                     for (int w = 0; w < 4; w++) {
-                        const float a0 = Mma16<T>::lo(w1[w]), a1 = Mma16<T>::hi(w1[w]);
-                        const float b0 = Mma16<T>::lo(w2[w]), b1 = Mma16<T>::hi(w2[w]);
-                        const float c0 = cs[ks][2 * w], s0 = sn[ks][2 * w];
-                        const float c1 = cs[ks][2 * w + 1], s1 = sn[ks][2 * w + 1];
-                        o1[w] = Mma16<T>::pack2(a0 * c0 - b0 * s0, a1 * c1 - b1 * s1);
-                        o2[w] = Mma16<T>::pack2(b0 * c0 + a0 * s0, b1 * c1 + a1 * s1);
+                        rope_ref_words<T>(w1[w], w2[w], cs[ks][2 * w], sn[ks][2 * w], cs[ks][2 * w + 1], sn[ks][2 * w + 1], p.key_scale, o1[w], o2[w]);
                     }
                     kop[ks] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
                     kop[ks + 2] = make_uint4(o2[0], o2[1], o2[2], o2[3]);
@@ -1978,7 +2003,8 @@ int launch_decode(const ckv_attn_args& a, hipStream_t stream) {
     p.part_o = reinterpret_cast<float*>(w); w += align_up(a.B * a.H * tiles_max * kD * 4, 256);
     p.lse2 = reinterpret_cast<float*>(w);
     p.shared_pos = a.sink_pos_stride[0] == 0 && a.sink_pos_stride[1] == 0 && a.pos_stride[0] == 0 && a.pos_stride[1] == 0;
-    p.scale_log2 = a.scale * 1.4426950408889634f;
+    p.key_scale = sqrtf(a.scale);
+    p.scale_log2 = 1.4426950408889634f;  // queries and keys each carry sqrt(scale)
     switch (a.dtype) {
         case CKV_F32: return run_decode_g<float>(p, (int)G, stream);
         case CKV_F16: return run_decode_g<__half>(p, (int)G, stream);

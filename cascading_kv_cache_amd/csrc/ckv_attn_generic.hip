@@ -35,11 +35,12 @@ __global__ void weights_kernel(float* w_ema, float* w_new, int64_t Q, double bet
 // prologue: rotate and gather.  One thread per (row, rotation pair).
 // Rotation is evaluated in the tensor dtype exactly like x*cos + rotate_half(x)*sin
 // (cascade_attention.py:31-35) with cos/sin from fp32 angles cast to the dtype
-// (modeling_llama.py:205-220).
+// (modeling_llama.py:205-220); the rotated row is then multiplied by sqrt(softmax scale) and rounded
+// again, as the eager path does to queries and keys alike (cascade_attention.py:284-291).
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __device__ inline void rotate_pair(const T* src, int64_t sd, T* dst, int64_t j, int64_t half, int64_t pos,
-                                   const float* inv_freq, float theta, int64_t D) {
+                                   const float* inv_freq, float theta, int64_t D, float post) {
     const float f = inv_freq ? inv_freq[j] : 1.0f / powf(theta, (float)(2 * j) / (float)D);
     const float ang = __fmul_rn((float)pos, f);
     float sn, cs;
@@ -51,12 +52,12 @@ __device__ inline void rotate_pair(const T* src, int64_t sd, T* dst, int64_t j, 
     // out[j] = x1*cos + (-x2)*sin ; out[j+half] = x2*cos + x1*sin, each product rounded first
     const float o1 = round_t<T>(__fadd_rn(round_t<T>(__fmul_rn(x1, cs)), round_t<T>(__fmul_rn(-x2, sn))));
     const float o2 = round_t<T>(__fadd_rn(round_t<T>(__fmul_rn(x2, cs)), round_t<T>(__fmul_rn(x1, sn))));
-    dst[j] = Elem<T>::from_float(o1);
-    dst[j + half] = Elem<T>::from_float(o2);
+    dst[j] = Elem<T>::from_float(__fmul_rn(o1, post));
+    dst[j + half] = Elem<T>::from_float(__fmul_rn(o2, post));
 }
 
 template <typename T>
-__global__ void prep_generic_kernel(ckv_attn_args a, T* qr, T* kr, T* vc, uint8_t* kmasked) {
+__global__ void prep_generic_kernel(ckv_attn_args a, T* qr, T* kr, T* vc, uint8_t* kmasked, float post) {
     const int64_t D = a.D, half = D / 2, NS = a.num_sink, S = a.S, Q = a.Q;
     const int64_t N = NS + S + Q;
     const int64_t n_key_items = a.B * a.KVH * N * half;
@@ -93,7 +94,7 @@ __global__ void prep_generic_kernel(ckv_attn_args a, T* qr, T* kr, T* vc, uint8_
         }
         T* kd = kr + ((b * a.KVH + kvh) * N + n) * D;
         T* vd = vc + ((b * a.KVH + kvh) * N + n) * D;
-        rotate_pair<T>(ks, sd, kd, j, half, pos, a.inv_freq, a.rope_theta, D);
+        rotate_pair<T>(ks, sd, kd, j, half, pos, a.inv_freq, a.rope_theta, D, post);
         vd[j] = vs[j * sd];
         vd[j + half] = vs[(j + half) * sd];
     }
@@ -104,7 +105,7 @@ __global__ void prep_generic_kernel(ckv_attn_args a, T* qr, T* kr, T* vc, uint8_
         const int64_t b = idx / (half * Q * a.H);
         const T* qs = (const T*)a.q + b * a.q_stride[0] + h * a.q_stride[1] + m * a.q_stride[2];
         T* qd = qr + ((b * a.H + h) * Q + m) * D;
-        rotate_pair<T>(qs, a.q_stride[3], qd, j, half, a.q_pos[m], a.inv_freq, a.rope_theta, D);
+        rotate_pair<T>(qs, a.q_stride[3], qd, j, half, a.q_pos[m], a.inv_freq, a.rope_theta, D, post);
     }
 }
 
@@ -378,18 +379,19 @@ int launch_prep_generic(const PrepProblem& p, hipStream_t stream) {
     if (qitems > items) items = qitems;
     if (a.num_sink + a.S > items) items = a.num_sink + a.S;
     const dim3 grid((unsigned)((items + 255) / 256)), block(256);
+    const float post = sqrtf(a.scale);  // on queries and keys: the caller's core kernel multiplies by nothing more
     switch (a.dtype) {
         case CKV_F32:
             hipLaunchKernelGGL(prep_generic_kernel<float>, grid, block, 0, stream, a, (float*)p.qr, (float*)p.kr,
-                               (float*)p.vc, p.kmasked);
+                               (float*)p.vc, p.kmasked, post);
             break;
         case CKV_F16:
             hipLaunchKernelGGL(prep_generic_kernel<__half>, grid, block, 0, stream, a, (__half*)p.qr, (__half*)p.kr,
-                               (__half*)p.vc, p.kmasked);
+                               (__half*)p.vc, p.kmasked, post);
             break;
         case CKV_BF16:
             hipLaunchKernelGGL(prep_generic_kernel<__hip_bfloat16>, grid, block, 0, stream, a,
-                               (__hip_bfloat16*)p.qr, (__hip_bfloat16*)p.kr, (__hip_bfloat16*)p.vc, p.kmasked);
+                               (__hip_bfloat16*)p.qr, (__hip_bfloat16*)p.kr, (__hip_bfloat16*)p.vc, p.kmasked, post);
             break;
         default: return CKV_ERR_DTYPE;
     }

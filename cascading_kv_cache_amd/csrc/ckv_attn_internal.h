@@ -102,6 +102,9 @@ struct MfmaProblem {
     int new_mode;
     int64_t B, H, KVH, Q, n, n_pad;
     float scale;
+    float key_scale;       // keys with position ids are multiplied by this after rotation and rounded again, the
+                           // queries carry scale / key_scale: sqrt(scale) for the cascade path, which follows the
+                           // eager arm (cascade_attention.py:284-291); 1 for keys that arrive rotated
     int dtype;
 };
 

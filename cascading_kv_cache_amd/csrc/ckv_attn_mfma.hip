@@ -89,6 +89,26 @@ __host__ __device__ inline int vt_slot(int k) {
 // ---------------------------------------------------------------------------------------------
 // staging
 // ---------------------------------------------------------------------------------------------
+// Rotary embedding of two neighbouring pairs (x1a, x2a), (x1b, x2b) (elements j, j+64 and j+1, j+65 of a row)
+// with the roundings of the eager path, which evaluates x*cos + rotate_half(x)*sin in the tensor dtype
+// (cascade_attention.py:31-35): cos and sin arrive rounded to the dtype (modeling_llama.py:219-220), each
+// product is rounded, then the sum, and then the product with sqrt(softmax scale) that the eager path applies
+// to queries and keys alike (cascade_attention.py:284-291); `post` is that factor (1: no such product).
+// Products of two 16-bit values and sums of two 16-bit values are exact in fp32, so rounding the fp32
+// result once is the reference's rounding.  Returns the packed pairs (first halves, second halves).
+template <typename T>
+__device__ inline void rope_ref_pairs(float x1a, float x1b, float x2a, float x2b, float ca, float sa, float cb, float sb,
+                                      float post, bool scale_after, uint32_t& first, uint32_t& second) {
+    const uint32_t pa = Mma<T>::pack2(x1a * ca, x2a * sa), qa = Mma<T>::pack2(x2a * ca, x1a * sa);
+    const uint32_t pb = Mma<T>::pack2(x1b * cb, x2b * sb), qb = Mma<T>::pack2(x2b * cb, x1b * sb);
+    first = Mma<T>::pack2(Mma<T>::lo_f(pa) - Mma<T>::hi_f(pa), Mma<T>::lo_f(pb) - Mma<T>::hi_f(pb));
+    second = Mma<T>::pack2(Mma<T>::lo_f(qa) + Mma<T>::hi_f(qa), Mma<T>::lo_f(qb) + Mma<T>::hi_f(qb));
+    if (scale_after) {
+        first = Mma<T>::pack2(Mma<T>::lo_f(first) * post, Mma<T>::hi_f(first) * post);
+        second = Mma<T>::pack2(Mma<T>::lo_f(second) * post, Mma<T>::hi_f(second) * post);
+    }
+}
+
 struct KeySegment {
     const void* k;
     const void* v;
@@ -104,6 +124,7 @@ struct StageParams {
     KeySegment seg[3];
     const float* inv_freq;
     float theta;
+    float key_scale;         // rotated keys are multiplied by this and rounded again (1: they are not)
     int shared_pos;          // every (b, kvh) uses position row [0, 0]
     void* kr;                // (B*KVH, n_pad/64) K tile images, see k_image_off
     void* vt;                // (B*KVH, n_pad/64) V^T tile images, see v_image_off
@@ -164,8 +185,11 @@ __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int sp
             const int j = stage_pair(quarter, i);
             const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
             fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
+            sn[i] = Mma<T>::round1(sn[i]);
+            cs[i] = Mma<T>::round1(cs[i]);
         }
     }
+    const bool key_scaled = p.key_scale != 1.0f;
     const int64_t nbh = p.B * p.KVH;
     // the rows of unit bh as this thread's eight 16-byte pieces (zeros past the last key)
     struct Rows {
@@ -223,6 +247,8 @@ __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int sp
                         const int j = stage_pair(quarter, i);
                         const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
                         fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
+                        sn[i] = Mma<T>::round1(sn[i]);
+                        cs[i] = Mma<T>::round1(cs[i]);
                     }
                 }
                 // on packed pairs: two elements per word, converted and rounded (to nearest even, like the
@@ -233,8 +259,8 @@ __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int sp
                 for (int k = 0; k < 8; k++) {
                     const float x1a = Mma<T>::lo_f(lw[k]), x1b = Mma<T>::hi_f(lw[k]);
                     const float x2a = Mma<T>::lo_f(hw[k]), x2b = Mma<T>::hi_f(hw[k]);
-                    lw[k] = Mma<T>::pack2(x1a * cs[2 * k] - x2a * sn[2 * k], x1b * cs[2 * k + 1] - x2b * sn[2 * k + 1]);
-                    hw[k] = Mma<T>::pack2(x2a * cs[2 * k] + x1a * sn[2 * k], x2b * cs[2 * k + 1] + x1b * sn[2 * k + 1]);
+                    rope_ref_pairs<T>(x1a, x1b, x2a, x2b, cs[2 * k], sn[2 * k], cs[2 * k + 1], sn[2 * k + 1], p.key_scale,
+                                      key_scaled, lw[k], hw[k]);
                 }
             }
         }
@@ -292,7 +318,7 @@ struct StageQParams {
     void* qr;                // (B*H, Q, D) contiguous
     int64_t rows;            // B*H*Q
     int64_t H, Q;
-    float qscale;            // softmax scale * log2(e), folded into the staged queries
+    float qscale;            // folded into the staged queries: softmax scale * log2(e), over the factor the keys carry
     int vec;                 // source rows can be read 16 bytes at a time
 };
 
@@ -313,6 +339,8 @@ __device__ inline void stage_q_block(const StageQParams& p, int blk, int share_i
             const int j = stage_pair(quarter, i);
             const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
             fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
+            sn[i] = Mma<T>::round1(sn[i]);
+            cs[i] = Mma<T>::round1(cs[i]);
         }
     }
     const int64_t nbh = p.rows / p.Q;
@@ -336,9 +364,10 @@ __device__ inline void stage_q_block(const StageQParams& p, int blk, int share_i
             }
         }
     };
-    // the softmax scale (times log2 e) rides on the staged queries: one rounding to the tensor
-    // dtype after rotation and scaling, and the attention kernels exponentiate the products as
-    // they come out of the matrix pipe
+    // the softmax scale (times log2 e) rides on the staged queries, so the attention kernels exponentiate the
+    // products as they come out of the matrix pipe: rotated with the eager path's roundings, then one rounding
+    // of the product with qscale (the eager path rounds the product with sqrt(scale) there; log2 e has to ride
+    // on one of the two operands, and noise on a query averages out over the rows a score sums)
     auto finish_row = [&](int64_t bh, Row& r) {
         if (bh >= nbh) return;
         uint32_t* lw = reinterpret_cast<uint32_t*>(r.lo);
@@ -348,10 +377,8 @@ __device__ inline void stage_q_block(const StageQParams& p, int blk, int share_i
             const float x1a = Mma<T>::lo_f(lw[k]), x1b = Mma<T>::hi_f(lw[k]);
             const float x2a = Mma<T>::lo_f(hw[k]), x2b = Mma<T>::hi_f(hw[k]);
             if (p.q_pos) {
-                lw[k] = Mma<T>::pack2((x1a * cs[2 * k] - x2a * sn[2 * k]) * p.qscale,
-                                      (x1b * cs[2 * k + 1] - x2b * sn[2 * k + 1]) * p.qscale);
-                hw[k] = Mma<T>::pack2((x2a * cs[2 * k] + x1a * sn[2 * k]) * p.qscale,
-                                      (x2b * cs[2 * k + 1] + x1b * sn[2 * k + 1]) * p.qscale);
+                rope_ref_pairs<T>(x1a, x1b, x2a, x2b, cs[2 * k], sn[2 * k], cs[2 * k + 1], sn[2 * k + 1], p.qscale, true,
+                                  lw[k], hw[k]);
             } else {
                 lw[k] = Mma<T>::pack2(x1a * p.qscale, x1b * p.qscale);
                 hw[k] = Mma<T>::pack2(x2a * p.qscale, x2b * p.qscale);
@@ -1284,6 +1311,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         }
         sp.inv_freq = mp.inv_freq;
         sp.theta = mp.theta;
+        sp.key_scale = mp.key_scale;
         sp.shared_pos = mp.shared_pos;
         sp.kr = mp.kr;
         sp.vt = mp.vt;
@@ -1309,7 +1337,7 @@ int run_mfma(const MfmaProblem& mp, hipStream_t stream) {
         sq.qr = mp.qr;
         sq.rows = mp.B * mp.H * mp.Q;
         sq.H = mp.H; sq.Q = mp.Q;
-        sq.qscale = scale_log2;
+        sq.qscale = mp.q_pos ? scale_log2 / mp.key_scale : scale_log2;  // rotated keys carry key_scale
         sq.vec = mp.q_stride[3] == 1 && reinterpret_cast<uintptr_t>(mp.q) % 16 == 0 && mp.q_stride[0] % 8 == 0 &&
                  mp.q_stride[1] % 8 == 0 && mp.q_stride[2] % 8 == 0;
         {

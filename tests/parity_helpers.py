@@ -122,5 +122,13 @@ class FlipLedger:
                 f"slots {self.min_margin:.3e} .. {self.max_margin:.3e} (worst {self.worst_ratio:.2f} of the 2-eps bound)")
 
 
+def flip_bound(ledger):
+    """How many slots of a 16-bit stream may hold another token than the oracle's (each of them already shown to be a
+    tie at the score tolerance): 0.25 % of the slots compared over the stream, about twice the largest rate measured
+    on any test stream (18 of 16384 slots; the streams of a few thousand slots show 0 to 2), and never fewer than 3
+    so that the smallest streams are not held to a fraction of a slot."""
+    return max(3, int(0.0025 * ledger.compared))
+
+
 def clone_oracle(cpu):
     return copy.deepcopy(cpu)
