@@ -14,8 +14,10 @@ sub-records carry their own roofline: `decode` (the single-token steps of the he
 bandwidth), `update` (the cache update of the headline chunk against HBM bandwidth, bytes counted from the
 state difference), `cfg2_prefill` (B=2, 8 x 2048 slots, 2048-token chunks) and `cfg3_decode` (B=16,
 4 x 8192 slots, one token) and `cfg4_full_model` (the whole 32-layer Llama-3.1-8B-shape decoder with random weights:
-131072 prompt tokens in 4096-token strides, then 256 greedy tokens; `--only cfg5` runs the Qwen2-7B-shape workload
-the same way).  `cpu_baseline` times the CPU oracle (the reference's eager PyTorch path restated,
+131072 prompt tokens in 4096-token strides, then 256 greedy tokens), `cfg5_full_model` (the Qwen2-7B-shape decoder,
+B=4, 262144 tokens per stream), each checked after its stream (every layer saw every token, every ring full, position
+ids a permutation, finite logits), `cfg1_gpu` (config 1, float32, on the device beside `cpu_config1`) and
+`short_stride` (128- and 512-token strides on the headline cache).  `cpu_baseline` times the CPU oracle (the reference's eager PyTorch path restated,
 plus the serial update) on a bounded sample of the headline workload on the box's host cores.
 """
 import argparse
@@ -457,6 +459,8 @@ def run_model(cfg, device, dtype, prompt=None):
     cache = model.new_cache(cfg["window"], cfg["cascades"], batch=cfg["B"])
     stride = cfg["stride"]
 
+    last = {}
+
     def stream(n_prompt, n_new):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -468,19 +472,40 @@ def run_model(cfg, device, dtype, prompt=None):
         for _ in range(n_new):
             logits = model(torch.argmax(logits[:, -1, :], dim=-1)[:, None], cache)
         torch.cuda.synchronize()
-        return t1 - t0, time.perf_counter() - t1
+        t2 = time.perf_counter()
+        last["logits"] = logits
+        return t1 - t0, t2 - t1
 
     with torch.no_grad():
         stream(2 * stride, 2)
         cache.reset(verbose=False)
         tp, td = stream(prompt, cfg["new"])
+    # untimed: the stream really went through every layer's cache.  Every token of the prompt and every generated
+    # token was fed once; a stream longer than sinks + window leaves every slot occupied and every ring full.
+    fed = prompt + cfg["new"]
+    W = cfg["window"] // cfg["cascades"]
+    checks = {"layers": mcfg.num_layers, "tokens_fed_per_stream": fed}
+    assert cache.seen_tokens_by_layer.tolist() == [fed] * mcfg.num_layers, "a layer missed tokens"
+    assert cache._seen_host == [fed] * mcfg.num_layers, "host counters out of step with the device"
+    assert bool(torch.isfinite(last["logits"].float()).all()), "non-finite logits"
+    if fed > cfg["window"] + 64:
+        for l in range(mcfg.num_layers):
+            assert not bool(cache.mask[l].any()) and not bool(cache.sink_mask[l].any()), f"layer {l}: empty slots"
+            assert bool((cache.stored_tokens[l] == W).all()), f"layer {l}: a ring is not full"
+            assert bool((cache.stored_sinks[l] == 64).all()), f"layer {l}: sinks"
+            row = cache.pos[l][0, 0].sort().values
+            assert torch.equal(row, torch.arange(cfg["window"], device=device)), f"layer {l}: position ids are not a permutation"
+        checks["every_layer_full_and_consistent"] = True
     n_p, n_d = cfg["B"] * prompt, cfg["B"] * cfg["new"]
     rec = {"workload": f"{cfg['preset']} shape, {mcfg.num_layers} layers, random weights, B={cfg['B']}: {prompt} uniform random "
                        f"token ids per stream in {stride}-token strides through sink 64 + {cfg['cascades']} x "
                        f"{cfg['window'] // cfg['cascades']} slots, then {cfg['new']} greedy tokens",
            "tokens_per_s": (n_p + n_d) / (tp + td), "prefill_tokens_per_s": n_p / tp, "prefill_s": tp,
-           "decode_tokens_per_s": (n_d / td) if n_d else None, "decode_ms_per_token": (td / cfg["new"] * 1e3) if n_d else None}
-    del model, cache, ids
+           "decode_tokens_per_s": (n_d / td) if n_d else None, "decode_ms_per_token": (td / cfg["new"] * 1e3) if n_d else None,
+           "checked_after_the_stream": checks}
+    if prompt != cfg["prompt"]:
+        rec["truncated"] = f"prompt shortened from {cfg['prompt']} to {prompt} tokens per stream (--model-prompt)"
+    del model, cache, ids, last
     torch.cuda.empty_cache()
     return rec
 
@@ -511,7 +536,7 @@ def cpu_model():
 
 def run_cpu_baseline(cache, pool, dtype):
     """The oracle on the host: the reference's eager path restated, on a bounded sample of the headline
-    workload (the same full cache contents, a 64-token chunk instead of 4096)."""
+    workload (the same full cache contents, a 256-token chunk instead of 4096)."""
     from oracle.attention import OracleCascadeAttention
     from oracle.update import OracleCache
 
@@ -524,7 +549,7 @@ def run_cpu_baseline(cache, pool, dtype):
         getattr(o, name).copy_(getattr(cache, name)[0].cpu())
     o.seen_tokens.fill_(int(cache._seen_host[0]))
     layer = OracleCascadeAttention(cfg["H"], cfg["KVH"], cfg["D"], rope_theta=cfg["theta"])
-    q_s = 64
+    q_s = 256
     q, k, v = (t[:, :, :q_s].cpu().contiguous() for t in pool[0])
     layer.query_pos = torch.arange(q_s).view(1, -1)
     layer.forward(q, k, v, o)  # untimed: first-touch of the cache copy and thread start-up
@@ -538,8 +563,8 @@ def run_cpu_baseline(cache, pool, dtype):
     dt = time.perf_counter() - t0
     return dict(value=cfg["B"] * q_s * reps / dt, unit="tokens/s", cores=threads, kind="port",
                 host_cores_reported=os.cpu_count(), cpu=cpu_model(),
-                sample=f"{reps} x (one {q_s}-token chunk over the full 64+65536-slot cache), i.e. 1/64 of one prefill "
-                       f"chunk's tokens per repetition; eager attention + score EMA + serial update in bf16 on "
+                sample=f"{reps} x (one {q_s}-token chunk over the full 64+65536-slot cache), i.e. 1/{cfg['Q'] // q_s} of one "
+                       f"prefill chunk's tokens per repetition; eager attention + score EMA + serial update in bf16 on "
                        f"{threads} threads")
 
 
@@ -562,6 +587,67 @@ def run_cpu_config1():
     dt = time.perf_counter() - t0
     return dict(value=4096 / dt, unit="tokens/s", seconds=dt, cores=host_threads(), kind="port",
                 sample="config 1 in full: 4096 tokens in 16 chunks of 256, float32")
+
+
+def run_gpu_config1(device):
+    """Config 1 on the device, beside `cpu_config1`: the same float32 stream (B=1, 32q/8kv heads, head_dim 128,
+    sink 4, window 512 in 4 cascades, 4096 tokens in 16 chunks of 256) through the library's fp32-math kernels."""
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
+    from cascading_kv_cache_amd.cascading_cache import CascadingKVCache
+
+    cache = CascadingKVCache(window_length=128, num_sink_tokens=4, max_batch_size=1, heads=8, dim=128, max_seq_len=512,
+                             device=device, dtype=torch.float32, layers=1, verbose=False)
+    inv_freq = default_inv_freq(128, 5e5, device)
+    g = torch.Generator().manual_seed(1)
+    chunks = [tuple(torch.randn(1, h, 256, 128, generator=g).to(device) for h in (32, 8, 8)) for _ in range(16)]
+
+    def stream():
+        cache.reset(verbose=False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for q, k, v in chunks:
+            cascade_attention(q, k, v, cache, 0, inv_freq)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    stream()
+    dt = min(stream() for _ in range(3))
+    assert cache._seen_host[0] == 4096 and not bool(cache.mask[0].any())
+    return dict(value=4096 / dt, unit="tokens/s", seconds=dt, dtype="f32",
+                sample="config 1 in full on the device: 4096 tokens in 16 chunks of 256, float32 (fp32-math kernels, "
+                       "no matrix cores); best of 3 streams")
+
+
+def run_short_strides(cache, dtype, device):
+    """The headline cache (64 sinks + 8 x 8192 slots, full) fed in the short strides the reference's own latency
+    script sweeps (test-latency.bash:14): per stride the time of a call, its stages, and tokens/s."""
+    from cascading_kv_cache_amd import _abi
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
+
+    cfg = LAYER
+    inv_freq = default_inv_freq(cfg["D"], cfg["theta"], device)
+    out = {}
+    for stride in (128, 512):
+        pool = chunk_pool(cfg, 4, dtype, device, q_len=stride, scale=1.0 / math.sqrt(cfg["D"]), seed_offset=200 + stride)
+        n_layers = cfg["layers"]
+        for i in range(4):
+            cascade_attention(*pool[i % 4], cache, i % n_layers, inv_freq)
+        torch.cuda.synchronize()
+        reps = 32
+        t0 = time.perf_counter()
+        for i in range(reps):
+            cascade_attention(*pool[i % 4], cache, i % n_layers, inv_freq)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / reps
+        _abi.profile_enable(1)
+        _abi.profile_read()
+        for i in range(8):
+            cascade_attention(*pool[i % 4], cache, i % n_layers, inv_freq)
+        torch.cuda.synchronize()
+        stages = stage_table(_abi.profile_read(), 8)
+        _abi.profile_enable(0)
+        out[f"stride_{stride}"] = dict(ms_per_call=dt * 1e3, tokens_per_s=cfg["B"] * stride / dt, stage_ms=stages)
+    return out
 
 
 def main():
@@ -606,16 +692,19 @@ def main():
         print(json.dumps({args.only: rec}))
         return
     layer, cache, pool = run_layer(args.steps, args.warmup, dtype, device)
+    sub = args.no_sub or args.only == "layer"
+    short = None if sub else run_short_strides(cache, dtype, device)
     cpu = None if args.no_cpu else run_cpu_baseline(cache, pool, dtype)
     cpu1 = None if args.no_cpu else run_cpu_config1()
     del cache, pool
     torch.cuda.empty_cache()
-    sub = args.no_sub or args.only == "layer"
+    gpu1 = None if sub else run_gpu_config1(device)
     cfg2 = None if sub else run_cfg2(max(args.steps, 20), args.warmup, dtype, device)
     torch.cuda.empty_cache()
     cfg3 = None if sub else run_cfg3(max(args.steps, 20), args.warmup, dtype, device)
     torch.cuda.empty_cache()
     cfg4 = None if (sub or args.no_model) else run_model(MODEL4, device, dtype, args.model_prompt)
+    cfg5 = None if (sub or args.no_model) else run_model(MODEL5, device, dtype, args.model_prompt)
     calibrate()
     cfg = LAYER
     line = {
@@ -637,15 +726,25 @@ def main():
                                "configuration), each = attention + score EMA + cache update; successive calls go round 4 "
                                "such layers, so no call finds its layer's rows in the last-level cache",
                    "tokens_per_step": cfg["B"] * (cfg["Q"] + cfg["decode_per_chunk"])},
+        # `value` is the rate of ONE attention layer (the hot path).  The same metric over the whole 32-layer
+        # decoder, projections and MLP included, is cfg4_full_model below; repeated here so that nobody reads the
+        # layer's figure as the model's.
+        "model_level_tokens_per_s": None if cfg4 is None else {
+            "llama3.1-8b_32_layers_B1_131072+256_tokens": cfg4["tokens_per_s"],
+            "prefill": cfg4["prefill_tokens_per_s"], "decode": cfg4["decode_tokens_per_s"],
+            "qwen2-7b_28_layers_B4_prefill": None if cfg5 is None else cfg5["prefill_tokens_per_s"]},
         "roofline": layer["roofline"],
         "cpu_baseline": cpu,
         "cpu_config1": cpu1,
+        "cfg1_gpu": gpu1,
         "prefill": layer["prefill"],
         "decode": layer["decode"],
         "update": layer["update"],
         "cfg2_prefill": cfg2,
         "cfg3_decode": cfg3,
         "cfg4_full_model": cfg4,
+        "cfg5_full_model": cfg5,
+        "short_stride": short,
     }
     print(json.dumps(line))
 

@@ -225,10 +225,18 @@ template <typename T>
 int run_bwd(const BwdParams& p, hipStream_t stream) {
     const ckv_dense_bwd_args& a = p.a;
     const int64_t rows = a.B * a.H * a.n_ctx;
-    hipLaunchKernelGGL(bwd_delta_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(kThreads), 0, stream, p);
-    CKV_HIP_TRY(hipGetLastError());
     const int pitch = (int)a.D + 1;
     const size_t lds_dq = sizeof(float) * ((size_t)(2 * kTile + 2 * kOwn) * pitch + (size_t)kOwn * (kTile + 1));
+    {
+        // both kernels stage fp32 tiles of D + 1 columns: a device whose workgroups get less LDS than they ask
+        // for is told so before anything is launched
+        const size_t lds_kv_ = sizeof(float) * ((size_t)(2 * kTile + 2 * kOwn) * pitch + (size_t)2 * kOwn * (kTile + 1) + 2 * kTile);
+        DeviceInfo di;
+        if (int rc = current_device_info(&di)) return rc;
+        if (lds_dq > (size_t)di.lds_max || lds_kv_ > (size_t)di.lds_max) return CKV_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(bwd_delta_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(kThreads), 0, stream, p);
+    CKV_HIP_TRY(hipGetLastError());
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(bwd_dq_kernel<T>), (int)lds_dq)) return rc;
     hipLaunchKernelGGL(bwd_dq_kernel<T>, dim3((unsigned)((a.n_ctx + kOwn - 1) / kOwn), (unsigned)(a.B * a.H)), dim3(kThreads),
                        lds_dq, stream, p);
@@ -258,6 +266,7 @@ extern "C" int ckv_attn_dense_bwd(const ckv_dense_bwd_args* args, void* stream_)
     if (a.dtype != CKV_F32 && a.dtype != CKV_F16 && a.dtype != CKV_BF16) return CKV_ERR_DTYPE;
     if (a.B <= 0 || a.H <= 0 || a.n_ctx <= 0 || a.n_kv < a.n_ctx || a.D <= 0) return CKV_ERR_SHAPE;
     if (a.D > kMaxD) return CKV_ERR_UNSUPPORTED;
+    if (a.D % 16 != 0) return CKV_ERR_UNSUPPORTED;  // the kernels deal the head dims out in steps of 16
     if (a.B * a.H > 65535) return CKV_ERR_UNSUPPORTED;
     if (!a.q || !a.k || !a.v || !a.out || !a.lse || !a.dout || !a.dq || !a.dk || !a.dv) return CKV_ERR_NULL;
     if (a.n_kv > a.n_ctx && !a.mask) return CKV_ERR_NULL;

@@ -135,7 +135,14 @@ class CascadeDecoder(nn.Module):
         return self
 
     def new_cache(self, window, cascades, batch=1, num_sink_tokens=64, **kw):
-        return CascadingKVCache(window // cascades, num_sink_tokens=num_sink_tokens, max_batch_size=batch,
+        """One cache layer per decoder layer: ``window`` slots split into ``cascades`` rings.  Both may be lists
+        with one entry per layer (the reference builds such caches, cascade/models/test.py:325-377)."""
+        if isinstance(window, (list, tuple)):
+            per_ring = [w // c for w, c in zip(window, cascades)]
+            window = list(window)
+        else:
+            per_ring = window // cascades
+        return CascadingKVCache(per_ring, num_sink_tokens=num_sink_tokens, max_batch_size=batch,
                                 heads=self.cfg.num_kv_heads, dim=self.cfg.head_dim, max_seq_len=window,
                                 dtype=self.dtype, device=self.device, head_reduction=self.cfg.head_reduction,
                                 layers=self.cfg.num_layers, verbose=False, **kw)

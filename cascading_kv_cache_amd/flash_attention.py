@@ -20,6 +20,9 @@ from . import _abi
 from .cascading_cache import _require_device, workspace
 
 
+MAX_BACKWARD_HEAD_DIM = 192   # ckv_attn_dense_bwd stages fp32 tiles of head_dim + 1 columns in LDS
+
+
 def _forward(q, k, v, causal, sm_scale, mask, beta, want_lse):
     _require_device(q, "q")
     # the reference's shape checks (flash_attention.py:545-551)
@@ -100,6 +103,9 @@ class _attention(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, causal, sm_scale, mask, beta):
         needs_grad = any(t.requires_grad for t in (q, k, v))
+        if needs_grad and q.shape[-1] > MAX_BACKWARD_HEAD_DIM:
+            raise _abi.CkvError(f"gradients are implemented for head_dim <= {MAX_BACKWARD_HEAD_DIM}, got {q.shape[-1]} "
+                                "(the forward pass alone takes it: call without requires_grad inputs)")
         o, scores, lse, mask = _forward(q, k, v, causal, sm_scale, mask, beta, needs_grad)
         if needs_grad:
             ctx.save_for_backward(q, k, v, o, lse, mask if mask is not None else torch.empty(0, dtype=torch.bool,

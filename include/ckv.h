@@ -131,7 +131,9 @@ int ckv_update(const ckv_update_args* args, void* stream);
  * process ends), so the call allocates nothing and needs no workspace from the caller.  Sizes whose
  * ckv_update_workspace_bytes(...) exceeds that array are refused with CKV_ERR_TOO_LARGE.  All calls on
  * one device share the array: calls that overlap in time on one device (different streams, or different
- * host threads) race on it; calls on one stream are ordered and safe. */
+ * host threads) race on it; calls on one stream are ordered and safe.  The first call on a device looks the
+ * array's address and the device's limits up (runtime queries that must not be recorded): a caller that captures
+ * the call into a HIP graph makes one ordinary call on that device first. */
 int64_t ckv_update_static_scratch_bytes(void);
 int ckv_update_static(const ckv_update_args* args, void* stream);
 
@@ -188,10 +190,15 @@ typedef struct ckv_attn_args {
     int32_t head_reduction;        /* ckv_head_reduction                                  */
     int32_t homogeneous_heads;     /* reduce over all H heads (cascade_attention.py:240-242) */
     int32_t dtype;                 /* ckv_dtype of every floating tensor above            */
-    int32_t filled_slots;          /* optional bound: cache slots at or past this index are hidden whatever `mask`
-                                      says (the cache fills from slot 0 up, cascading_cache.py:381-726, so the
-                                      tokens stored so far bound it); 0 = no bound, every slot is looked at.  Lets
-                                      the single-token kernels skip the empty part of a cache that is still filling. */
+    int32_t filled_slots;          /* optional hint, never a second mask: the caller promises that every cache slot
+                                      at or past this index is masked in `mask` (the cache fills from slot 0 up,
+                                      cascading_cache.py:381-726, so the tokens stored so far bound it); 0 = no
+                                      promise.  Kernels may then skip such slots without reading `mask` (the 16-bit
+                                      single-token kernels skip whole 128-key tiles of a cache that is still
+                                      filling) or ignore the hint altogether; visibility is decided by `mask` alone,
+                                      so with a hint that keeps its promise the results do not depend on it, and a
+                                      hint that contradicts `mask` gives unspecified results for the slots it
+                                      covers. */
 
     void* workspace;
     int64_t workspace_bytes;
@@ -241,7 +248,9 @@ int ckv_attn_dense(const ckv_dense_args* args, void* stream);
  * Backward of ckv_attn_dense: replaces _attention.backward -> _attn_bwd_preprocess / _attn_bwd
  * (flash_attention.py:279-537, 654-710).  Given the forward's inputs, its output and row normalisers and the
  * gradient of the output, writes dq, dk, dv (dtype and shapes of q, k, v); the scores carry no gradient, as
- * in the reference.  Masked cached keys receive zero gradients.  head_dim up to 192.
+ * in the reference.  Masked cached keys receive zero gradients.  head_dim: a multiple of 16, up to 192 (anything
+ * else, or a device whose workgroups get less LDS than the fp32 tiles of head_dim + 1 columns need, is refused with
+ * CKV_ERR_UNSUPPORTED before anything is launched).
  * ---------------------------------------------------------------------------------------- */
 typedef struct ckv_dense_bwd_args {
     const void* q;                 /* (B, H, n_ctx, D) */

@@ -384,6 +384,7 @@ def test_attention_rejects_cpu_tensors():
     (1, 2, 128, 128, 64), (1, 2, 256, 256, 64), (1, 2, 512, 512, 64), (1, 1, 128, 128 + 128, 64),
     (1, 2, 1024, 16384 + 1024, 64), (2, 32, 1024, 16384 + 1024, 128), (1, 2, 512, 2560, 64),
     (1, 2, 500, 2048 + 500, 64), (1, 2, 500, 2048 + 64 + 500, 64), (2, 3, 77, 300 + 77, 32),
+    (1, 3, 90, 200 + 90, 16),   # the smallest head size the operator takes
 ])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 def test_dense_operator_backward(Z, H, N_CTX, N_KV, HEAD_DIM, dtype):
@@ -496,3 +497,26 @@ def test_reference_mixin_surface(flavour):
         assert same.float().mean().item() >= 0.99, f"chunk {c}: {(~same).sum().item()} slots hold another token"
         sh, sf = by_hand.score_cache[0].float(), fused.score_cache[0].float()
         assert_scores_close(torch.where(same, sh, sf), sf, dtype, f"chunk {c}: score cache")
+
+
+def test_backward_is_refused_up_front_for_head_sizes_it_does_not_tile():
+    """head_dim 256 runs forward (the reference operator's set is 16 .. 256) but the backward kernels stage fp32
+    rows of at most 192 columns: asking for gradients raises at the call, not later inside ``.backward()``; head
+    sizes that are not a multiple of 16 never reach the operator (flash_attention.py:545-551), and the C entry point
+    refuses them too."""
+    import ctypes as C
+
+    from cascading_kv_cache_amd import _abi
+    from cascading_kv_cache_amd.flash_attention import attention
+
+    q = torch.randn(1, 1, 32, 256, device="cuda", dtype=torch.float16)
+    k = torch.randn(1, 1, 48, 256, device="cuda", dtype=torch.float16)
+    mask = torch.zeros(16, dtype=torch.bool, device="cuda")
+    out, _ = attention(q, k, k.clone(), True, 0.1, mask, 1.0)          # inference: fine
+    assert out.shape == q.shape and bool(torch.isfinite(out.float()).all())
+    with pytest.raises(_abi.CkvError):
+        attention(q.clone().requires_grad_(), k, k.clone(), True, 0.1, mask, 1.0)
+    g = _abi.DenseBwdArgs()
+    g.dtype = _abi.CKV_F16
+    g.B, g.H, g.n_ctx, g.n_kv, g.D = 1, 1, 16, 32, 80
+    assert _abi.lib().ckv_attn_dense_bwd(C.byref(g), None) == -6       # CKV_ERR_UNSUPPORTED

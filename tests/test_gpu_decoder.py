@@ -57,9 +57,13 @@ def test_small_decoder_prefill_and_greedy_steps_against_the_oracle(dtype):
             assert torch.equal(getattr(cache, name)[i].cpu(), getattr(oc, name)), f"layer {i}: {name}"
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_decoder_layers_past_the_window_teacher_forced(dtype):
-    """The multi-layer path once the cascades evict: a stream of more than twice the window goes through a
+@pytest.mark.parametrize("dtype,layer_sizes", [(torch.bfloat16, None), (torch.float16, None),
+                                               (torch.bfloat16, [(32, 4), (16, 2)]), (torch.float16, [(8, 8), (64, 1)])])
+def test_decoder_layers_past_the_window_teacher_forced(dtype, layer_sizes):
+    """``layer_sizes``: (slots per ring, rings) of every layer when the layers differ in size, as the caches of
+    cascade/models/test.py:325-377 do (per-layer ``window_length`` / ``max_seq_len`` lists).
+
+    The multi-layer path once the cascades evict: a stream of more than twice the window goes through a
     two-layer decoder in strides and then token by token.  Every layer's cache layer restarts each step from
     that layer's oracle state and the oracle's attention gets the device's own q/k/v, so a tie-level decision
     cannot snowball; per layer and step the attention output, both score inputs, the metadata, the update
@@ -69,14 +73,20 @@ def test_decoder_layers_past_the_window_teacher_forced(dtype):
 
     cfg = PRESETS["tiny"]
     model = CascadeDecoder(cfg, dtype=dtype, device="cuda:0", seed=7)
-    B, NS, W, C = 2, 4, 32, 4
-    cache = model.new_cache(W * C, C, batch=B, num_sink_tokens=NS)
-    caches = [OracleCache(window_length=W, num_sink_tokens=NS, max_batch_size=B, heads=cfg.num_kv_heads,
-                          dim=cfg.head_dim, max_seq_len=W * C, dtype=dtype) for _ in range(cfg.num_layers)]
+    B, NS = 2, 4
+    sizes = layer_sizes or [(32, 4)] * cfg.num_layers
+    if layer_sizes:
+        cache = model.new_cache([w * c for w, c in sizes], [c for _, c in sizes], batch=B, num_sink_tokens=NS)
+        assert cache.window_length == [w for w, _ in sizes] and cache.cascades == [c for _, c in sizes]
+        assert [t.size(2) for t in cache.key_cache] == [w * c for w, c in sizes]
+    else:
+        cache = model.new_cache(32 * 4, 4, batch=B, num_sink_tokens=NS)
+    caches = [OracleCache(window_length=w, num_sink_tokens=NS, max_batch_size=B, heads=cfg.num_kv_heads,
+                          dim=cfg.head_dim, max_seq_len=w * c, dtype=dtype) for w, c in sizes]
     oracles = [OracleCascadeAttention(cfg.num_heads, cfg.num_kv_heads, cfg.head_dim, rope_theta=cfg.rope_theta,
                                       head_reduction=cfg.head_reduction) for _ in range(cfg.num_layers)]
     inv_freq = default_inv_freq(cfg.head_dim, cfg.rope_theta, "cuda:0")
-    steps = [48] * 6 + [1] * 14          # 302 tokens through a 4 + 128-slot cache
+    steps = [48] * 6 + [1] * 14          # 302 tokens through caches of 4 sinks + at most 128 slots
     ids = torch.randint(0, cfg.vocab_size, (B, sum(steps)), generator=torch.Generator().manual_seed(8)).cuda()
     ledger = FlipLedger(dtype)
     done = 0
@@ -109,13 +119,14 @@ def test_decoder_layers_past_the_window_teacher_forced(dtype):
                 check_update_against_replay(cache, replay, kc, vc, scores_g, new_g.cpu(), layer=li, ctx=ctx)
                 og_g = cache.og_pos[li].cpu()
                 margins = flip_margins(og_g, oc, pre, seen_before, attn_o.last_score_cache, new_c)
-                ledger.record(margins, eps, og_g.numel(), primary_only=qn < 2 * W, ctx=ctx)
+                ledger.record(margins, eps, og_g.numel(), primary_only=qn < 2 * sizes[li][0], ctx=ctx)
                 x = x + layer.self_attn.o_proj(out_g.transpose(1, 2).reshape(B, qn, -1))
                 x = x + layer.mlp(layer.post_attention_layernorm(x))
             done += qn
     print(ledger.summary())
     assert cache.seen_tokens_by_layer.cpu().tolist() == [done] * cfg.num_layers
-    assert not bool(caches[0].mask.any()) and int(caches[0].start_indices.sum()) > 0, "the cascades must have evicted"
+    for oc in caches:
+        assert not bool(oc.mask.any()) and int(oc.start_indices.sum()) > 0, "the cascades must have evicted"
     assert ledger.flips <= flip_bound(ledger), ledger.summary()
 
 

@@ -85,3 +85,64 @@ def test_static_scratch_update_refuses_sizes_beyond_its_array():
     torch.cuda.synchronize()
     for n in STATE:
         assert torch.equal(getattr(cache, n)[0], before[n]), f"{n} was touched by a refused call"
+
+
+def test_static_scratch_update_recorded_into_a_graph():
+    """The callers the entry point is for include code under HIP graph capture: after one ordinary call on the
+    device (which looks the array's address and the device's limits up), the call is recorded, and every replay —
+    with eager work and synchronisations of the program in between, fresh inputs copied into the recorded buffers —
+    leaves the state bit-identical to ckv_update on a second cache."""
+    from cascading_kv_cache_amd import _abi
+
+    lib = _abi.lib()
+    dtype = torch.bfloat16
+    B, KVH, D, NS, W, Cn, q = 2, 2, 128, 4, 32, 4, 24
+    ref, sta = make_cache(B, KVH, D, NS, W, Cn, dtype), make_cache(B, KVH, D, NS, W, Cn, dtype)
+    gen = torch.Generator().manual_seed(29)
+    k = torch.zeros(B, KVH, q, D, dtype=dtype, device="cuda:0")
+    v, s = torch.zeros_like(k), torch.zeros(B, KVH, q, dtype=dtype, device="cuda:0")
+    a, b = describe(ref, k, v, s), describe(sta, k, v, s)
+    need = lib.ckv_update_workspace_bytes(a.N, a.H, a.K, a.max_seq_len, a.cascades)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda:0")
+    a.workspace, a.workspace_bytes = ws.data_ptr(), need
+
+    def fresh_inputs():
+        k.copy_(torch.randn(B, KVH, q, D, generator=gen).to(dtype))
+        v.copy_(torch.randn(B, KVH, q, D, generator=gen).to(dtype))
+        s.copy_((torch.randint(0, 6, (B, KVH, q), generator=gen).float() / 8).to(dtype))
+
+    def advance():
+        for c in (ref, sta):
+            c.seen_tokens_by_layer[0] += q
+            c._seen_host[0] += q
+
+    def same(what):
+        torch.cuda.synchronize()
+        for name in STATE:
+            g, w = getattr(sta, name)[0], getattr(ref, name)[0]
+            if g.dtype.is_floating_point:
+                g, w = g.view(torch.int16), w.view(torch.int16)
+            assert torch.equal(g, w), f"{what}: {name}"
+
+    # the ordinary call that must come first on a device
+    fresh_inputs()
+    stream = torch.cuda.current_stream().cuda_stream
+    _abi.check(lib.ckv_update(C.byref(a), C.c_void_p(stream)), "ckv_update")
+    _abi.check(lib.ckv_update_static(C.byref(b), C.c_void_p(stream)), "ckv_update_static")
+    advance()
+    same("eager call")
+    assert _abi.profile_enable(0) == 0     # stage timing records events: off while a call is recorded
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _abi.check(lib.ckv_update_static(C.byref(b), C.c_void_p(torch.cuda.current_stream().cuda_stream)),
+                   "ckv_update_static under capture")
+    scratch = torch.zeros(1 << 14, device="cuda:0")
+    for rep in range(8):                   # 8 x 24 tokens: the 4 + 128-slot cache fills and evicts
+        fresh_inputs()
+        _abi.check(lib.ckv_update(C.byref(a), C.c_void_p(torch.cuda.current_stream().cuda_stream)), "ckv_update")
+        graph.replay()
+        advance()
+        scratch.add_(1.0).mul_(0.5)        # the program's own eager work between two replays
+        same(f"replay {rep}")
+    assert not bool(ref.mask[0].any()) and int(ref.start_indices[0].sum()) > 0
