@@ -803,7 +803,6 @@ constexpr int kOneMinUnits = 32;
 __global__ void __launch_bounds__(kOneThreads) ckv_update_one_kernel(UpdateParams p) {
     __shared__ int sh_chain[kOneWaves];
     __shared__ int sh_n, sh_pos;
-    __shared__ int sh_stored[kOneWaves], sh_start[kOneWaves];
     __shared__ int sh_write[kOneWaves];                     // position ids of the cascade are written
     __shared__ unsigned sh_seg[kOneWaves], sh_add[kOneWaves];
     __shared__ long long sh_base[kOneWaves];
@@ -878,9 +877,23 @@ __global__ void __launch_bounds__(kOneThreads) ckv_update_one_kernel(UpdateParam
                 break;
             }
         }
-        if (lane < C) {
-            sh_stored[lane] = st_new;
-            sh_start[lane] = sx_new;
+        // ---- parameters of the position ids (cascading_cache.py:728-774, 129-142) from the trackers after the
+        //      call, which lane i holds for cascade i: the same closed form as the position blocks of the apply
+        //      kernel.  Cascade i is written while every earlier cascade holds tokens and ids are left for it.
+        {
+            long long tot = lane < C ? (long long)st_new : 0;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) tot += __shfl_xor(tot, off);
+            const unsigned long long empty = __builtin_amdgcn_ballot_w64(lane < C && st_new <= 0);
+            const int first_empty = empty ? __builtin_ctzll(empty) : C;
+            if (lane < C) {
+                const long long ub = tot - (long long)lane * W;   // ids still to hand out when cascade `lane` is reached
+                const unsigned seg = (unsigned)((long long)st_new < W ? st_new : (int32_t)W);
+                sh_write[lane] = (lane <= first_empty && (lane == 0 || ub > 0) && seg != 0) ? 1 : 0;
+                sh_seg[lane] = seg;
+                sh_add[lane] = seg - (unsigned)sx_new;  // start < seg or start == 0
+                sh_base[lane] = ub - (long long)seg;
+            }
         }
         if (lane == 0) {
             sh_n = n_chain;
@@ -890,27 +903,6 @@ __global__ void __launch_bounds__(kOneThreads) ckv_update_one_kernel(UpdateParam
     __syncthreads();
     const int n_chain = sh_n;
     const bool do_pos = sh_pos != 0;
-
-    // ---- position ids (cascading_cache.py:728-774, 129-142): per cascade the same closed form as the position
-    //      blocks of the apply kernel, from the trackers after the call
-    if (do_pos && tid < C) {
-        const int i = tid;
-        long long ub = 0;
-        for (int c = 0; c < C; c++) ub += sh_stored[c];
-        bool wr = true;
-        for (int c = 0; c < i; c++) {
-            if (sh_stored[c] <= 0) wr = false;
-            ub -= W;
-            if (ub <= 0) wr = false;
-        }
-        const long long stv = sh_stored[i];
-        const unsigned seg = (unsigned)(stv < W ? stv : W);
-        if (seg == 0) wr = false;
-        sh_write[i] = wr ? 1 : 0;
-        sh_seg[i] = seg;
-        sh_add[i] = seg - (unsigned)sh_start[i];  // start < seg or start == 0
-        sh_base[i] = ub - (long long)seg;
-    }
 
     // ---- rows: wavefront j takes the row that ends in chain[j] (the token, or the old content of chain[j - 1])
     const int chunks = (int)(A.HID * es / 16);
@@ -949,7 +941,31 @@ __global__ void __launch_bounds__(kOneThreads) ckv_update_one_kernel(UpdateParam
             }
         }
     }
-    __syncthreads();  // every displaced row is in registers, the position parameters are in LDS
+    // ---- position ids: they need the plan alone, so their stores go out while the displaced rows are on their way
+    if (do_pos) {
+        int64_t* pos = A.pos + n * A.pos_stride[0] + h * A.pos_stride[1];
+        auto id_of = [&](int i, unsigned j) -> int64_t {
+            const unsigned seg = sh_seg[i];
+            unsigned x = j + sh_add[i];
+            if (x >= seg) x -= seg;
+            if (x >= seg) x %= seg;  // slots past the stored tokens of a cascade that is not full
+            return (int64_t)x + sh_base[i];
+        };
+        if (A.pos_stride[2] == 1 && (reinterpret_cast<uintptr_t>(pos) & 15u) == 0 && (W & 1) == 0) {
+            for (int i = 0; i < C; i++) {
+                if (!sh_write[i]) continue;
+                int64_t* pc = pos + (int64_t)i * W;
+                for (int64_t j = 2 * (int64_t)tid; j < W; j += 2 * kOneThreads)
+                    *reinterpret_cast<longlong2*>(pc + j) = make_longlong2(id_of(i, (unsigned)j), id_of(i, (unsigned)j + 1));
+            }
+        } else {
+            for (int i = 0; i < C; i++) {
+                if (!sh_write[i]) continue;
+                for (int64_t j = tid; j < W; j += kOneThreads) pos[((int64_t)i * W + j) * A.pos_stride[2]] = id_of(i, (unsigned)j);
+            }
+        }
+    }
+    __syncthreads();  // every displaced row is in registers
     if (mover) {
         const int d = sh_chain[wave];
         if (d >= S) {  // sink slot (cascading_cache.py:61-109); only the token itself gets here
@@ -975,28 +991,6 @@ __global__ void __launch_bounds__(kOneThreads) ckv_update_one_kernel(UpdateParam
                 og[(int64_t)d * A.og_pos_stride[2]] = r_og;
                 (A.mask + n * A.mask_stride[0] + h * A.mask_stride[1])[(int64_t)d * A.mask_stride[2]] = 0;
             }
-        }
-    }
-    if (!do_pos) return;
-    int64_t* pos = A.pos + n * A.pos_stride[0] + h * A.pos_stride[1];
-    auto id_of = [&](int i, unsigned j) -> int64_t {
-        const unsigned seg = sh_seg[i];
-        unsigned x = j + sh_add[i];
-        if (x >= seg) x -= seg;
-        if (x >= seg) x %= seg;  // slots past the stored tokens of a cascade that is not full
-        return (int64_t)x + sh_base[i];
-    };
-    if (A.pos_stride[2] == 1 && (reinterpret_cast<uintptr_t>(pos) & 15u) == 0 && (W & 1) == 0) {
-        for (int i = 0; i < C; i++) {
-            if (!sh_write[i]) continue;
-            int64_t* pc = pos + (int64_t)i * W;
-            for (int64_t j = 2 * (int64_t)tid; j < W; j += 2 * kOneThreads)
-                *reinterpret_cast<longlong2*>(pc + j) = make_longlong2(id_of(i, (unsigned)j), id_of(i, (unsigned)j + 1));
-        }
-    } else {
-        for (int i = 0; i < C; i++) {
-            if (!sh_write[i]) continue;
-            for (int64_t j = tid; j < W; j += kOneThreads) pos[((int64_t)i * W + j) * A.pos_stride[2]] = id_of(i, (unsigned)j);
         }
     }
 }

@@ -25,10 +25,7 @@ MAX_BACKWARD_HEAD_DIM = 192   # ckv_attn_dense_bwd stages fp32 tiles of head_dim
 
 def _forward(q, k, v, causal, sm_scale, mask, beta, want_lse):
     _require_device(q, "q")
-    # the reference's shape checks (flash_attention.py:545-551)
-    HEAD_DIM_Q, HEAD_DIM_K, HEAD_DIM_V = q.shape[-1], k.shape[-1], v.shape[-1]
-    assert HEAD_DIM_Q == HEAD_DIM_K and HEAD_DIM_K == HEAD_DIM_V
-    assert HEAD_DIM_K in {16, 32, 64, 128, 256}
+    assert q.shape[-1] == k.shape[-1] == v.shape[-1]
     assert k.size(2) == v.size(2)
     assert _abi.same_layout(k, v)
     B, H, n_ctx, D = q.shape
@@ -102,6 +99,9 @@ class _attention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, causal, sm_scale, mask, beta):
+        # the reference operator's head sizes (flash_attention.py:545-551); the library itself takes any even
+        # head size up to 256 forward and any multiple of 16 up to 192 backward
+        assert q.shape[-1] in {16, 32, 64, 128, 256}
         needs_grad = any(t.requires_grad for t in (q, k, v))
         if needs_grad and q.shape[-1] > MAX_BACKWARD_HEAD_DIM:
             raise _abi.CkvError(f"gradients are implemented for head_dim <= {MAX_BACKWARD_HEAD_DIM}, got {q.shape[-1]} "

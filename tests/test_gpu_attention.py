@@ -518,5 +518,36 @@ def test_backward_is_refused_up_front_for_head_sizes_it_does_not_tile():
         attention(q.clone().requires_grad_(), k, k.clone(), True, 0.1, mask, 1.0)
     g = _abi.DenseBwdArgs()
     g.dtype = _abi.CKV_F16
-    g.B, g.H, g.n_ctx, g.n_kv, g.D = 1, 1, 16, 32, 80
+    g.B, g.H, g.n_ctx, g.n_kv, g.D = 1, 1, 16, 32, 72
     assert _abi.lib().ckv_attn_dense_bwd(C.byref(g), None) == -6       # CKV_ERR_UNSUPPORTED
+
+
+@pytest.mark.parametrize("D,dtype", [(80, torch.float16), (192, torch.bfloat16), (192, torch.float32), (48, torch.float32)])
+def test_backward_head_sizes_outside_the_reference_set(D, dtype):
+    """The C entry points take head sizes the reference operator does not (any multiple of 16 up to 192 backward):
+    forward and backward of the dense operator, called below the operator's own shape check, against autograd
+    through the dense formula."""
+    from cascading_kv_cache_amd import flash_attention as fa
+
+    torch.manual_seed(21)
+    Z, H, N_CTX, N_KV = 1, 2, 70, 150 + 70
+    q = torch.empty((Z, H, N_CTX, D), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
+    k = torch.empty((Z, H, N_KV, D), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
+    v = torch.empty((Z, H, N_KV, D), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
+    mask = torch.rand(N_KV - N_CTX, device="cuda") > 0.5
+    full = torch.cat((mask[None, :].expand(N_CTX, -1),
+                      torch.ones(N_CTX, N_CTX, dtype=torch.bool, device="cuda").triu(1)), dim=-1)
+    sm_scale = 1.0 / math.sqrt(D)
+    dout = torch.randn_like(q)
+    p = (torch.matmul(q, k.transpose(2, 3)) * sm_scale).masked_fill(full, float("-inf"))
+    ref_out = torch.matmul(torch.softmax(p.float(), dim=-1).to(dtype), v)
+    ref_out.backward(dout)
+    with torch.no_grad():
+        out, _, lse, m = fa._forward(q, k, v, True, sm_scale, mask, 1.0, True)
+        dq, dk, dv = fa._backward(q, k, v, out, lse, m, dout, sm_scale)
+    atol = {torch.float32: 1e-4, torch.float16: 1e-2, torch.bfloat16: 2e-2}[dtype]
+    assert (out.float() - ref_out.float()).abs().max().item() <= atol
+    for name, got, want in (("dv", dv, v.grad), ("dk", dk, k.grad), ("dq", dq, q.grad)):
+        rtol = 2.0 ** -6 if dtype == torch.bfloat16 else 0.0
+        excess = ((got.float() - want.float()).abs() - rtol * want.float().abs()).max().item()
+        assert excess <= atol, f"{name}: error exceeds the allowance by {excess:.3e}"
