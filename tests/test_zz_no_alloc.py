@@ -138,11 +138,11 @@ def test_static_scratch_update_recorded_into_a_graph():
         _abi.check(lib.ckv_update_static(C.byref(b), C.c_void_p(torch.cuda.current_stream().cuda_stream)),
                    "ckv_update_static under capture")
     scratch = torch.zeros(1 << 14, device="cuda:0")
-    for rep in range(8):                   # 8 x 24 tokens: the 4 + 128-slot cache fills and evicts
+    for rep in range(8):                   # 8 x 24 tokens: the first ring of the 4 + 4 x 32-slot cache fills and evicts
         fresh_inputs()
         _abi.check(lib.ckv_update(C.byref(a), C.c_void_p(torch.cuda.current_stream().cuda_stream)), "ckv_update")
         graph.replay()
         advance()
         scratch.add_(1.0).mul_(0.5)        # the program's own eager work between two replays
         same(f"replay {rep}")
-    assert not bool(ref.mask[0].any()) and int(ref.start_indices[0].sum()) > 0
+    assert int(ref.start_indices[0].sum()) > 0 and int((~ref.mask[0]).sum()) > 32 * B * KVH
