@@ -400,27 +400,13 @@ struct Mma16<__half> {
     }
 };
 
-// rope_ref on packed words: w1 holds elements (j, j+1) of a key row, w2 their partners (j+64, j+65); c0/s0 and
-// c1/s1 are the rounded cos/sin of the two pairs.  Products of two 16-bit values and sums of two 16-bit values are
-// exact in fp32, so each packed conversion below is one of the reference's roundings.
+// cos / sin of the two rotation pairs a word covers, at the given angles
 template <typename T>
-__device__ inline void rope_ref_words(uint32_t w1, uint32_t w2, float c0, float s0, float c1, float s1, float post,
-                                      uint32_t& o1, uint32_t& o2) {
-    const float a0 = Mma16<T>::lo(w1), a1 = Mma16<T>::hi(w1), b0 = Mma16<T>::lo(w2), b1 = Mma16<T>::hi(w2);
-    const uint32_t p0 = Mma16<T>::pack2(a0 * c0, b0 * s0), q0 = Mma16<T>::pack2(b0 * c0, a0 * s0);
-    const uint32_t p1 = Mma16<T>::pack2(a1 * c1, b1 * s1), q1 = Mma16<T>::pack2(b1 * c1, a1 * s1);
-    o1 = Mma16<T>::pack2(Mma16<T>::lo(p0) - Mma16<T>::hi(p0), Mma16<T>::lo(p1) - Mma16<T>::hi(p1));
-    o2 = Mma16<T>::pack2(Mma16<T>::lo(q0) + Mma16<T>::hi(q0), Mma16<T>::lo(q1) + Mma16<T>::hi(q1));
-    o1 = Mma16<T>::pack2(Mma16<T>::lo(o1) * post, Mma16<T>::hi(o1) * post);
-    o2 = Mma16<T>::pack2(Mma16<T>::lo(o2) * post, Mma16<T>::hi(o2) * post);
-}
-// cos / sin of an angle, rounded to the tensor dtype as the reference's rotary module hands them out
-template <typename T>
-__device__ inline void sincos_ref(float angle, float* sn, float* cs) {
-    float s_, c_;
-    fast_sincos(angle, &s_, &c_);
-    *sn = Mma16<T>::lo(Mma16<T>::pack2(s_, 0.f));
-    *cs = Mma16<T>::lo(Mma16<T>::pack2(c_, 0.f));
+__device__ inline RopeWord<T> rope_word_at(float angle0, float angle1) {
+    float s0, c0, s1, c1;
+    fast_sincos(angle0, &s0, &c0);
+    fast_sincos(angle1, &s1, &c1);
+    return RopeWord<T>::make(c0, s0, c1, s1);
 }
 
 template <typename T, int G>
@@ -446,7 +432,7 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
     int64_t koff1[2];
     int seg1[2];
     bool vis1[2];
-    float cs[2][2][8], sn[2][2][8];
+    RopeWord<T> rw[2][2][4];  // [key of this lane][ks][word]
 #pragma unroll
     for (int gi = 0; gi < 2; gi++) {
         const int64_t n = n_wave + 16 * gi + key16;
@@ -469,10 +455,11 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
 #pragma unroll
             for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const int f = 32 * ks + 8 * kq + e;
-                    const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                    sincos_ref<T>(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
+                for (int w = 0; w < 4; w++) {
+                    const int f = 32 * ks + 8 * kq + 2 * w;
+                    const float f0 = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
+                    const float f1 = a.inv_freq ? a.inv_freq[f + 1] : 1.0f / powf(a.rope_theta, (float)(2 * f + 2) / (float)kD);
+                    rw[gi][ks][w] = rope_word_at<T>(__fmul_rn((float)pos, f0), __fmul_rn((float)pos, f1));
                 }
         }
     }
@@ -537,10 +524,11 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const int f = 32 * ks + 8 * kq + e;
-                        const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                        sincos_ref<T>(__fmul_rn((float)pos, fr), &sn[gi][ks][e], &cs[gi][ks][e]);
+                    for (int w = 0; w < 4; w++) {
+                        const int f = 32 * ks + 8 * kq + 2 * w;
+                        const float f0 = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
+                        const float f1 = a.inv_freq ? a.inv_freq[f + 1] : 1.0f / powf(a.rope_theta, (float)(2 * f + 2) / (float)kD);
+                        rw[gi][ks][w] = rope_word_at<T>(__fmul_rn((float)pos, f0), __fmul_rn((float)pos, f1));
                     }
             }
             uint4 kop[4];
@@ -551,7 +539,7 @@ __global__ void __launch_bounds__(256, 2) decode_main_mfma_kernel(DecodeParams p
                 uint32_t o1[4], o2[4];
 #pragma unroll
                 for (int w = 0; w < 4; w++) {
-                    rope_ref_words<T>(w1[w], w2[w], cs[gi][ks][2 * w], sn[gi][ks][2 * w], cs[gi][ks][2 * w + 1], sn[gi][ks][2 * w + 1], p.key_scale, o1[w], o2[w]);
+                    rw[gi][ks][w].rotate(w1[w], w2[w], p.key_scale, true, o1[w], o2[w]);
                 }
                 kop[ks] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
                 kop[ks + 2] = make_uint4(o2[0], o2[1], o2[2], o2[3]);
@@ -760,7 +748,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
 
         // ---- per-tile constants (the same for every (b, kvh): positions are shared)
         bool vis1 = false;
-        float cs[2][8], sn[2][8];
+        RopeWord<T> rw[2][4];  // [ks][word]: dims 32 ks + 8 kq + 2 w, + 1 and their partners 64 further
         {
             const int64_t n = n_wave + key16;
             int64_t pos = 0;
@@ -770,10 +758,11 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
 #pragma unroll
             for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const int f = 32 * ks + 8 * kq + e;
-                    const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                    sincos_ref<T>(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
+                for (int w = 0; w < 4; w++) {
+                    const int f = 32 * ks + 8 * kq + 2 * w;
+                    const float f0 = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
+                    const float f1 = a.inv_freq ? a.inv_freq[f + 1] : 1.0f / powf(a.rope_theta, (float)(2 * f + 2) / (float)kD);
+                    rw[ks][w] = rope_word_at<T>(__fmul_rn((float)pos, f0), __fmul_rn((float)pos, f1));
                 }
         }
         // Rows of hidden slots may hold anything (their probability is zero, but 0 * NaN is not), so
@@ -949,7 +938,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                     uint32_t o1[4], o2[4];
 #pragma unroll
                     for (int w = 0; w < 4; w++) {
-                        rope_ref_words<T>(w1[w], w2[w], cs[ks][2 * w], sn[ks][2 * w], cs[ks][2 * w + 1], sn[ks][2 * w + 1], p.key_scale, o1[w], o2[w]);
+                        rw[ks][w].rotate(w1[w], w2[w], p.key_scale, true, o1[w], o2[w]);
                     }
                     kop[ks] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
                     kop[ks + 2] = make_uint4(o2[0], o2[1], o2[2], o2[3]);
@@ -1134,7 +1123,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
 
         // ---- per-tile constants (the same for every (b, kvh): positions are shared)
         bool vis1 = false;
-        float cs[2][8], sn[2][8];
+        RopeWord<T> rw[2][4];  // [ks][word]: dims 32 ks + 8 kq + 2 w, + 1 and their partners 64 further
         {
             const int64_t n = n_wave + key16;
             int64_t pos = 0;
@@ -1144,10 +1133,11 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
 #pragma unroll
             for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const int f = 32 * ks + 8 * kq + e;
-                    const float fr = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
-                    sincos_ref<T>(__fmul_rn((float)pos, fr), &sn[ks][e], &cs[ks][e]);
+                for (int w = 0; w < 4; w++) {
+                    const int f = 32 * ks + 8 * kq + 2 * w;
+                    const float f0 = a.inv_freq ? a.inv_freq[f] : 1.0f / powf(a.rope_theta, (float)(2 * f) / (float)kD);
+                    const float f1 = a.inv_freq ? a.inv_freq[f + 1] : 1.0f / powf(a.rope_theta, (float)(2 * f + 2) / (float)kD);
+                    rw[ks][w] = rope_word_at<T>(__fmul_rn((float)pos, f0), __fmul_rn((float)pos, f1));
                 }
         }
         // rows of hidden slots are zeroed on the way into the P.V product (0 * NaN): masks of this lane's
@@ -1287,7 +1277,7 @@ __global__ void __launch_bounds__(kStreamThreads, kStreamWgPerCu) decode_stream_
                     uint32_t o1[4], o2[4];
 #pragma unroll
                     for (int w = 0; w < 4; w++) {
-                        rope_ref_words<T>(w1[w], w2[w], cs[ks][2 * w], sn[ks][2 * w], cs[ks][2 * w + 1], sn[ks][2 * w + 1], p.key_scale, o1[w], o2[w]);
+                        rw[ks][w].rotate(w1[w], w2[w], p.key_scale, true, o1[w], o2[w]);
                     }
                     kop[ks] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
                     kop[ks + 2] = make_uint4(o2[0], o2[1], o2[2], o2[3]);

@@ -89,26 +89,6 @@ __host__ __device__ inline int vt_slot(int k) {
 // ---------------------------------------------------------------------------------------------
 // staging
 // ---------------------------------------------------------------------------------------------
-// Rotary embedding of two neighbouring pairs (x1a, x2a), (x1b, x2b) (elements j, j+64 and j+1, j+65 of a row)
-// with the roundings of the eager path, which evaluates x*cos + rotate_half(x)*sin in the tensor dtype
-// (cascade_attention.py:31-35): cos and sin arrive rounded to the dtype (modeling_llama.py:219-220), each
-// product is rounded, then the sum, and then the product with sqrt(softmax scale) that the eager path applies
-// to queries and keys alike (cascade_attention.py:284-291); `post` is that factor (1: no such product).
-// Products of two 16-bit values and sums of two 16-bit values are exact in fp32, so rounding the fp32
-// result once is the reference's rounding.  Returns the packed pairs (first halves, second halves).
-template <typename T>
-__device__ inline void rope_ref_pairs(float x1a, float x1b, float x2a, float x2b, float ca, float sa, float cb, float sb,
-                                      float post, bool scale_after, uint32_t& first, uint32_t& second) {
-    const uint32_t pa = Mma<T>::pack2(x1a * ca, x2a * sa), qa = Mma<T>::pack2(x2a * ca, x1a * sa);
-    const uint32_t pb = Mma<T>::pack2(x1b * cb, x2b * sb), qb = Mma<T>::pack2(x2b * cb, x1b * sb);
-    first = Mma<T>::pack2(Mma<T>::lo_f(pa) - Mma<T>::hi_f(pa), Mma<T>::lo_f(pb) - Mma<T>::hi_f(pb));
-    second = Mma<T>::pack2(Mma<T>::lo_f(qa) + Mma<T>::hi_f(qa), Mma<T>::lo_f(qb) + Mma<T>::hi_f(qb));
-    if (scale_after) {
-        first = Mma<T>::pack2(Mma<T>::lo_f(first) * post, Mma<T>::hi_f(first) * post);
-        second = Mma<T>::pack2(Mma<T>::lo_f(second) * post, Mma<T>::hi_f(second) * post);
-    }
-}
-
 struct KeySegment {
     const void* k;
     const void* v;
@@ -176,19 +156,23 @@ __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int sp
         if (tid == 0) p.tile_vis[tile] = bal;
     }
 
-    float cs[16], sn[16];
-    const bool rotate = sidx >= 0 && p.seg[sidx].pos != nullptr;
-    if (rotate && p.shared_pos) {
-        const int64_t pos = p.seg[sidx].pos[local] + p.seg[sidx].pos_shift;
+    // cos / sin of this thread's 16 rotation pairs, two per word, rounded to the tensor dtype (see RopeWord)
+    RopeWord<T> rw[8];
+    auto trig_at = [&](int64_t pos) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int j = stage_pair(quarter, i);
-            const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
-            fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
-            sn[i] = Mma<T>::round1(sn[i]);
-            cs[i] = Mma<T>::round1(cs[i]);
+        for (int k = 0; k < 8; k++) {
+            float sn[2], cs[2];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int j = stage_pair(quarter, 2 * k + e);
+                const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
+                fast_sincos(__fmul_rn((float)pos, f), &sn[e], &cs[e]);
+            }
+            rw[k] = RopeWord<T>::make(cs[0], sn[0], cs[1], sn[1]);
         }
-    }
+    };
+    const bool rotate = sidx >= 0 && p.seg[sidx].pos != nullptr;
+    if (rotate && p.shared_pos) trig_at(p.seg[sidx].pos[local] + p.seg[sidx].pos_shift);
     const bool key_scaled = p.key_scale != 1.0f;
     const int64_t nbh = p.B * p.KVH;
     // the rows of unit bh as this thread's eight 16-byte pieces (zeros past the last key)
@@ -240,28 +224,12 @@ __device__ inline void stage_keys_block(const StageParams& p, int tile_i, int sp
         if (sidx >= 0) {
             const KeySegment& sg = p.seg[sidx];
             if (rotate) {
-                if (!p.shared_pos) {
-                    const int64_t pos = sg.pos[b * sg.pos_stride[0] + kvh * sg.pos_stride[1] + local] + sg.pos_shift;
-#pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        const int j = stage_pair(quarter, i);
-                        const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
-                        fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
-                        sn[i] = Mma<T>::round1(sn[i]);
-                        cs[i] = Mma<T>::round1(cs[i]);
-                    }
-                }
-                // on packed pairs: two elements per word, converted and rounded (to nearest even, like the
-                // element-wise casts) by the packed conversion instructions
+                if (!p.shared_pos)
+                    trig_at(sg.pos[b * sg.pos_stride[0] + kvh * sg.pos_stride[1] + local] + sg.pos_shift);
                 uint32_t* lw = reinterpret_cast<uint32_t*>(lo);
                 uint32_t* hw = reinterpret_cast<uint32_t*>(hi);
 #pragma unroll
-                for (int k = 0; k < 8; k++) {
-                    const float x1a = Mma<T>::lo_f(lw[k]), x1b = Mma<T>::hi_f(lw[k]);
-                    const float x2a = Mma<T>::lo_f(hw[k]), x2b = Mma<T>::hi_f(hw[k]);
-                    rope_ref_pairs<T>(x1a, x1b, x2a, x2b, cs[2 * k], sn[2 * k], cs[2 * k + 1], sn[2 * k + 1], p.key_scale,
-                                      key_scaled, lw[k], hw[k]);
-                }
+                for (int k = 0; k < 8; k++) rw[k].rotate(lw[k], hw[k], p.key_scale, key_scaled, lw[k], hw[k]);
             }
         }
         char* kimg = (char*)p.kr + (bh * (p.n_pad / kBN) + tile) * (int64_t)(kD * kBN * sizeof(T));
@@ -331,16 +299,19 @@ __device__ inline void stage_q_block(const StageQParams& p, int blk, int share_i
     const int64_t m = idx >> 2;
     const int quarter = idx & 3;
     if (m >= p.Q) return;
-    float cs[16], sn[16];
+    RopeWord<T> rw[8];
     if (p.q_pos) {
         const int64_t pos = p.q_pos[m];
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int j = stage_pair(quarter, i);
-            const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
-            fast_sincos(__fmul_rn((float)pos, f), &sn[i], &cs[i]);
-            sn[i] = Mma<T>::round1(sn[i]);
-            cs[i] = Mma<T>::round1(cs[i]);
+        for (int k = 0; k < 8; k++) {
+            float sn[2], cs[2];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int j = stage_pair(quarter, 2 * k + e);
+                const float f = p.inv_freq ? p.inv_freq[j] : 1.0f / powf(p.theta, (float)(2 * j) / (float)kD);
+                fast_sincos(__fmul_rn((float)pos, f), &sn[e], &cs[e]);
+            }
+            rw[k] = RopeWord<T>::make(cs[0], sn[0], cs[1], sn[1]);
         }
     }
     const int64_t nbh = p.rows / p.Q;
@@ -374,14 +345,11 @@ __device__ inline void stage_q_block(const StageQParams& p, int blk, int share_i
         uint32_t* hw = reinterpret_cast<uint32_t*>(r.hi);
 #pragma unroll
         for (int k = 0; k < 8; k++) {  // on packed pairs, as in stage_keys_block
-            const float x1a = Mma<T>::lo_f(lw[k]), x1b = Mma<T>::hi_f(lw[k]);
-            const float x2a = Mma<T>::lo_f(hw[k]), x2b = Mma<T>::hi_f(hw[k]);
             if (p.q_pos) {
-                rope_ref_pairs<T>(x1a, x1b, x2a, x2b, cs[2 * k], sn[2 * k], cs[2 * k + 1], sn[2 * k + 1], p.qscale, true,
-                                  lw[k], hw[k]);
+                rw[k].rotate(lw[k], hw[k], p.qscale, true, lw[k], hw[k]);
             } else {
-                lw[k] = Mma<T>::pack2(x1a * p.qscale, x1b * p.qscale);
-                hw[k] = Mma<T>::pack2(x2a * p.qscale, x2b * p.qscale);
+                lw[k] = Mma<T>::pack2(Mma<T>::lo_f(lw[k]) * p.qscale, Mma<T>::hi_f(lw[k]) * p.qscale);
+                hw[k] = Mma<T>::pack2(Mma<T>::lo_f(hw[k]) * p.qscale, Mma<T>::hi_f(hw[k]) * p.qscale);
             }
         }
         T* dst = (T*)p.qr + (bh * p.Q + m) * kD;

@@ -113,6 +113,78 @@ __device__ inline void fast_sincos(float x, float* sn, float* cs) {
     *cs = __builtin_amdgcn_cosf(rev);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Rotary embedding on packed 16-bit words with the roundings of the reference's eager path, which evaluates
+// x*cos + rotate_half(x)*sin in the tensor dtype (cascade_attention.py:31-35; cos and sin cast to the dtype,
+// modeling_llama.py:219-220) and then multiplies queries and keys alike by sqrt(softmax scale)
+// (cascade_attention.py:284-291).  w1 holds elements (j, j+1) of a row, w2 their rotation partners (j+64, j+65);
+// RopeWord carries the rounded cos / sin of the two pairs in the form the arithmetic consumes.  Every product of
+// two 16-bit values and every sum of two 16-bit values is exact in fp32, so each conversion to the tensor dtype
+// is one of the reference's roundings: the four products, the two sums, and the products with `post`.
+// ---------------------------------------------------------------------------------------------
+typedef __bf16 ckv_bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 ckv_f16x2 __attribute__((ext_vector_type(2)));
+typedef float ckv_f32x2 __attribute__((ext_vector_type(2)));
+
+template <typename T>
+struct RopeWord;
+// bfloat16 has no packed arithmetic on this chip, but v_dot2_f32_bf16 multiplies both halves of a word without
+// unpacking them: with (c, 0) or (0, c) as the other operand it returns one exact product, with (1, -1) or (1, 1)
+// the exact difference or sum of a packed pair.
+template <>
+struct RopeWord<__hip_bfloat16> {
+    uint32_t c_lo, c_hi, s_lo, s_hi;  // (c0, 0), (0, c1), (s0, 0), (0, s1)
+    __device__ static uint32_t pack2(float a, float b) {
+        ckv_f32x2 f = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, ckv_bf16x2));
+    }
+    __device__ static float lo(uint32_t w) { return __uint_as_float(w << 16); }
+    __device__ static float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+    __device__ static RopeWord make(float c0, float s0, float c1, float s1) {
+        return RopeWord{pack2(c0, 0.f), pack2(0.f, c1), pack2(s0, 0.f), pack2(0.f, s1)};
+    }
+    __device__ static float dot(uint32_t a, uint32_t b) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(ckv_bf16x2, a), __builtin_bit_cast(ckv_bf16x2, b), 0.f, false);
+    }
+    // scaled == false: the rotation alone
+    __device__ void rotate(uint32_t w1, uint32_t w2, float post, bool scaled, uint32_t& o1, uint32_t& o2) const {
+        const uint32_t p0 = pack2(dot(w1, c_lo), dot(w2, s_lo)), q0 = pack2(dot(w2, c_lo), dot(w1, s_lo));
+        const uint32_t p1 = pack2(dot(w1, c_hi), dot(w2, s_hi)), q1 = pack2(dot(w2, c_hi), dot(w1, s_hi));
+        constexpr uint32_t kOneMinusOne = 0xbf803f80u, kOneOne = 0x3f803f80u;  // (1, -1), (1, 1)
+        o1 = pack2(dot(p0, kOneMinusOne), dot(p1, kOneMinusOne));
+        o2 = pack2(dot(q0, kOneOne), dot(q1, kOneOne));
+        if (scaled) {
+            o1 = pack2(lo(o1) * post, hi(o1) * post);
+            o2 = pack2(lo(o2) * post, hi(o2) * post);
+        }
+    }
+};
+// float16: the packed multiply, subtract and add round each result to float16, which is the reference's arithmetic
+template <>
+struct RopeWord<__half> {
+    uint32_t c, s;  // (c0, c1), (s0, s1)
+    __device__ static uint32_t pack2(float a, float b) {
+        ckv_f32x2 f = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, ckv_f16x2));
+    }
+    __device__ static float lo(uint32_t w) { return (float)__builtin_bit_cast(ckv_f16x2, w)[0]; }
+    __device__ static float hi(uint32_t w) { return (float)__builtin_bit_cast(ckv_f16x2, w)[1]; }
+    __device__ static RopeWord make(float c0, float s0, float c1, float s1) { return RopeWord{pack2(c0, c1), pack2(s0, s1)}; }
+    __device__ void rotate(uint32_t w1, uint32_t w2, float post, bool scaled, uint32_t& o1, uint32_t& o2) const {
+#pragma clang fp contract(off)  // a fused multiply-add would skip the rounding of the product
+        const ckv_f16x2 x1 = __builtin_bit_cast(ckv_f16x2, w1), x2 = __builtin_bit_cast(ckv_f16x2, w2);
+        const ckv_f16x2 cc = __builtin_bit_cast(ckv_f16x2, c), ss = __builtin_bit_cast(ckv_f16x2, s);
+        const ckv_f16x2 a1 = x1 * cc, b1 = x2 * ss, a2 = x2 * cc, b2 = x1 * ss;
+        const ckv_f16x2 r1 = a1 - b1, r2 = a2 + b2;
+        o1 = __builtin_bit_cast(uint32_t, r1);
+        o2 = __builtin_bit_cast(uint32_t, r2);
+        if (scaled) {
+            o1 = pack2(lo(o1) * post, hi(o1) * post);
+            o2 = pack2(lo(o2) * post, hi(o2) * post);
+        }
+    }
+};
+
 __device__ inline const void* uniform_ptr(const void* p) {
     const uint64_t v = reinterpret_cast<uint64_t>(p);
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
