@@ -551,3 +551,35 @@ def test_backward_head_sizes_outside_the_reference_set(D, dtype):
         rtol = 2.0 ** -6 if dtype == torch.bfloat16 else 0.0
         excess = ((got.float() - want.float()).abs() - rtol * want.float().abs()).max().item()
         assert excess <= atol, f"{name}: error exceeds the allowance by {excess:.3e}"
+
+
+@pytest.mark.parametrize("dtype,H,KVH", [(torch.bfloat16, 8, 2), (torch.float16, 14, 2), (torch.float32, 8, 2)])
+def test_filled_slots_hint_changes_nothing(dtype, H, KVH):
+    """``ckv_attn_args.filled_slots`` is a hint, never a second mask: single-token steps on a cache that is still
+    filling give bit-identical outputs, scores and score cache whether the caller passes the hint (the host wrapper
+    does, from its token counter) or not (``replayable=True`` leaves it out) -- on the streaming kernels, which use
+    it to skip empty tiles, and on the paths that ignore it."""
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
+
+    B, D, NS, W, C = 2, 128, 4, 256, 4
+    with_hint, without = (make_pair(B, KVH, D, NS, W, C, dtype)[0] for _ in range(2))
+    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    gen = torch.Generator().manual_seed(31)
+    q = (torch.randn(B, H, 150, D, generator=gen) * 0.7).to(dtype).cuda()
+    k = (torch.randn(B, KVH, 150, D, generator=gen) * 0.7).to(dtype).cuda()
+    v = (torch.randn(B, KVH, 150, D, generator=gen) * 0.7).to(dtype).cuda()
+    for c in (with_hint, without):
+        cascade_attention(q, k, v, c, 0, inv_freq)         # 146 of 1024 slots filled
+    for step in range(6):
+        q1 = (torch.randn(B, H, 1, D, generator=gen) * 0.7).to(dtype).cuda()
+        k1 = (torch.randn(B, KVH, 1, D, generator=gen) * 0.7).to(dtype).cuda()
+        v1 = (torch.randn(B, KVH, 1, D, generator=gen) * 0.7).to(dtype).cuda()
+        out_a, new_a = cascade_attention(q1, k1, v1, with_hint, 0, inv_freq)
+        out_b, new_b = cascade_attention(q1, k1, v1, without, 0, inv_freq, replayable=True)
+        torch.cuda.synchronize()
+        assert torch.equal(out_a.view(torch.uint8), out_b.view(torch.uint8)), f"step {step}: out"
+        assert torch.equal(new_a.view(torch.uint8), new_b.view(torch.uint8)), f"step {step}: new scores"
+        for name in STATE:
+            a, b = getattr(with_hint, name)[0], getattr(without, name)[0]
+            assert torch.equal(a.view(torch.uint8) if a.dtype.is_floating_point else a,
+                               b.view(torch.uint8) if b.dtype.is_floating_point else b), f"step {step}: {name}"
