@@ -209,3 +209,47 @@ def test_config3_consecutive_decode_steps_update_bit_exact():
             g, w = bits(getattr(gpu, name)[0].cpu()), bits(getattr(cpu, name))
             assert torch.equal(g, w), f"step {step}: {name} differs from the oracle"
         assert int(gpu.seen_tokens_by_layer[0]) == int(cpu.seen_tokens)
+
+
+def test_config3_all_1024_decode_steps():
+    """Config 3 as it is written: the cache pre-filled full, then 1024 single-token steps in a row through the real
+    path (attention, score EMA, update).  The oracle's update follows with the library's own scores; the trackers are
+    compared after every step, every other state tensor but K and V every 64 steps, K and V at the end: bit for
+    bit.  Outputs stay finite and the position ids a permutation throughout."""
+    from cascading_kv_cache_amd.cascade_attention import cascade_attention, default_inv_freq
+    from parity_helpers import STATE, bits, push_state
+    from test_gpu_update import make_pair
+
+    dtype = torch.bfloat16
+    B, H, KVH, D, NS, W, C = 16, 32, 8, 128, 64, 8192, 4
+    gpu, cpu = make_pair(B, KVH, D, NS, W, C, dtype)
+    gen = torch.Generator().manual_seed(47)
+    for _ in range(5):  # 40960 tokens through the oracle alone: cache full, every cascade evicting
+        n = 8192
+        k = torch.randn(B, KVH, n, D, generator=gen).to(dtype)
+        v = torch.randn(B, KVH, n, D, generator=gen).to(dtype)
+        cpu.update(k, v, (torch.rand(B, KVH, n, generator=gen) * 1e-6).to(dtype))
+    del k, v
+    push_state(gpu, cpu)
+    inv_freq = default_inv_freq(D, 5e5, "cuda:0")
+    qs = torch.randn(8, B, H, 1, D, generator=gen).to(dtype).cuda()
+    ks = torch.randn(8, B, KVH, 1, D, generator=gen).to(dtype)
+    vs = torch.randn(8, B, KVH, 1, D, generator=gen).to(dtype)
+    ks_d, vs_d = ks.cuda(), vs.cuda()
+    light = ("stored_tokens", "start_indices", "stored_sinks")
+    for step in range(1024):
+        i = step % 8
+        out, new_g = cascade_attention(qs[i], ks_d[i], vs_d[i], gpu, 0, inv_freq, update_cache=False)
+        cpu.score_cache.copy_(gpu.score_cache[0])          # the update's score inputs are the library's own
+        gpu.update(ks_d[i], vs_d[i], 0, score_states=new_g)
+        cpu.update(ks[i], vs[i], new_g.cpu())
+        last = step == 1023
+        names = STATE if last else (tuple(n for n in STATE if n not in ("key_cache", "value_cache")) if step % 64 == 63 else light)
+        for name in names:
+            g, w = bits(getattr(gpu, name)[0].cpu()), bits(getattr(cpu, name))
+            assert torch.equal(g, w), f"step {step}: {name} differs from the oracle"
+        if step % 64 == 63 or last:
+            assert bool(torch.isfinite(out.float()).all()), f"step {step}: output"
+            row = gpu.pos[0][0, 0].sort().values
+            assert torch.equal(row, torch.arange(W * C, device="cuda:0")), f"step {step}: position ids"
+    assert int(gpu.seen_tokens_by_layer[0]) == int(cpu.seen_tokens) == 5 * 8192 + 1024
