@@ -237,6 +237,7 @@ int run_bwd(const BwdParams& p, hipStream_t stream) {
     }
     hipLaunchKernelGGL(bwd_delta_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(kThreads), 0, stream, p);
     CKV_HIP_TRY(hipGetLastError());
+    if (bwd_mfma_supported(a)) return launch_bwd_mfma(a, p.delta, stream);
     if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(bwd_dq_kernel<T>), (int)lds_dq)) return rc;
     hipLaunchKernelGGL(bwd_dq_kernel<T>, dim3((unsigned)((a.n_ctx + kOwn - 1) / kOwn), (unsigned)(a.B * a.H)), dim3(kThreads),
                        lds_dq, stream, p);

@@ -1,0 +1,450 @@
+// Backward of the dense-input attention operator on the matrix cores (cascade/models/flash_attention.py:279-537):
+// bf16 / fp16, head_dim 128, v_mfma_f32_32x32x16.  Two kernels, as in the reference (_attn_bwd_dq, _attn_bwd_dkdv),
+// so that no gradient is accumulated with atomics; both recompute the probabilities from the row normalisers of
+// the forward pass and take delta[m] = sum_d out[m, d] dout[m, d] from the caller.
+//
+//   dq     a wavefront owns 32 query rows, a workgroup 128; 32-key blocks of K and V stream through LDS.
+//          S^T = K Q^T and dP^T = V dO^T keep a query in one lane (its normaliser and delta are one value per
+//          lane), dS^T = P^T (dP^T - delta) scale is, packed, directly the B operand of dQ^T += K^T dS^T.
+//   dkdv   a wavefront owns 32 keys, a workgroup 128; 32-row blocks of Q and dO stream through LDS.
+//          S = Q K^T and dP = dO V^T keep a key in one lane; P and dS are the B operands of
+//          dV^T += dO^T P and dK^T += Q^T dS.
+//
+// The A operands K^T, Q^T and dO^T are read from the row-major tiles in LDS with the transposing read
+// ds_read_b64_tr_b16: lane i of a 16-lane group receives element [4e + i/4][i%4] (e = 0..3) of the 16 x 4 matrix
+// whose row r is the 8 bytes lane r points at; with lane r pointing at dims 4 (r%4) .. +3 of row r/4 of a
+// 4-row group, lane i receives dim i of the four rows.  Rows are 256 bytes; the 16-byte piece c of row r sits in
+// slot c ^ (((r & 3) << 2) | ((r >> 2) & 3)), which keeps both the 16-byte row reads (32 rows, one piece) and the
+// transposing reads (4 rows x 64 bytes) off each other's banks.
+#include "ckv_attn_internal.h"
+
+namespace ckv {
+namespace {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kHD = 128;              // head dim
+constexpr int kBlk = 32;              // rows of a streamed block
+constexpr int kWaves = 4;             // wavefronts of a workgroup, 32 stationary rows each
+constexpr int kThreads = kWaves * CKV_WAVE;
+constexpr int kOwn = kWaves * 32;     // stationary rows of a workgroup
+constexpr int kRowBytes = kHD * 2;    // 256
+constexpr int kTile = kBlk * kRowBytes;  // 8 KiB
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<__hip_bfloat16> {
+    __device__ static f32x16 mma(uint4 a, uint4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c,
+                                                       0, 0, 0);
+    }
+    __device__ static uint32_t pack2(float lo, float hi) {
+        f32x2 f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+    }
+};
+template <>
+struct Mma<__half> {
+    __device__ static f32x16 mma(uint4 a, uint4 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0,
+                                                      0, 0);
+    }
+    __device__ static uint32_t pack2(float lo, float hi) {
+        f32x2 f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+    }
+};
+
+struct BwdMfmaParams {
+    ckv_dense_bwd_args a;
+    const float* delta;  // (B, H, n_ctx)
+};
+
+__device__ inline int swz(int row, int piece) { return piece ^ (((row & 3) << 2) | ((row >> 2) & 3)); }
+
+// The two 16-byte pieces a thread carries of a 32-row block: rows tid/16 and tid/16 + 16, piece tid%16.
+struct BlockRegs {
+    uint4 p[2];
+};
+
+__device__ inline BlockRegs load_block(const char* base, int64_t row_bytes, int64_t first, int64_t limit, int tid) {
+    BlockRegs r;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int64_t row = first + tid / 16 + 16 * j;
+        r.p[j] = make_uint4(0u, 0u, 0u, 0u);
+        if (row < limit) r.p[j] = *reinterpret_cast<const uint4*>(base + row * row_bytes + (tid % 16) * 16);
+    }
+    return r;
+}
+
+__device__ inline void store_block(unsigned char* tile, const BlockRegs& r, int tid) {
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int row = tid / 16 + 16 * j;
+        *reinterpret_cast<uint4*>(tile + row * kRowBytes + swz(row, tid % 16) * 16) = r.p[j];
+    }
+}
+
+// A operand of a product that contracts over the head dims: row lane%32 of the tile, dims 16 ds + 8 (lane/32) .. +7
+__device__ inline uint4 row_operand(const unsigned char* tile, int lane, int ds) {
+    const int row = lane & 31;
+    return *reinterpret_cast<const uint4*>(tile + row * kRowBytes + swz(row, 2 * ds + (lane >> 5)) * 16);
+}
+
+// A operand of a product that contracts over the rows of the tile: dim 32 db + lane%32 of rows
+// 16 s + 8 a + 4 (lane/32) + e (elements 4 a + e), the order in which the packed B operand holds them.
+// `tr_base[a]` is the lane's address for db = 0, s = 0; blocks of 32 dims flip bits 2-3 of the slot.
+__device__ inline uint4 col_operand(uint32_t tile_lds, const int (&tr_base)[2], int s, int db) {
+    uint4 r;
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+        const uint32_t addr = tile_lds + (uint32_t)((tr_base[a] ^ (db << 6)) + s * 16 * kRowBytes);
+        const s16x4_t v =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(uintptr_t)addr);
+        const uint2 u = __builtin_bit_cast(uint2, v);
+        if (a == 0) {
+            r.x = u.x;
+            r.y = u.y;
+        } else {
+            r.z = u.x;
+            r.w = u.y;
+        }
+    }
+    return r;
+}
+
+__device__ inline void col_operand_setup(int lane, int (&tr_base)[2]) {
+    const int h = lane >> 5, g16 = (lane >> 4) & 1, rl = lane & 15;
+#pragma unroll
+    for (int a = 0; a < 2; a++) {
+        const int row = 8 * a + 4 * h + (rl >> 2);             // + 16 s
+        const int piece = 2 * g16 + ((rl & 3) >> 1);           // + 4 db
+        tr_base[a] = row * kRowBytes + swz(row, piece) * 16 + 8 * (rl & 1);
+    }
+}
+
+template <typename T>
+__device__ inline uint4 pack8(const f32x16& v, int s) {
+    return make_uint4(Mma<T>::pack2(v[8 * s + 0], v[8 * s + 1]), Mma<T>::pack2(v[8 * s + 2], v[8 * s + 3]),
+                      Mma<T>::pack2(v[8 * s + 4], v[8 * s + 5]), Mma<T>::pack2(v[8 * s + 6], v[8 * s + 7]));
+}
+
+__device__ inline f32x16 zero16() {
+    f32x16 z;
+#pragma unroll
+    for (int i = 0; i < 16; i++) z[i] = 0.f;
+    return z;
+}
+
+// ---------------------------------------------------------------------------------------------
+// dq
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(kThreads) bwd_mfma_dq_kernel(BwdMfmaParams p) {
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2][2][kTile];  // [stage][K, V]
+    const ckv_dense_bwd_args& a = p.a;
+    const int tid = threadIdx.x, wave = tid / CKV_WAVE, lane = tid % CKV_WAVE, h = lane >> 5;
+    const int64_t n_ctx = a.n_ctx, n_kv = a.n_kv, n_cached = n_kv - n_ctx;
+    const int64_t bh = blockIdx.y, b = bh / a.H, hd = bh % a.H;
+    const int64_t m_wg = (int64_t)blockIdx.x * kOwn;
+    const int64_t m_lane = m_wg + wave * 32 + (lane & 31);  // this lane's query
+    const char* kb = reinterpret_cast<const char*>(a.k) + (b * a.kv_stride[0] + hd * a.kv_stride[1]) * 2;
+    const char* vb = reinterpret_cast<const char*>(a.v) + (b * a.kv_stride[0] + hd * a.kv_stride[1]) * 2;
+    const int64_t kv_row = a.kv_stride[2] * 2;
+
+    // stationary B operands: Q^T and dO^T of this lane's query, dims 16 ds + 8 h .. +7
+    uint4 qreg[kHD / 16], greg[kHD / 16];
+    {
+        const char* qrow = reinterpret_cast<const char*>(a.q) +
+                           (b * a.q_stride[0] + hd * a.q_stride[1] + m_lane * a.q_stride[2]) * 2;
+        const char* grow = reinterpret_cast<const char*>(a.dout) +
+                           (b * a.dout_stride[0] + hd * a.dout_stride[1] + m_lane * a.dout_stride[2]) * 2;
+#pragma unroll
+        for (int ds = 0; ds < kHD / 16; ds++) {
+            qreg[ds] = greg[ds] = make_uint4(0u, 0u, 0u, 0u);
+            if (m_lane < n_ctx) {
+                qreg[ds] = *reinterpret_cast<const uint4*>(qrow + (16 * ds + 8 * h) * 2);
+                greg[ds] = *reinterpret_cast<const uint4*>(grow + (16 * ds + 8 * h) * 2);
+            }
+        }
+    }
+    const bool row_ok = m_lane < n_ctx;
+    const float nlse2 = row_ok ? -a.lse[bh * n_ctx + m_lane] * kLog2e : 0.f;
+    const float delta = row_ok ? p.delta[bh * n_ctx + m_lane] : 0.f;
+    const float c2 = a.scale * kLog2e;
+
+    int tr_base[2];
+    col_operand_setup(lane, tr_base);
+    const uint32_t lds0 = lds_address(&smem[0][0][0]);
+
+    f32x16 dq[kHD / 32];
+#pragma unroll
+    for (int db = 0; db < kHD / 32; db++) dq[db] = zero16();
+
+    // keys past the diagonal of the workgroup's last row are visible to none of its rows
+    int64_t m_last = m_wg + kOwn - 1;
+    if (m_last > n_ctx - 1) m_last = n_ctx - 1;
+    const int64_t n_end = n_cached + m_last + 1;
+    const int nblk = (int)((n_end + kBlk - 1) / kBlk);
+
+    {
+        const BlockRegs k0 = load_block(kb, kv_row, 0, n_kv, tid), v0 = load_block(vb, kv_row, 0, n_kv, tid);
+        store_block(smem[0][0], k0, tid);
+        store_block(smem[0][1], v0, tid);
+    }
+    __syncthreads();
+    for (int blk = 0; blk < nblk; blk++) {
+        const int st = blk & 1;
+        const int64_t n0 = (int64_t)blk * kBlk;
+        BlockRegs kn, vn;
+        const bool more = blk + 1 < nblk;
+        if (more) {
+            kn = load_block(kb, kv_row, n0 + kBlk, n_kv, tid);
+            vn = load_block(vb, kv_row, n0 + kBlk, n_kv, tid);
+        }
+        // which keys of the block any query may see: inside the tensor, and not masked if cached
+        uint32_t vis;
+        {
+            const int64_t n = n0 + (lane & 31);
+            bool ok = n < n_kv;
+            if (ok && n < n_cached) ok = a.mask[n] == 0;
+            vis = (uint32_t)__ballot(ok);
+        }
+        // keys of this block that are chunk keys past this wavefront's last row: nothing to do for it
+        const bool chunk_part = n0 + kBlk > n_cached;
+        const int64_t wave_last = m_wg + wave * 32 + 31;
+        const bool dead = vis == 0u || (n0 >= n_cached && n0 - n_cached > wave_last);
+        if (!dead) {
+            const unsigned char* kt = smem[st][0];
+            const unsigned char* vt = smem[st][1];
+            f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+            for (int ds = 0; ds < kHD / 16; ds++) s = Mma<T>::mma(row_operand(kt, lane, ds), qreg[ds], s);
+#pragma unroll
+            for (int ds = 0; ds < kHD / 16; ds++) dp = Mma<T>::mma(row_operand(vt, lane, ds), greg[ds], dp);
+            f32x16 dsv;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int r = 8 * (i / 4) + 4 * h + (i % 4);  // key of the block
+                bool ok = ((vis >> r) & 1u) != 0u && row_ok;
+                if (chunk_part) {
+                    const int64_t n = n0 + r;
+                    if (n >= n_cached) ok = ok && (n - n_cached) <= m_lane;
+                }
+                const float pe = ok ? __builtin_amdgcn_exp2f(fmaf(s[i], c2, nlse2)) : 0.f;
+                dsv[i] = pe * (dp[i] - delta) * a.scale;
+            }
+            const uint32_t kt_lds = lds0 + (uint32_t)(st * 2 * kTile);
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                const uint4 bop = pack8<T>(dsv, s2);
+#pragma unroll
+                for (int db = 0; db < kHD / 32; db++) dq[db] = Mma<T>::mma(col_operand(kt_lds, tr_base, s2, db), bop, dq[db]);
+            }
+        }
+        if (more) {
+            store_block(smem[st ^ 1][0], kn, tid);
+            store_block(smem[st ^ 1][1], vn, tid);
+        }
+        __syncthreads();
+    }
+    if (row_ok) {
+        char* out = reinterpret_cast<char*>(a.dq) + (b * a.dq_stride[0] + hd * a.dq_stride[1] + m_lane * a.dq_stride[2]) * 2;
+#pragma unroll
+        for (int db = 0; db < kHD / 32; db++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int d = 32 * db + 8 * j + 4 * h;
+                *reinterpret_cast<uint2*>(out + d * 2) = make_uint2(Mma<T>::pack2(dq[db][4 * j], dq[db][4 * j + 1]),
+                                                                    Mma<T>::pack2(dq[db][4 * j + 2], dq[db][4 * j + 3]));
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dk, dv
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(kThreads) bwd_mfma_dkdv_kernel(BwdMfmaParams p) {
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2][2][kTile];  // [stage][Q, dO]
+    __shared__ __attribute__((aligned(16))) float rowv[2][2][kBlk];                                       // [stage][-lse log2 e, delta]
+    const ckv_dense_bwd_args& a = p.a;
+    const int tid = threadIdx.x, wave = tid / CKV_WAVE, lane = tid % CKV_WAVE, h = lane >> 5;
+    const int64_t n_ctx = a.n_ctx, n_kv = a.n_kv, n_cached = n_kv - n_ctx;
+    const int64_t bh = blockIdx.y, b = bh / a.H, hd = bh % a.H;
+    const int64_t n_wg = (int64_t)blockIdx.x * kOwn;
+    const int64_t n_lane = n_wg + wave * 32 + (lane & 31);  // this lane's key
+    const char* qb = reinterpret_cast<const char*>(a.q) + (b * a.q_stride[0] + hd * a.q_stride[1]) * 2;
+    const char* gb = reinterpret_cast<const char*>(a.dout) + (b * a.dout_stride[0] + hd * a.dout_stride[1]) * 2;
+    const int64_t q_row = a.q_stride[2] * 2, g_row = a.dout_stride[2] * 2;
+    const float* lse = a.lse + bh * n_ctx;
+    const float* dl = p.delta + bh * n_ctx;
+
+    // stationary B operands: K^T and V^T of this lane's key
+    uint4 kreg[kHD / 16], vreg[kHD / 16];
+    {
+        const int64_t off = (b * a.kv_stride[0] + hd * a.kv_stride[1] + n_lane * a.kv_stride[2]) * 2;
+        const char* krow = reinterpret_cast<const char*>(a.k) + off;
+        const char* vrow = reinterpret_cast<const char*>(a.v) + off;
+#pragma unroll
+        for (int ds = 0; ds < kHD / 16; ds++) {
+            kreg[ds] = vreg[ds] = make_uint4(0u, 0u, 0u, 0u);
+            if (n_lane < n_kv) {
+                kreg[ds] = *reinterpret_cast<const uint4*>(krow + (16 * ds + 8 * h) * 2);
+                vreg[ds] = *reinterpret_cast<const uint4*>(vrow + (16 * ds + 8 * h) * 2);
+            }
+        }
+    }
+    bool key_ok = n_lane < n_kv;
+    if (key_ok && n_lane < n_cached) key_ok = a.mask[n_lane] == 0;
+    const int64_t first_row = n_lane < n_cached ? 0 : n_lane - n_cached;  // the first query that sees this key
+    const float c2 = a.scale * kLog2e;
+
+    int tr_base[2];
+    col_operand_setup(lane, tr_base);
+    const uint32_t lds0 = lds_address(&smem[0][0][0]);
+
+    f32x16 dk[kHD / 32], dv[kHD / 32];
+#pragma unroll
+    for (int db = 0; db < kHD / 32; db++) dk[db] = dv[db] = zero16();
+
+    // the first query block any key of the workgroup can be seen from
+    const int64_t m_first = n_wg < n_cached ? 0 : n_wg - n_cached;
+    const int blk0 = (int)(m_first / kBlk);
+    const int nblk = (int)((n_ctx + kBlk - 1) / kBlk);
+    // does any key of this wavefront exist and pass its mask?
+    const bool wave_alive = __ballot(key_ok) != 0ull;
+    const int64_t wave_first_key = n_wg + wave * 32;
+
+    auto load_rowv = [&](int st, int64_t m0) {
+        if (tid < 2 * kBlk) {
+            const int64_t m = m0 + (tid & (kBlk - 1));
+            float v = 0.f;
+            if (m < n_ctx) v = tid < kBlk ? -lse[m] * kLog2e : dl[m];
+            rowv[st][tid / kBlk][tid & (kBlk - 1)] = v;
+        }
+    };
+    if (blk0 < nblk) {
+        const BlockRegs q0 = load_block(qb, q_row, (int64_t)blk0 * kBlk, n_ctx, tid);
+        const BlockRegs g0 = load_block(gb, g_row, (int64_t)blk0 * kBlk, n_ctx, tid);
+        store_block(smem[blk0 & 1][0], q0, tid);
+        store_block(smem[blk0 & 1][1], g0, tid);
+        load_rowv(blk0 & 1, (int64_t)blk0 * kBlk);
+    }
+    __syncthreads();
+    for (int blk = blk0; blk < nblk; blk++) {
+        const int st = blk & 1;
+        const int64_t m0 = (int64_t)blk * kBlk;
+        BlockRegs qn, gn;
+        const bool more = blk + 1 < nblk;
+        if (more) {
+            qn = load_block(qb, q_row, m0 + kBlk, n_ctx, tid);
+            gn = load_block(gb, g_row, m0 + kBlk, n_ctx, tid);
+        }
+        // rows before the first chunk key of the wavefront's keys see none of them when all its keys are chunk keys
+        const bool dead = !wave_alive || (wave_first_key >= n_cached && wave_first_key - n_cached > m0 + kBlk - 1);
+        if (!dead) {
+            const unsigned char* qt = smem[st][0];
+            const unsigned char* gt = smem[st][1];
+            f32x16 s = zero16(), dp = zero16();
+#pragma unroll
+            for (int ds = 0; ds < kHD / 16; ds++) s = Mma<T>::mma(row_operand(qt, lane, ds), kreg[ds], s);
+#pragma unroll
+            for (int ds = 0; ds < kHD / 16; ds++) dp = Mma<T>::mma(row_operand(gt, lane, ds), vreg[ds], dp);
+            f32x16 pv, dsv;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float4 nl = *reinterpret_cast<const float4*>(&rowv[st][0][8 * j + 4 * h]);
+                const float4 de = *reinterpret_cast<const float4*>(&rowv[st][1][8 * j + 4 * h]);
+                const float nls[4] = {nl.x, nl.y, nl.z, nl.w}, des[4] = {de.x, de.y, de.z, de.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int i = 4 * j + e;
+                    const int64_t m = m0 + 8 * j + 4 * h + e;
+                    const bool ok = key_ok && m < n_ctx && m >= first_row;
+                    const float pe = ok ? __builtin_amdgcn_exp2f(fmaf(s[i], c2, nls[e])) : 0.f;
+                    pv[i] = pe;
+                    dsv[i] = pe * (dp[i] - des[e]) * a.scale;
+                }
+            }
+            const uint32_t qt_lds = lds0 + (uint32_t)(st * 2 * kTile), gt_lds = qt_lds + kTile;
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                const uint4 pb = pack8<T>(pv, s2), db_ = pack8<T>(dsv, s2);
+#pragma unroll
+                for (int db = 0; db < kHD / 32; db++) {
+                    dv[db] = Mma<T>::mma(col_operand(gt_lds, tr_base, s2, db), pb, dv[db]);
+                    dk[db] = Mma<T>::mma(col_operand(qt_lds, tr_base, s2, db), db_, dk[db]);
+                }
+            }
+        }
+        if (more) {
+            store_block(smem[st ^ 1][0], qn, tid);
+            store_block(smem[st ^ 1][1], gn, tid);
+            load_rowv(st ^ 1, m0 + kBlk);
+        }
+        __syncthreads();
+    }
+    if (n_lane < n_kv) {
+        const int64_t off = (b * a.dkv_stride[0] + hd * a.dkv_stride[1] + n_lane * a.dkv_stride[2]) * 2;
+        char* ok_ = reinterpret_cast<char*>(a.dk) + off;
+        char* ov_ = reinterpret_cast<char*>(a.dv) + off;
+#pragma unroll
+        for (int db = 0; db < kHD / 32; db++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int d = 32 * db + 8 * j + 4 * h;
+                *reinterpret_cast<uint2*>(ok_ + d * 2) = make_uint2(Mma<T>::pack2(dk[db][4 * j], dk[db][4 * j + 1]),
+                                                                    Mma<T>::pack2(dk[db][4 * j + 2], dk[db][4 * j + 3]));
+                *reinterpret_cast<uint2*>(ov_ + d * 2) = make_uint2(Mma<T>::pack2(dv[db][4 * j], dv[db][4 * j + 1]),
+                                                                    Mma<T>::pack2(dv[db][4 * j + 2], dv[db][4 * j + 3]));
+            }
+        }
+    }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+inline bool rows_ok(const int64_t* st) { return st[3] == 1 && st[2] % 8 == 0 && st[1] % 8 == 0 && st[0] % 8 == 0; }
+
+template <typename T>
+int run(const BwdMfmaParams& p, hipStream_t stream) {
+    const ckv_dense_bwd_args& a = p.a;
+    hipLaunchKernelGGL(bwd_mfma_dq_kernel<T>, dim3((unsigned)((a.n_ctx + kOwn - 1) / kOwn), (unsigned)(a.B * a.H)),
+                       dim3(kThreads), 0, stream, p);
+    CKV_HIP_TRY(hipGetLastError());
+    hipLaunchKernelGGL(bwd_mfma_dkdv_kernel<T>, dim3((unsigned)((a.n_kv + kOwn - 1) / kOwn), (unsigned)(a.B * a.H)),
+                       dim3(kThreads), 0, stream, p);
+    CKV_HIP_TRY(hipGetLastError());
+    return CKV_OK;
+}
+
+}  // namespace
+
+bool bwd_mfma_supported(const ckv_dense_bwd_args& a) {
+    if (a.dtype != CKV_F16 && a.dtype != CKV_BF16) return false;
+    if (a.D != kHD) return false;
+    if (!rows_ok(a.q_stride) || !rows_ok(a.kv_stride) || !rows_ok(a.dout_stride) || !rows_ok(a.dq_stride) ||
+        !rows_ok(a.dkv_stride))
+        return false;
+    return aligned16(a.q) && aligned16(a.k) && aligned16(a.v) && aligned16(a.dout) && aligned16(a.dq) &&
+           aligned16(a.dk) && aligned16(a.dv);
+}
+
+int launch_bwd_mfma(const ckv_dense_bwd_args& a, const float* delta, hipStream_t stream) {
+    BwdMfmaParams p;
+    p.a = a;
+    p.delta = delta;
+    return a.dtype == CKV_F16 ? run<__half>(p, stream) : run<__hip_bfloat16>(p, stream);
+}
+
+}  // namespace ckv

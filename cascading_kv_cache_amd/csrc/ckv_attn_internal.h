@@ -117,6 +117,10 @@ int mfma_device_cus();  // compute units of the current device (256 where none c
 bool mfma_fits(int64_t n);  // the per-tile bookkeeping of n keys fits in LDS
 int launch_mfma(const MfmaProblem& p, hipStream_t stream);
 
+// ---- backward of the dense operator on the matrix cores (16-bit, head_dim 128, 16-byte addressable rows) ----
+bool bwd_mfma_supported(const ckv_dense_bwd_args& a);
+int launch_bwd_mfma(const ckv_dense_bwd_args& a, const float* delta, hipStream_t stream);  // delta: (B, H, n_ctx)
+
 // ---- single-token decode family (Q == 1, head_dim 128) ----
 bool decode_supported(const ckv_attn_args& a);
 int64_t decode_workspace_bytes(int64_t B, int64_t H, int64_t KVH, int64_t num_sink, int64_t S);

@@ -170,3 +170,34 @@ def test_fused_projections_keep_the_decoder(preset_bias):
     for name in ("mask", "sink_mask", "pos", "sink_pos", "stored_tokens", "start_indices", "stored_sinks"):
         for i in range(cfg.num_layers):
             assert torch.equal(getattr(ca, name)[i], getattr(cb, name)[i]), f"layer {i}: {name}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_chunked_prefill_equals_one_dense_shot_while_the_stream_fits(dtype):
+    """cascade/models/test.py:123-165 on the device: sinks 64, window 2048 as one cascade, stride 128, a 988-token
+    prompt.  While nothing has been evicted, streaming the prompt through the cache in strides gives the logits of
+    one dense causal pass over the whole prompt (here: the same decoder fed the prompt as a single chunk into a fresh
+    cache, which is plain causal attention with ordinary positions): within 1e-1 of each other relative to the
+    logits' scale, and the same argmax wherever the dense pass's best logit leads by more than that tolerance."""
+    from cascading_kv_cache_amd.decoder import PRESETS, CascadeDecoder
+
+    cfg = PRESETS["tiny"]
+    model = CascadeDecoder(cfg, dtype=dtype, device="cuda:0", seed=11)
+    n, stride = 988, 128
+    ids = torch.randint(0, cfg.vocab_size, (1, n), generator=torch.Generator().manual_seed(12)).cuda()
+    with torch.no_grad():
+        dense = model(ids, model.new_cache(2048, 1, batch=1, num_sink_tokens=64), last_only=False).float()
+        cache = model.new_cache(2048, 1, batch=1, num_sink_tokens=64)
+        chunked = torch.cat([model(ids[:, i:i + stride], cache, last_only=False) for i in range(0, n, stride)], 1).float()
+    assert chunked.shape == dense.shape == (1, n, cfg.vocab_size)
+    scale = dense.abs().max().item()
+    err = (chunked - dense).abs().max().item()
+    rel = 1e-4 if dtype == torch.float32 else 3e-2
+    assert err <= rel * scale, f"{dtype}: logits differ by {err:.3e} (scale {scale:.3e})"
+    top2 = dense.topk(2, dim=-1).values
+    clear = (top2[..., 0] - top2[..., 1]) > 2 * rel * scale
+    # float32 leaves nearly every position with a clear winner; at the 16-bit tolerance about four in ten
+    assert int(clear.sum()) > (n // 2 if dtype == torch.float32 else n // 4), "too few clear winners to compare"
+    assert torch.equal(chunked.argmax(-1)[clear], dense.argmax(-1)[clear])
+    assert cache.seen_tokens_by_layer.cpu().tolist() == [n] * cfg.num_layers
+    assert int(cache.start_indices[0].sum()) == 0, "nothing may have been evicted"
