@@ -650,6 +650,37 @@ def run_short_strides(cache, dtype, device):
     return out
 
 
+def run_dense_backward(device, dtype):
+    """Backward of the dense operator ``attention(q, k, v, causal, sm_scale, mask, beta)`` at the largest shape of the
+    reference's own test (cascade/models/test.py:255-267: Z=2, H=32, 1024 rows, 16384 cached + 1024 chunk keys,
+    head_dim 128, half of the cached keys masked): dq, dk, dv on the matrix cores.  Algorithmic work = the five matrix
+    products of the backward over the visible (row, key) pairs; the kernels run seven (both recompute QK^T and
+    dO V^T) over every unmasked 32-key block."""
+    from cascading_kv_cache_amd import flash_attention as fa
+
+    Z, H, n_ctx, n_kv, D = 2, 32, 1024, 16384 + 1024, 128
+    g = torch.Generator(device=device).manual_seed(20)
+    q, k, v, do = (torch.randn(Z, H, n, D, device=device, dtype=torch.float32, generator=g).mul_(0.5).to(dtype)
+                   for n in (n_ctx, n_kv, n_kv, n_ctx))
+    mask = torch.rand(n_kv - n_ctx, device=device, generator=g) > 0.5
+    o, _, lse, m = fa._forward(q, k, v, True, 0.5, mask, 0.999, True)
+    for _ in range(2):
+        dq, dk, dv = fa._backward(q, k, v, o, lse, m, do, 0.5)
+    assert all(bool(torch.isfinite(t.float()).all()) for t in (dq, dk, dv))
+    reps = 10
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fa._backward(q, k, v, o, lse, m, do, 0.5)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / reps
+    visible = float((~mask).sum()) + (n_ctx + 1) / 2
+    flops = 5 * 2.0 * Z * H * n_ctx * visible * D
+    return dict(workload=f"dq, dk, dv of the dense operator: Z={Z}, H={H}, {n_ctx} rows, {n_kv - n_ctx} cached (half "
+                         f"masked) + {n_ctx} chunk keys, head_dim {D}, bf16",
+                ms=dt * 1e3, algorithmic_tflop=flops / 1e12, tflops=flops / dt / 1e12, frac_of_bf16_peak=flops / dt / 2.5e15)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -659,7 +690,7 @@ def main():
     ap.add_argument("--no-sub", action="store_true", help="skip the cfg2 / cfg3 sub-records")
     ap.add_argument("--no-model", action="store_true", help="skip the full-model record (cfg4)")
     ap.add_argument("--model-prompt", type=int, default=None, help="shorter prompt for the full-model records")
-    ap.add_argument("--only", choices=["layer", "cfg2", "cfg3", "cfg4", "cfg5"], default=None,
+    ap.add_argument("--only", choices=["layer", "cfg2", "cfg3", "cfg4", "cfg5", "bwd"], default=None,
                     help="run one workload only (for profiler runs); the JSON line then carries that record alone")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 512 MiB device copy, the known-size reference that scales the "
@@ -686,6 +717,9 @@ def main():
     if args.only in ("cfg4", "cfg5"):
         print(json.dumps({args.only: run_model(MODEL4 if args.only == "cfg4" else MODEL5, device, dtype, args.model_prompt)}))
         return
+    if args.only == "bwd":
+        print(json.dumps({"dense_backward": run_dense_backward(device, dtype)}))
+        return
     if args.only in ("cfg2", "cfg3"):
         rec = (run_cfg2 if args.only == "cfg2" else run_cfg3)(max(args.steps, 3), args.warmup, dtype, device)
         calibrate()
@@ -699,6 +733,8 @@ def main():
     del cache, pool
     torch.cuda.empty_cache()
     gpu1 = None if sub else run_gpu_config1(device)
+    bwd = None if sub else run_dense_backward(device, dtype)
+    torch.cuda.empty_cache()
     cfg2 = None if sub else run_cfg2(max(args.steps, 20), args.warmup, dtype, device)
     torch.cuda.empty_cache()
     cfg3 = None if sub else run_cfg3(max(args.steps, 1024), args.warmup, dtype, device)   # the configuration's 1024 steps
@@ -745,6 +781,7 @@ def main():
         "cfg4_full_model": cfg4,
         "cfg5_full_model": cfg5,
         "short_stride": short,
+        "dense_backward": bwd,
     }
     print(json.dumps(line))
 

@@ -1,8 +1,9 @@
 // Backward of the dense-input attention operator (cascade/models/flash_attention.py:279-537, 654-710):
 // dq, dk, dv of  out = softmax(scale * q k^T + masks) v  with the cache mask on the first n_kv - n_ctx keys
-// and the causal mask on the last n_ctx.  Only training reaches it (the inference path never differentiates),
-// so these are plain fp32-math kernels for every dtype and head size up to 192, tiled through LDS; the
-// probabilities are recomputed from the row normalisers the forward pass returns.
+// and the causal mask on the last n_ctx.  Only training reaches it (the inference path never differentiates).
+// The kernels in this file are plain fp32-math kernels for every dtype and head size up to 192, tiled through
+// LDS; 16-bit tensors with head_dim 128 go to the matrix-core kernels of ckv_attn_bwd_mfma.hip after the delta
+// kernel.  The probabilities are recomputed from the row normalisers the forward pass returns.
 //
 //   delta   delta[m] = sum_d out[m, d] * dout[m, d]                      (flash_attention.py:279-294)
 //   dq      one workgroup = 16 query rows of a head, key tiles of 64 stream through LDS:

@@ -37,6 +37,10 @@ constexpr int kOwn = kWaves * 32;     // stationary rows of a workgroup
 constexpr int kRowBytes = kHD * 2;    // 256
 constexpr int kTile = kBlk * kRowBytes;  // 8 KiB
 constexpr float kLog2e = 1.4426950408889634f;
+// dynamic LDS of the dk/dv kernel: two stages of (Q, dO) tiles, the per-row scalars of both stages, V^T operands
+constexpr int kDkdvRowv = 2 * 2 * kTile;
+constexpr int kDkdvV = kDkdvRowv + 2 * 2 * kBlk * (int)sizeof(float);
+constexpr int kDkdvLds = kDkdvV + kWaves * (kHD / 16) * CKV_WAVE * 16;
 
 template <typename T>
 struct Mma;
@@ -70,27 +74,20 @@ struct BwdMfmaParams {
 
 __device__ inline int swz(int row, int piece) { return piece ^ (((row & 3) << 2) | ((row >> 2) & 3)); }
 
-// The two 16-byte pieces a thread carries of a 32-row block: rows tid/16 and tid/16 + 16, piece tid%16.
-struct BlockRegs {
-    uint4 p[2];
-};
-
-__device__ inline BlockRegs load_block(const char* base, int64_t row_bytes, int64_t first, int64_t limit, int tid) {
-    BlockRegs r;
+// A 32-row block of a (rows, 128) tensor into a tile, global -> LDS without registers: wavefront w copies rows
+// 8 w .. 8 w + 7 with two instructions of 64 x 16 bytes; lane i fills slot i % 16 of row 4 (2 w + j) + i / 16 with
+// the piece that belongs there.  Rows at or past `limit` repeat row limit - 1 (finite values; whatever is
+// computed from them is masked).  The caller waits with vmcnt(0) before the barrier that publishes the tile.
+__device__ inline void copy_block(const char* base, int64_t row_bytes, int64_t first, int64_t limit, uint32_t tile_lds,
+                                  int wave, int lane) {
+    const char* blk = base + first * row_bytes;  // uniform
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-        const int64_t row = first + tid / 16 + 16 * j;
-        r.p[j] = make_uint4(0u, 0u, 0u, 0u);
-        if (row < limit) r.p[j] = *reinterpret_cast<const uint4*>(base + row * row_bytes + (tid % 16) * 16);
-    }
-    return r;
-}
-
-__device__ inline void store_block(unsigned char* tile, const BlockRegs& r, int tid) {
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int row = tid / 16 + 16 * j;
-        *reinterpret_cast<uint4*>(tile + row * kRowBytes + swz(row, tid % 16) * 16) = r.p[j];
+        const int row = 4 * (2 * wave + j) + (lane >> 4);
+        int64_t rr = row;
+        if (first + rr > limit - 1) rr = limit - 1 - first;
+        const uint32_t voff = (uint32_t)(rr * row_bytes) + (uint32_t)(swz(row, lane & 15) << 4);
+        async_copy16(blk, voff, tile_lds + (uint32_t)(4 * (2 * wave + j) * kRowBytes));
     }
 }
 
@@ -149,7 +146,7 @@ __device__ inline f32x16 zero16() {
 // dq
 // ---------------------------------------------------------------------------------------------
 template <typename T>
-__global__ void __launch_bounds__(kThreads) bwd_mfma_dq_kernel(BwdMfmaParams p) {
+__global__ void __launch_bounds__(kThreads, 2) bwd_mfma_dq_kernel(BwdMfmaParams p) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[2][2][kTile];  // [stage][K, V]
     const ckv_dense_bwd_args& a = p.a;
     const int tid = threadIdx.x, wave = tid / CKV_WAVE, lane = tid % CKV_WAVE, h = lane >> 5;
@@ -196,31 +193,37 @@ __global__ void __launch_bounds__(kThreads) bwd_mfma_dq_kernel(BwdMfmaParams p) 
     const int64_t n_end = n_cached + m_last + 1;
     const int nblk = (int)((n_end + kBlk - 1) / kBlk);
 
-    {
-        const BlockRegs k0 = load_block(kb, kv_row, 0, n_kv, tid), v0 = load_block(vb, kv_row, 0, n_kv, tid);
-        store_block(smem[0][0], k0, tid);
-        store_block(smem[0][1], v0, tid);
-    }
+    // which keys of a block any query may see: inside the tensor, and not masked if cached.  The mask byte of the
+    // block after this one is requested before that block's copies and looked at after this block's work, so
+    // that nothing in between waits for memory.
+    auto mask_byte = [&](int64_t n0) -> uint32_t {
+        const int64_t n = n0 + (lane & 31);
+        return n < n_kv ? (n < n_cached ? (uint32_t)a.mask[n] : 0u) : 1u;
+    };
+    uint32_t vis = (uint32_t)__ballot(mask_byte(0) == 0u);
+    copy_block(kb, kv_row, 0, n_kv, lds0, wave, lane);
+    copy_block(vb, kv_row, 0, n_kv, lds0 + kTile, wave, lane);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
     for (int blk = 0; blk < nblk; blk++) {
         const int st = blk & 1;
         const int64_t n0 = (int64_t)blk * kBlk;
-        BlockRegs kn, vn;
-        const bool more = blk + 1 < nblk;
-        if (more) {
-            kn = load_block(kb, kv_row, n0 + kBlk, n_kv, tid);
-            vn = load_block(vb, kv_row, n0 + kBlk, n_kv, tid);
+        uint32_t mb_next = 1u;
+        if (blk + 1 < nblk) {  // the other stage was last read before the barrier that ended the step before
+            mb_next = mask_byte(n0 + kBlk);
+            __builtin_amdgcn_sched_barrier(0);
+            copy_block(kb, kv_row, n0 + kBlk, n_kv, lds0 + (uint32_t)((st ^ 1) * 2 * kTile), wave, lane);
+            copy_block(vb, kv_row, n0 + kBlk, n_kv, lds0 + (uint32_t)((st ^ 1) * 2 * kTile + kTile), wave, lane);
         }
-        // which keys of the block any query may see: inside the tensor, and not masked if cached
-        uint32_t vis;
-        {
-            const int64_t n = n0 + (lane & 31);
-            bool ok = n < n_kv;
-            if (ok && n < n_cached) ok = a.mask[n] == 0;
-            vis = (uint32_t)__ballot(ok);
-        }
+        __builtin_amdgcn_sched_barrier(0);
         // keys of this block that are chunk keys past this wavefront's last row: nothing to do for it
         const bool chunk_part = n0 + kBlk > n_cached;
+        // chunk key r of the block is visible to this lane's query iff r <= r_last (every r when the block is cached)
+        int64_t r_last64 = m_lane + n_cached - n0;
+        if (r_last64 > kBlk) r_last64 = kBlk;
+        if (r_last64 < -1) r_last64 = -1;
+        const int r_last = (int)r_last64;
+        const int r_cached = n_cached - n0 >= kBlk ? kBlk : (n_cached > n0 ? (int)(n_cached - n0) : 0);  // r < r_cached: cached
         const int64_t wave_last = m_wg + wave * 32 + 31;
         const bool dead = vis == 0u || (n0 >= n_cached && n0 - n_cached > wave_last);
         if (!dead) {
@@ -228,18 +231,21 @@ __global__ void __launch_bounds__(kThreads) bwd_mfma_dq_kernel(BwdMfmaParams p) 
             const unsigned char* vt = smem[st][1];
             f32x16 s = zero16(), dp = zero16();
 #pragma unroll
-            for (int ds = 0; ds < kHD / 16; ds++) s = Mma<T>::mma(row_operand(kt, lane, ds), qreg[ds], s);
+            for (int ds = 0; ds < kHD / 16; ds++) {
+                s = Mma<T>::mma(row_operand(kt, lane, ds), qreg[ds], s);
+                if ((ds & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
-            for (int ds = 0; ds < kHD / 16; ds++) dp = Mma<T>::mma(row_operand(vt, lane, ds), greg[ds], dp);
+            for (int ds = 0; ds < kHD / 16; ds++) {
+                dp = Mma<T>::mma(row_operand(vt, lane, ds), greg[ds], dp);
+                if ((ds & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+            }
             f32x16 dsv;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int r = 8 * (i / 4) + 4 * h + (i % 4);  // key of the block
                 bool ok = ((vis >> r) & 1u) != 0u && row_ok;
-                if (chunk_part) {
-                    const int64_t n = n0 + r;
-                    if (n >= n_cached) ok = ok && (n - n_cached) <= m_lane;
-                }
+                if (chunk_part) ok = ok && (r < r_cached || r <= r_last);
                 const float pe = ok ? __builtin_amdgcn_exp2f(fmaf(s[i], c2, nlse2)) : 0.f;
                 dsv[i] = pe * (dp[i] - delta) * a.scale;
             }
@@ -248,13 +254,15 @@ __global__ void __launch_bounds__(kThreads) bwd_mfma_dq_kernel(BwdMfmaParams p) 
             for (int s2 = 0; s2 < 2; s2++) {
                 const uint4 bop = pack8<T>(dsv, s2);
 #pragma unroll
-                for (int db = 0; db < kHD / 32; db++) dq[db] = Mma<T>::mma(col_operand(kt_lds, tr_base, s2, db), bop, dq[db]);
+                for (int db = 0; db < kHD / 32; db++) {
+                    dq[db] = Mma<T>::mma(col_operand(kt_lds, tr_base, s2, db), bop, dq[db]);
+                    if (db & 1) __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
-        if (more) {
-            store_block(smem[st ^ 1][0], kn, tid);
-            store_block(smem[st ^ 1][1], vn, tid);
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's copies of the next block have landed
+        vis = (uint32_t)__ballot(mb_next == 0u);
         __syncthreads();
     }
     if (row_ok) {
@@ -275,9 +283,14 @@ __global__ void __launch_bounds__(kThreads) bwd_mfma_dq_kernel(BwdMfmaParams p) 
 // dk, dv
 // ---------------------------------------------------------------------------------------------
 template <typename T>
-__global__ void __launch_bounds__(kThreads) bwd_mfma_dkdv_kernel(BwdMfmaParams p) {
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2][2][kTile];  // [stage][Q, dO]
-    __shared__ __attribute__((aligned(16))) float rowv[2][2][kBlk];                                       // [stage][-lse log2 e, delta]
+__global__ void __launch_bounds__(kThreads, 2) bwd_mfma_dkdv_kernel(BwdMfmaParams p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char dyn_smem[];
+    typedef unsigned char (*TilePtr)[2][kTile];
+    typedef float (*RowPtr)[2][kBlk];
+    TilePtr smem = reinterpret_cast<TilePtr>(dyn_smem);                                  // [stage][Q, dO]
+    RowPtr rowv = reinterpret_cast<RowPtr>(dyn_smem + kDkdvRowv);                        // [stage][-lse log2 e, delta]
+    // the V^T operands of a wavefront's 32 keys, in operand order: [wave][ds][lane] 16 bytes each
+    uint4* vstat = reinterpret_cast<uint4*>(dyn_smem + kDkdvV) + (threadIdx.x / CKV_WAVE) * (kHD / 16) * CKV_WAVE;
     const ckv_dense_bwd_args& a = p.a;
     const int tid = threadIdx.x, wave = tid / CKV_WAVE, lane = tid % CKV_WAVE, h = lane >> 5;
     const int64_t n_ctx = a.n_ctx, n_kv = a.n_kv, n_cached = n_kv - n_ctx;
@@ -290,19 +303,21 @@ __global__ void __launch_bounds__(kThreads) bwd_mfma_dkdv_kernel(BwdMfmaParams p
     const float* lse = a.lse + bh * n_ctx;
     const float* dl = p.delta + bh * n_ctx;
 
-    // stationary B operands: K^T and V^T of this lane's key
-    uint4 kreg[kHD / 16], vreg[kHD / 16];
+    // stationary B operands: K^T of this lane's key in registers, V^T in LDS (the registers go to the accumulators)
+    uint4 kreg[kHD / 16];
     {
         const int64_t off = (b * a.kv_stride[0] + hd * a.kv_stride[1] + n_lane * a.kv_stride[2]) * 2;
         const char* krow = reinterpret_cast<const char*>(a.k) + off;
         const char* vrow = reinterpret_cast<const char*>(a.v) + off;
 #pragma unroll
         for (int ds = 0; ds < kHD / 16; ds++) {
-            kreg[ds] = vreg[ds] = make_uint4(0u, 0u, 0u, 0u);
+            kreg[ds] = make_uint4(0u, 0u, 0u, 0u);
+            uint4 vv = make_uint4(0u, 0u, 0u, 0u);
             if (n_lane < n_kv) {
                 kreg[ds] = *reinterpret_cast<const uint4*>(krow + (16 * ds + 8 * h) * 2);
-                vreg[ds] = *reinterpret_cast<const uint4*>(vrow + (16 * ds + 8 * h) * 2);
+                vv = *reinterpret_cast<const uint4*>(vrow + (16 * ds + 8 * h) * 2);
             }
+            vstat[ds * CKV_WAVE + lane] = vv;
         }
     }
     bool key_ok = n_lane < n_kv;
@@ -312,7 +327,7 @@ __global__ void __launch_bounds__(kThreads) bwd_mfma_dkdv_kernel(BwdMfmaParams p
 
     int tr_base[2];
     col_operand_setup(lane, tr_base);
-    const uint32_t lds0 = lds_address(&smem[0][0][0]);
+    const uint32_t lds0 = lds_address(dyn_smem);
 
     f32x16 dk[kHD / 32], dv[kHD / 32];
 #pragma unroll
@@ -335,64 +350,95 @@ __global__ void __launch_bounds__(kThreads) bwd_mfma_dkdv_kernel(BwdMfmaParams p
         }
     };
     if (blk0 < nblk) {
-        const BlockRegs q0 = load_block(qb, q_row, (int64_t)blk0 * kBlk, n_ctx, tid);
-        const BlockRegs g0 = load_block(gb, g_row, (int64_t)blk0 * kBlk, n_ctx, tid);
-        store_block(smem[blk0 & 1][0], q0, tid);
-        store_block(smem[blk0 & 1][1], g0, tid);
+        copy_block(qb, q_row, (int64_t)blk0 * kBlk, n_ctx, lds0 + (uint32_t)((blk0 & 1) * 2 * kTile), wave, lane);
+        copy_block(gb, g_row, (int64_t)blk0 * kBlk, n_ctx, lds0 + (uint32_t)((blk0 & 1) * 2 * kTile + kTile), wave, lane);
         load_rowv(blk0 & 1, (int64_t)blk0 * kBlk);
     }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
     for (int blk = blk0; blk < nblk; blk++) {
         const int st = blk & 1;
         const int64_t m0 = (int64_t)blk * kBlk;
-        BlockRegs qn, gn;
         const bool more = blk + 1 < nblk;
-        if (more) {
-            qn = load_block(qb, q_row, m0 + kBlk, n_ctx, tid);
-            gn = load_block(gb, g_row, m0 + kBlk, n_ctx, tid);
+        float rv_next = 0.f;  // this thread's per-row scalar of the next block: requested first, parked in LDS last
+        if (more) {  // the other stage was last read before the barrier that ended the step before
+            if (tid < 2 * kBlk) {
+                const int64_t m = m0 + kBlk + (tid & (kBlk - 1));
+                if (m < n_ctx) rv_next = tid < kBlk ? lse[m] : dl[m];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            copy_block(qb, q_row, m0 + kBlk, n_ctx, lds0 + (uint32_t)((st ^ 1) * 2 * kTile), wave, lane);
+            copy_block(gb, g_row, m0 + kBlk, n_ctx, lds0 + (uint32_t)((st ^ 1) * 2 * kTile + kTile), wave, lane);
         }
         // rows before the first chunk key of the wavefront's keys see none of them when all its keys are chunk keys
         const bool dead = !wave_alive || (wave_first_key >= n_cached && wave_first_key - n_cached > m0 + kBlk - 1);
         if (!dead) {
             const unsigned char* qt = smem[st][0];
             const unsigned char* gt = smem[st][1];
-            f32x16 s = zero16(), dp = zero16();
+            // rows r of the block with r_lo <= r < r_hi see this lane's key
+            int64_t lo64 = first_row - m0, hi64 = n_ctx - m0;
+            if (lo64 < 0) lo64 = 0;
+            if (lo64 > kBlk) lo64 = kBlk;
+            if (hi64 > kBlk) hi64 = kBlk;
+            const int r_lo = key_ok ? (int)lo64 : kBlk, r_hi = (int)hi64;
+            const uint32_t qt_lds = lds0 + (uint32_t)(st * 2 * kTile), gt_lds = qt_lds + kTile;
+            // The phases are fenced so that the compiler keeps their registers apart: P, then dV, then dP and dS, then dK.
+            f32x16 pv = zero16();
 #pragma unroll
-            for (int ds = 0; ds < kHD / 16; ds++) s = Mma<T>::mma(row_operand(qt, lane, ds), kreg[ds], s);
-#pragma unroll
-            for (int ds = 0; ds < kHD / 16; ds++) dp = Mma<T>::mma(row_operand(gt, lane, ds), vreg[ds], dp);
-            f32x16 pv, dsv;
+            for (int ds = 0; ds < kHD / 16; ds++) {
+                pv = Mma<T>::mma(row_operand(qt, lane, ds), kreg[ds], pv);
+                if ((ds & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const float4 nl = *reinterpret_cast<const float4*>(&rowv[st][0][8 * j + 4 * h]);
-                const float4 de = *reinterpret_cast<const float4*>(&rowv[st][1][8 * j + 4 * h]);
-                const float nls[4] = {nl.x, nl.y, nl.z, nl.w}, des[4] = {de.x, de.y, de.z, de.w};
+                const float nls[4] = {nl.x, nl.y, nl.z, nl.w};
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    const int i = 4 * j + e;
-                    const int64_t m = m0 + 8 * j + 4 * h + e;
-                    const bool ok = key_ok && m < n_ctx && m >= first_row;
-                    const float pe = ok ? __builtin_amdgcn_exp2f(fmaf(s[i], c2, nls[e])) : 0.f;
-                    pv[i] = pe;
-                    dsv[i] = pe * (dp[i] - des[e]) * a.scale;
+                    const int i = 4 * j + e, r = 8 * j + 4 * h + e;
+                    pv[i] = r >= r_lo && r < r_hi ? __builtin_amdgcn_exp2f(fmaf(pv[i], c2, nls[e])) : 0.f;
                 }
             }
-            const uint32_t qt_lds = lds0 + (uint32_t)(st * 2 * kTile), gt_lds = qt_lds + kTile;
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++) {
-                const uint4 pb = pack8<T>(pv, s2), db_ = pack8<T>(dsv, s2);
+                const uint4 pb = pack8<T>(pv, s2);
 #pragma unroll
                 for (int db = 0; db < kHD / 32; db++) {
                     dv[db] = Mma<T>::mma(col_operand(gt_lds, tr_base, s2, db), pb, dv[db]);
+                    if (db & 1) __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            f32x16 dp = zero16();
+#pragma unroll
+            for (int ds = 0; ds < kHD / 16; ds++) {
+                dp = Mma<T>::mma(row_operand(gt, lane, ds), vstat[ds * CKV_WAVE + lane], dp);
+                if (ds & 1) __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float4 de = *reinterpret_cast<const float4*>(&rowv[st][1][8 * j + 4 * h]);
+                const float des[4] = {de.x, de.y, de.z, de.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int i = 4 * j + e;
+                    dp[i] = pv[i] * (dp[i] - des[e]) * a.scale;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                const uint4 db_ = pack8<T>(dp, s2);
+#pragma unroll
+                for (int db = 0; db < kHD / 32; db++) {
                     dk[db] = Mma<T>::mma(col_operand(qt_lds, tr_base, s2, db), db_, dk[db]);
+                    if (db & 1) __builtin_amdgcn_sched_barrier(0);
                 }
             }
         }
-        if (more) {
-            store_block(smem[st ^ 1][0], qn, tid);
-            store_block(smem[st ^ 1][1], gn, tid);
-            load_rowv(st ^ 1, m0 + kBlk);
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's copies of the next block have landed
+        if (more && tid < 2 * kBlk) rowv[st ^ 1][tid / kBlk][tid & (kBlk - 1)] = tid < kBlk ? -rv_next * kLog2e : rv_next;
         __syncthreads();
     }
     if (n_lane < n_kv) {
@@ -422,8 +468,9 @@ int run(const BwdMfmaParams& p, hipStream_t stream) {
     hipLaunchKernelGGL(bwd_mfma_dq_kernel<T>, dim3((unsigned)((a.n_ctx + kOwn - 1) / kOwn), (unsigned)(a.B * a.H)),
                        dim3(kThreads), 0, stream, p);
     CKV_HIP_TRY(hipGetLastError());
+    if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(bwd_mfma_dkdv_kernel<T>), kDkdvLds)) return rc;
     hipLaunchKernelGGL(bwd_mfma_dkdv_kernel<T>, dim3((unsigned)((a.n_kv + kOwn - 1) / kOwn), (unsigned)(a.B * a.H)),
-                       dim3(kThreads), 0, stream, p);
+                       dim3(kThreads), kDkdvLds, stream, p);
     CKV_HIP_TRY(hipGetLastError());
     return CKV_OK;
 }

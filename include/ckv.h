@@ -250,7 +250,10 @@ int ckv_attn_dense(const ckv_dense_args* args, void* stream);
  * gradient of the output, writes dq, dk, dv (dtype and shapes of q, k, v); the scores carry no gradient, as
  * in the reference.  Masked cached keys receive zero gradients.  head_dim: a multiple of 16, up to 192 (anything
  * else, or a device whose workgroups get less LDS than the fp32 tiles of head_dim + 1 columns need, is refused with
- * CKV_ERR_UNSUPPORTED before anything is launched).
+ * CKV_ERR_UNSUPPORTED before anything is launched).  bf16 / fp16 tensors with head_dim 128, unit stride along the
+ * head dim, every other stride a multiple of 8 elements and 16-byte aligned base addresses run on the matrix cores
+ * (probabilities and dS rounded to the tensor dtype for the products, fp32 accumulation); everything else runs
+ * fp32-math kernels.
  * ---------------------------------------------------------------------------------------- */
 typedef struct ckv_dense_bwd_args {
     const void* q;                 /* (B, H, n_ctx, D) */

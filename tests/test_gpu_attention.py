@@ -354,56 +354,21 @@ def dense_reference(q, k, v, mask, sm_scale):
 def test_dense_operator_forward(Z, H, N_CTX, N_KV, HEAD_DIM, dtype):
     """The forward half of cascade/models/test.py:177-269: seed 20, N(0, 0.5) inputs, sm_scale 0.5,
     random cache mask, atol 1e-2 (1e-4 in float32)."""
-    from cascading_kv_cache_amd.flash_attention import attention
-
-    torch.manual_seed(20)
-    q = torch.empty((Z, H, N_CTX, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5)
-    k = torch.empty((Z, H, N_KV, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5)
-    v = torch.empty((Z, H, N_KV, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5)
-    mask = torch.rand(N_KV - N_CTX, device="cuda") > 0.5
-    ref, p = dense_reference(q, k, v, mask, 0.5)
-    out, scores = attention(q, k, v, True, 0.5, mask, 0.9999)
-    atol = 1e-4 if dtype == torch.float32 else 1e-2
-    assert (out.float() - ref).abs().max().item() <= atol
-    # exact version of what cascade/models/test.py:271-318 only rank-correlates
-    w = (1 - 0.9999) * 0.9999 ** torch.arange(N_CTX - 1, -1, -1, device="cuda", dtype=torch.float64)
-    want = (p.double() * w[None, None, :, None]).sum(dim=2)
-    assert_scores_close(scores, want, dtype, "dense scores")
-
-
-def test_attention_rejects_cpu_tensors():
-    from cascading_kv_cache_amd import _abi
-    from cascading_kv_cache_amd.flash_attention import attention
-
-    q = torch.zeros(1, 1, 16, 64)
-    with pytest.raises(_abi.CkvError):
-        attention(q, q, q, True, 1.0, torch.zeros(0, dtype=torch.bool), 0.9)
-
-
-@pytest.mark.parametrize("Z,H,N_CTX,N_KV,HEAD_DIM", [
-    (1, 2, 128, 128, 64), (1, 2, 256, 256, 64), (1, 2, 512, 512, 64), (1, 1, 128, 128 + 128, 64),
-    (1, 2, 1024, 16384 + 1024, 64), (2, 32, 1024, 16384 + 1024, 128), (1, 2, 512, 2560, 64),
-    (1, 2, 500, 2048 + 500, 64), (1, 2, 500, 2048 + 64 + 500, 64), (2, 3, 77, 300 + 77, 32),
-    (1, 3, 90, 200 + 90, 16),   # the smallest head size the operator takes
-])
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
-def test_dense_operator_backward(Z, H, N_CTX, N_KV, HEAD_DIM, dtype):
-    """The backward half of cascade/models/test.py:177-269: seed 20, N(0, 0.5) inputs, sm_scale 0.5, random cache
-    mask; dq, dk, dv of the operator against autograd through the dense formula (softmax in float32, then the
-    product with v in the tensor dtype), atol 1e-2 in float16 as in the reference's test, 1e-4 in float32, 2e-2 in
-    bfloat16 plus two units in the last place of the value (gradients of a key seen by hundreds of rows reach
-    magnitudes of 4 to 8, where neighbouring bfloat16 values are 3e-2 apart, and the reference formula rounds P
-    and the products to bfloat16 where the kernels round once)."""
-    from cascading_kv_cache_amd.flash_attention import attention
-
     torch.manual_seed(20)
     q = torch.empty((Z, H, N_CTX, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
     k = torch.empty((Z, H, N_KV, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
     v = torch.empty((Z, H, N_KV, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
     mask = torch.rand(N_KV - N_CTX, device="cuda") > 0.5
+    check_backward_against_autograd(q, k, v, mask, dtype)
+
+
+def check_backward_against_autograd(q, k, v, mask, dtype, sm_scale=0.5):
+    """dq, dk, dv of ``attention`` against autograd through the dense formula; q, k, v are leaves."""
+    from cascading_kv_cache_amd.flash_attention import attention
+
+    N_CTX, N_KV = q.size(2), k.size(2)
     full = torch.cat((mask[None, :].expand(N_CTX, -1),
                       torch.ones(N_CTX, N_CTX, dtype=torch.bool, device="cuda").triu(1)), dim=-1)
-    sm_scale = 0.5
     dout = torch.randn_like(q)
     p = torch.matmul(q, k.transpose(2, 3)) * sm_scale
     p = p.masked_fill(full, float("-inf"))
@@ -428,6 +393,40 @@ def test_dense_operator_backward(Z, H, N_CTX, N_KV, HEAD_DIM, dtype):
     if int(mask.sum()) > 0:
         assert k.grad[:, :, : N_KV - N_CTX][:, :, mask].abs().max().item() == 0.0
         assert v.grad[:, :, : N_KV - N_CTX][:, :, mask].abs().max().item() == 0.0
+
+
+@pytest.mark.parametrize("Z,H,N_CTX,N_KV", [
+    (1, 2, 128, 128), (1, 2, 100, 100), (1, 1, 128, 128 + 128), (1, 2, 500, 2048 + 64 + 500), (2, 3, 77, 300 + 77),
+    (1, 2, 33, 1 + 33), (1, 1, 1, 40 + 1), (1, 2, 260, 95 + 260),
+])
+@pytest.mark.parametrize("masking", ["random", "none", "stretches"])
+@pytest.mark.parametrize("layout", ["heads_first", "tokens_first"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_backward_on_the_matrix_cores(Z, H, N_CTX, N_KV, masking, layout, dtype):
+    """head_dim 128 in the 16-bit formats runs the backward on the matrix cores (32-row blocks, 128 stationary rows
+    per workgroup): sizes that are no multiple of either, cached stretches that end inside a block, no cached keys
+    at all, whole blocks of masked keys, and tensors laid out (batch, tokens, heads, dim) as projections leave them."""
+    torch.manual_seed(21)
+    D = 128
+
+    def leaf(n):
+        if layout == "heads_first":
+            t = torch.empty((Z, H, n, D), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5)
+        else:
+            t = torch.empty((Z, n, H, D), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).transpose(1, 2)
+        return t.requires_grad_()
+
+    q, k, v = leaf(N_CTX), leaf(N_KV), leaf(N_KV)
+    n_cached = N_KV - N_CTX
+    if masking == "random":
+        mask = torch.rand(n_cached, device="cuda") > 0.5
+    elif masking == "none":
+        mask = torch.zeros(n_cached, dtype=torch.bool, device="cuda")
+    else:  # whole 32-key blocks hidden, and a stretch that starts and ends inside blocks
+        mask = torch.zeros(n_cached, dtype=torch.bool, device="cuda")
+        mask[: min(96, n_cached)] = True
+        mask[min(130, n_cached): min(171, n_cached)] = True
+    check_backward_against_autograd(q, k, v, mask, dtype)
 
 
 @pytest.mark.parametrize("flavour", ["llama", "qwen2"])
