@@ -240,14 +240,21 @@ __global__ void __launch_bounds__(kThreads, 2) bwd_mfma_dq_kernel(BwdMfmaParams 
                 dp = Mma<T>::mma(row_operand(vt, lane, ds), greg[ds], dp);
                 if ((ds & 3) == 3) __builtin_amdgcn_sched_barrier(0);
             }
+            // A lane is a query: a row past the end spoils only its own accumulators, which are never stored, so
+            // no element tests its row.  A cached block with every key visible tests nothing at all.
             f32x16 dsv;
+            if (vis == 0xffffffffu && !chunk_part) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int r = 8 * (i / 4) + 4 * h + (i % 4);  // key of the block
-                bool ok = ((vis >> r) & 1u) != 0u && row_ok;
-                if (chunk_part) ok = ok && (r < r_cached || r <= r_last);
-                const float pe = ok ? __builtin_amdgcn_exp2f(fmaf(s[i], c2, nlse2)) : 0.f;
-                dsv[i] = pe * (dp[i] - delta) * a.scale;
+                for (int i = 0; i < 16; i++) dsv[i] = __builtin_amdgcn_exp2f(fmaf(s[i], c2, nlse2)) * (dp[i] - delta) * a.scale;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int r = 8 * (i / 4) + 4 * h + (i % 4);  // key of the block
+                    bool ok = ((vis >> r) & 1u) != 0u;
+                    if (chunk_part) ok = ok && (r < r_cached || r <= r_last);
+                    const float pe = ok ? __builtin_amdgcn_exp2f(fmaf(s[i], c2, nlse2)) : 0.f;
+                    dsv[i] = pe * (dp[i] - delta) * a.scale;
+                }
             }
             const uint32_t kt_lds = lds0 + (uint32_t)(st * 2 * kTile);
 #pragma unroll
@@ -380,7 +387,9 @@ __global__ void __launch_bounds__(kThreads, 2) bwd_mfma_dkdv_kernel(BwdMfmaParam
             if (lo64 < 0) lo64 = 0;
             if (lo64 > kBlk) lo64 = kBlk;
             if (hi64 > kBlk) hi64 = kBlk;
-            const int r_lo = key_ok ? (int)lo64 : kBlk, r_hi = (int)hi64;
+            // A lane is a key: a masked or absent key spoils only its own accumulators, which are stored as zeros.
+            const int r_lo = (int)lo64, r_hi = (int)hi64;
+            const bool plain = __ballot(r_lo > 0) == 0ull && r_hi == kBlk;  // every row of the block sees every key
             const uint32_t qt_lds = lds0 + (uint32_t)(st * 2 * kTile), gt_lds = qt_lds + kTile;
             // The phases are fenced so that the compiler keeps their registers apart: P, then dV, then dP and dS, then dK.
             f32x16 pv = zero16();
@@ -396,7 +405,8 @@ __global__ void __launch_bounds__(kThreads, 2) bwd_mfma_dkdv_kernel(BwdMfmaParam
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const int i = 4 * j + e, r = 8 * j + 4 * h + e;
-                    pv[i] = r >= r_lo && r < r_hi ? __builtin_amdgcn_exp2f(fmaf(pv[i], c2, nls[e])) : 0.f;
+                    const float pe = __builtin_amdgcn_exp2f(fmaf(pv[i], c2, nls[e]));
+                    pv[i] = plain || (r >= r_lo && r < r_hi) ? pe : 0.f;
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -440,6 +450,10 @@ __global__ void __launch_bounds__(kThreads, 2) bwd_mfma_dkdv_kernel(BwdMfmaParam
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's copies of the next block have landed
         if (more && tid < 2 * kBlk) rowv[st ^ 1][tid / kBlk][tid & (kBlk - 1)] = tid < kBlk ? -rv_next * kLog2e : rv_next;
         __syncthreads();
+    }
+    if (!key_ok) {
+#pragma unroll
+        for (int db = 0; db < kHD / 32; db++) dk[db] = dv[db] = zero16();
     }
     if (n_lane < n_kv) {
         const int64_t off = (b * a.dkv_stride[0] + hd * a.dkv_stride[1] + n_lane * a.dkv_stride[2]) * 2;
