@@ -135,6 +135,15 @@ __device__ inline uint4 pack8(const f32x16& v, int s) {
                       Mma<T>::pack2(v[8 * s + 4], v[8 * s + 5]), Mma<T>::pack2(v[8 * s + 6], v[8 * s + 7]));
 }
 
+// bits [0, n) set, for 0 <= n <= 32
+__device__ inline uint32_t low_bits(int n) { return n >= 32 ? 0xffffffffu : ((1u << n) - 1u); }
+
+// v if bit `bit` of `word` is set, else +0: a sign-extended one-bit field and a bitwise and
+__device__ inline float keep_if_bit(float v, uint32_t word, int bit) {
+    const int32_t m = (int32_t)(word << (31 - bit)) >> 31;
+    return __uint_as_float(__float_as_uint(v) & (uint32_t)m);
+}
+
 __device__ inline f32x16 zero16() {
     f32x16 z;
 #pragma unroll
@@ -247,12 +256,13 @@ __global__ void __launch_bounds__(kThreads, 2) bwd_mfma_dq_kernel(BwdMfmaParams 
 #pragma unroll
                 for (int i = 0; i < 16; i++) dsv[i] = __builtin_amdgcn_exp2f(fmaf(s[i], c2, nlse2)) * (dp[i] - delta) * a.scale;
             } else {
+                // bit r of `allow`: key r of the block is visible to this lane's query
+                uint32_t allow = vis;
+                if (chunk_part) allow &= low_bits(r_cached) | low_bits(r_last + 1);
+                allow >>= 4 * h;  // element i looks at key 8 (i / 4) + 4 h + i % 4
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    const int r = 8 * (i / 4) + 4 * h + (i % 4);  // key of the block
-                    bool ok = ((vis >> r) & 1u) != 0u;
-                    if (chunk_part) ok = ok && (r < r_cached || r <= r_last);
-                    const float pe = ok ? __builtin_amdgcn_exp2f(fmaf(s[i], c2, nlse2)) : 0.f;
+                    const float pe = keep_if_bit(__builtin_amdgcn_exp2f(fmaf(s[i], c2, nlse2)), allow, 8 * (i / 4) + (i % 4));
                     dsv[i] = pe * (dp[i] - delta) * a.scale;
                 }
             }
@@ -390,6 +400,8 @@ __global__ void __launch_bounds__(kThreads, 2) bwd_mfma_dkdv_kernel(BwdMfmaParam
             // A lane is a key: a masked or absent key spoils only its own accumulators, which are stored as zeros.
             const int r_lo = (int)lo64, r_hi = (int)hi64;
             const bool plain = __ballot(r_lo > 0) == 0ull && r_hi == kBlk;  // every row of the block sees every key
+            // bit r of `allow`: row r of the block sees this lane's key; element i looks at row 8 (i / 4) + 4 h + i % 4
+            const uint32_t allow = (low_bits(r_hi) & ~low_bits(r_lo)) >> (4 * h);
             const uint32_t qt_lds = lds0 + (uint32_t)(st * 2 * kTile), gt_lds = qt_lds + kTile;
             // The phases are fenced so that the compiler keeps their registers apart: P, then dV, then dP and dS, then dK.
             f32x16 pv = zero16();
@@ -403,11 +415,11 @@ __global__ void __launch_bounds__(kThreads, 2) bwd_mfma_dkdv_kernel(BwdMfmaParam
                 const float4 nl = *reinterpret_cast<const float4*>(&rowv[st][0][8 * j + 4 * h]);
                 const float nls[4] = {nl.x, nl.y, nl.z, nl.w};
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int i = 4 * j + e, r = 8 * j + 4 * h + e;
-                    const float pe = __builtin_amdgcn_exp2f(fmaf(pv[i], c2, nls[e]));
-                    pv[i] = plain || (r >= r_lo && r < r_hi) ? pe : 0.f;
-                }
+                for (int e = 0; e < 4; e++) pv[4 * j + e] = __builtin_amdgcn_exp2f(fmaf(pv[4 * j + e], c2, nls[e]));
+            }
+            if (!plain) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) pv[i] = keep_if_bit(pv[i], allow, 8 * (i / 4) + (i % 4));
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -474,7 +486,10 @@ __global__ void __launch_bounds__(kThreads, 2) bwd_mfma_dkdv_kernel(BwdMfmaParam
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
-inline bool rows_ok(const int64_t* st) { return st[3] == 1 && st[2] % 8 == 0 && st[1] % 8 == 0 && st[0] % 8 == 0; }
+// unit stride along the head dim, 16-byte addressable rows, and 32 rows apart still within a 32-bit byte offset
+inline bool rows_ok(const int64_t* st) {
+    return st[3] == 1 && st[2] % 8 == 0 && st[1] % 8 == 0 && st[0] % 8 == 0 && st[2] > 0 && st[2] < (1 << 24);
+}
 
 template <typename T>
 int run(const BwdMfmaParams& p, hipStream_t stream) {
