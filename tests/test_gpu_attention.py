@@ -354,6 +354,46 @@ def dense_reference(q, k, v, mask, sm_scale):
 def test_dense_operator_forward(Z, H, N_CTX, N_KV, HEAD_DIM, dtype):
     """The forward half of cascade/models/test.py:177-269: seed 20, N(0, 0.5) inputs, sm_scale 0.5,
     random cache mask, atol 1e-2 (1e-4 in float32)."""
+    from cascading_kv_cache_amd.flash_attention import attention
+
+    torch.manual_seed(20)
+    q = torch.empty((Z, H, N_CTX, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5)
+    k = torch.empty((Z, H, N_KV, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5)
+    v = torch.empty((Z, H, N_KV, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5)
+    mask = torch.rand(N_KV - N_CTX, device="cuda") > 0.5
+    ref, p = dense_reference(q, k, v, mask, 0.5)
+    out, scores = attention(q, k, v, True, 0.5, mask, 0.9999)
+    atol = 1e-4 if dtype == torch.float32 else 1e-2
+    assert (out.float() - ref).abs().max().item() <= atol
+    # exact version of what cascade/models/test.py:271-318 only rank-correlates
+    w = (1 - 0.9999) * 0.9999 ** torch.arange(N_CTX - 1, -1, -1, device="cuda", dtype=torch.float64)
+    want = (p.double() * w[None, None, :, None]).sum(dim=2)
+    assert_scores_close(scores, want, dtype, "dense scores")
+
+
+def test_attention_rejects_cpu_tensors():
+    from cascading_kv_cache_amd import _abi
+    from cascading_kv_cache_amd.flash_attention import attention
+
+    q = torch.zeros(1, 1, 16, 64)
+    with pytest.raises(_abi.CkvError):
+        attention(q, q, q, True, 1.0, torch.zeros(0, dtype=torch.bool), 0.9)
+
+
+@pytest.mark.parametrize("Z,H,N_CTX,N_KV,HEAD_DIM", [
+    (1, 2, 128, 128, 64), (1, 2, 256, 256, 64), (1, 2, 512, 512, 64), (1, 1, 128, 128 + 128, 64),
+    (1, 2, 1024, 16384 + 1024, 64), (2, 32, 1024, 16384 + 1024, 128), (1, 2, 512, 2560, 64),
+    (1, 2, 500, 2048 + 500, 64), (1, 2, 500, 2048 + 64 + 500, 64), (2, 3, 77, 300 + 77, 32),
+    (1, 3, 90, 200 + 90, 16),   # the smallest head size the operator takes
+])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_dense_operator_backward(Z, H, N_CTX, N_KV, HEAD_DIM, dtype):
+    """The backward half of cascade/models/test.py:177-269: seed 20, N(0, 0.5) inputs, sm_scale 0.5, random cache
+    mask; dq, dk, dv of the operator against autograd through the dense formula (softmax in float32, then the
+    product with v in the tensor dtype), atol 1e-2 in float16 as in the reference's test, 1e-4 in float32, 2e-2 in
+    bfloat16 plus two units in the last place of the value (gradients of a key seen by hundreds of rows reach
+    magnitudes of 4 to 8, where neighbouring bfloat16 values are 3e-2 apart, and the reference formula rounds P
+    and the products to bfloat16 where the kernels round once)."""
     torch.manual_seed(20)
     q = torch.empty((Z, H, N_CTX, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
     k = torch.empty((Z, H, N_KV, HEAD_DIM), dtype=dtype, device="cuda").normal_(mean=0.0, std=0.5).requires_grad_()
