@@ -110,42 +110,114 @@ __global__ void prep_generic_kernel(ckv_attn_args a, T* qr, T* kr, T* vc, uint8_
 }
 
 // ---------------------------------------------------------------------------------------------
-// forward: one wavefront per query row, lanes = keys for the logits, lanes = dims for P.V
+// forward: one wavefront per query row, lanes = keys for the logits, lanes = dims for P.V.  The four rows of a
+// workgroup are consecutive; when they belong to one (batch, kv head) the workgroup stages each chunk of 64 keys
+// in LDS once for all four (K rows 16-byte aligned at a pitch of D + 4 floats, V as is), otherwise every
+// wavefront reads its own rows from memory.  Either way a row sees the same operands in the same order, and
+// every sum is one chain of fused multiply-adds in ascending order of its index, so the result does not depend
+// on the path.  DS > 0: the head size, known at compile time (the query row then lives in registers).
 // ---------------------------------------------------------------------------------------------
 constexpr int kMaxD = 256;
 
+// element e of a 16-byte piece of a row of T, as a float
 template <typename T>
-__global__ void fwd_generic_kernel(CoreProblem p) {
-    __shared__ float q_lds[4][kMaxD];
+__device__ inline float piece_elem(const uint32_t (&w)[4], int e) {
+    if constexpr (sizeof(T) == 4) {
+        return __uint_as_float(w[e]);
+    } else {
+        const uint16_t bits = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+        return Elem<T>::to_float(__builtin_bit_cast(T, bits));
+    }
+}
+
+template <typename T, int DS>
+__global__ void __launch_bounds__(256) fwd_generic_kernel(CoreProblem p) {
+    extern __shared__ __attribute__((aligned(16))) float kv_tile[];  // K [64][D + 4], V [64][D]
+    __shared__ __attribute__((aligned(16))) float q_lds[4][kMaxD];
+    __shared__ __attribute__((aligned(16))) float pe_lds[4][CKV_WAVE];
+    __shared__ int64_t n_end_lds[4];
     const int wave = threadIdx.x / CKV_WAVE, lane = threadIdx.x % CKV_WAVE;
     const int64_t rows = p.B * p.H * p.Q;
-    int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    const int64_t row0 = (int64_t)blockIdx.x * 4;
+    int64_t row = row0 + wave;
     const bool active = row < rows;
     if (!active) row = rows - 1;
     const int64_t m = row % p.Q;
     const int64_t h = (row / p.Q) % p.H;
     const int64_t b = row / (p.Q * p.H);
     const int64_t G = p.H / p.KVH, kvh = h / G;
-    const int64_t D = p.D, N = p.N, Nc = N - p.Q;
+    const int64_t D = DS > 0 ? DS : p.D, N = p.N, Nc = N - p.Q;
     const T* qrow = (const T*)p.q + b * p.q_stride[0] + h * p.q_stride[1] + m * p.q_stride[2];
     for (int64_t d = lane; d < D; d += CKV_WAVE) q_lds[wave][d] = Elem<T>::to_float(qrow[d * p.q_stride[3]]);
+    const int64_t n_end = Nc + m + 1;  // keys past the diagonal are never visible
+    if (lane == 0) n_end_lds[wave] = active ? n_end : 0;
     __syncthreads();
-    if (!active) return;
+    // one (batch, kv head) for the whole workgroup?  Rows are ordered (batch, head, position), so the first and
+    // the last row decide.
+    const int64_t row3 = row0 + 3 < rows ? row0 + 3 : rows - 1;
+    const bool shared_kv = row0 / (p.Q * p.H) == row3 / (p.Q * p.H) &&
+                           ((row0 / p.Q) % p.H) / G == ((row3 / p.Q) % p.H) / G;
+    int64_t n_end_wg = n_end_lds[0];
+    for (int w = 1; w < 4; w++) n_end_wg = n_end_lds[w] > n_end_wg ? n_end_lds[w] : n_end_wg;
     const T* kbase = (const T*)p.k + b * p.kv_stride[0] + kvh * p.kv_stride[1];
     const T* vbase = (const T*)p.v + b * p.kv_stride[0] + kvh * p.kv_stride[1];
+    const int64_t pitch = D + 4;
+    float* k_t = kv_tile;
+    float* v_t = kv_tile + CKV_WAVE * pitch;
+    float qreg[DS > 0 ? DS : 1];
+    if (DS > 0) {
+#pragma unroll
+        for (int d = 0; d < DS; d += 4) {
+            const float4 q4 = *reinterpret_cast<const float4*>(&q_lds[wave][d]);
+            qreg[d] = q4.x;
+            qreg[d + 1] = q4.y;
+            qreg[d + 2] = q4.z;
+            qreg[d + 3] = q4.w;
+        }
+    }
 
     float m_run = -INFINITY, l_run = 0.f;
     float o[kMaxD / CKV_WAVE] = {0.f, 0.f, 0.f, 0.f};
-    const int64_t n_end = Nc + m + 1;  // keys past the diagonal are never visible
-    for (int64_t base = 0; base < n_end; base += CKV_WAVE) {
+    for (int64_t base = 0; base < n_end_wg; base += CKV_WAVE) {
+        if (shared_kv) {
+            __syncthreads();  // the chunk before is no longer read
+            for (int64_t i = threadIdx.x; i < CKV_WAVE * D; i += 256) {
+                const int64_t r = i / D, d = i % D, nn = base + r;
+                float kx = 0.f, vx = 0.f;
+                if (nn < n_end_wg) {
+                    kx = Elem<T>::to_float(kbase[nn * p.kv_stride[2] + d * p.kv_stride[3]]);
+                    vx = Elem<T>::to_float(vbase[nn * p.kv_stride[2] + d * p.kv_stride[3]]);
+                }
+                k_t[r * pitch + d] = kx;
+                v_t[r * D + d] = vx;
+            }
+            __syncthreads();
+        }
+        if (!active || base >= n_end) continue;
         const int64_t n = base + lane;
         bool valid = n < n_end;
         if (valid && n < Nc && p.kmasked) valid = p.kmasked[n] == 0;
         float s = -INFINITY;
         if (valid) {
-            const T* kr = kbase + n * p.kv_stride[2];
             float acc = 0.f;
-            for (int64_t d = 0; d < D; d++) acc = fmaf(q_lds[wave][d], Elem<T>::to_float(kr[d * p.kv_stride[3]]), acc);
+            if (shared_kv) {
+                const float* kr = k_t + lane * pitch;
+                if (DS > 0) {
+#pragma unroll
+                    for (int d = 0; d < DS; d += 4) {
+                        const float4 k4 = *reinterpret_cast<const float4*>(kr + d);
+                        acc = fmaf(qreg[d], k4.x, acc);
+                        acc = fmaf(qreg[d + 1], k4.y, acc);
+                        acc = fmaf(qreg[d + 2], k4.z, acc);
+                        acc = fmaf(qreg[d + 3], k4.w, acc);
+                    }
+                } else {
+                    for (int64_t d = 0; d < D; d++) acc = fmaf(q_lds[wave][d], kr[d], acc);
+                }
+            } else {
+                const T* kr = kbase + n * p.kv_stride[2];
+                for (int64_t d = 0; d < D; d++) acc = fmaf(q_lds[wave][d], Elem<T>::to_float(kr[d * p.kv_stride[3]]), acc);
+            }
             s = acc * p.scale;
         }
         float cmax = s;
@@ -161,17 +233,36 @@ __global__ void fwd_generic_kernel(CoreProblem p) {
 #pragma unroll
         for (int r = 0; r < kMaxD / CKV_WAVE; r++) o[r] *= alpha;
         const int64_t cnt = n_end - base < CKV_WAVE ? n_end - base : CKV_WAVE;
-        for (int j = 0; j < cnt; j++) {
-            const float pj = __shfl(pe, j);
-            if (pj == 0.f) continue;
-            const T* vr = vbase + (base + j) * p.kv_stride[2];
+        // the probabilities of the chunk go through LDS: every lane reads them all, four at a time (the wavefront's
+        // own row of pe_lds: written and read by the same wavefront, in program order)
+        pe_lds[wave][lane] = pe;
+        for (int j4 = 0; j4 < cnt; j4 += 4) {
+            const float4 p4 = *reinterpret_cast<const float4*>(&pe_lds[wave][j4]);
+            const float pj4[4] = {p4.x, p4.y, p4.z, p4.w};
 #pragma unroll
-            for (int r = 0; r < kMaxD / CKV_WAVE; r++) {
-                const int64_t d = lane + r * CKV_WAVE;
-                if (d < D) o[r] = fmaf(pj, Elem<T>::to_float(vr[d * p.kv_stride[3]]), o[r]);
+            for (int e = 0; e < 4; e++) {
+                const int j = j4 + e;
+                const float pj = pj4[e];
+                if (j >= cnt || pj == 0.f) continue;  // a hidden key's V row is never touched (it may hold anything)
+                if (shared_kv) {
+                    const float* vr = v_t + j * D;
+#pragma unroll
+                    for (int r = 0; r < kMaxD / CKV_WAVE; r++) {
+                        const int64_t d = lane + r * CKV_WAVE;
+                        if (d < D) o[r] = fmaf(pj, vr[d], o[r]);
+                    }
+                } else {
+                    const T* vr = vbase + (base + j) * p.kv_stride[2];
+#pragma unroll
+                    for (int r = 0; r < kMaxD / CKV_WAVE; r++) {
+                        const int64_t d = lane + r * CKV_WAVE;
+                        if (d < D) o[r] = fmaf(pj, Elem<T>::to_float(vr[d * p.kv_stride[3]]), o[r]);
+                    }
+                }
             }
         }
     }
+    if (!active) return;
     const float inv = 1.f / l_run;
     T* orow = (T*)p.out + b * p.out_stride[0] + h * p.out_stride[1] + m * p.out_stride[2];
 #pragma unroll
@@ -183,13 +274,15 @@ __global__ void fwd_generic_kernel(CoreProblem p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// score sums: one wavefront per (b, h, 64 keys); lanes = keys, loop over the query rows
+// score sums: one wavefront per (b, h, 64 keys); lanes = keys, loop over the query rows.  DS > 0: the head size,
+// known at compile time: the lane's key row then lives in registers and a logit is one chain of DS fused
+// multiply-adds against query elements every lane reads from the same address.
 // ---------------------------------------------------------------------------------------------
-template <typename T>
-__global__ void colsum_generic_kernel(CoreProblem p) {
+template <typename T, int DS>
+__global__ void __launch_bounds__(CKV_WAVE) colsum_generic_kernel(CoreProblem p) {
     extern __shared__ float k_lds[];  // [64][D + 1]
     const int lane = threadIdx.x;
-    const int64_t D = p.D, N = p.N, Q = p.Q, Nc = N - Q;
+    const int64_t D = DS > 0 ? DS : p.D, N = p.N, Q = p.Q, Nc = N - Q;
     const int64_t chunks = (N + CKV_WAVE - 1) / CKV_WAVE;
     const int64_t c = blockIdx.x % chunks;
     const int64_t h = (blockIdx.x / chunks) % p.H;
@@ -204,6 +297,11 @@ __global__ void colsum_generic_kernel(CoreProblem p) {
         k_lds[r * pitch + d] = nn < N ? Elem<T>::to_float(kbase[nn * p.kv_stride[2] + d * p.kv_stride[3]]) : 0.f;
     }
     __syncthreads();
+    float kreg[DS > 0 ? DS : 1];
+    if (DS > 0) {
+#pragma unroll
+        for (int d = 0; d < DS; d++) kreg[d] = k_lds[lane * pitch + d];
+    }
     bool live = n < N;
     if (live && n < Nc && p.kmasked) live = p.kmasked[n] == 0;
     const int64_t nrel = n - Nc;  // >= 0 for chunk keys
@@ -212,11 +310,32 @@ __global__ void colsum_generic_kernel(CoreProblem p) {
     if (m0 < 0) m0 = 0;
     const T* qbase = (const T*)p.q + b * p.q_stride[0] + h * p.q_stride[1];
     const float* lse = p.lse + (b * p.H + h) * Q;
+    // rows of 16-byte pieces: unit stride along the head dim, every row 16-byte aligned
+    const bool q_contig = p.q_stride[3] == 1 && (reinterpret_cast<uintptr_t>(p.q) & 15) == 0 &&
+                          (p.q_stride[0] * sizeof(T)) % 16 == 0 && (p.q_stride[1] * sizeof(T)) % 16 == 0 &&
+                          (p.q_stride[2] * sizeof(T)) % 16 == 0;
     float acc = 0.f;
     for (int64_t m = m0; m < Q; m++) {
         const T* qr = qbase + m * p.q_stride[2];
         float s = 0.f;
-        for (int64_t d = 0; d < D; d++) s = fmaf(Elem<T>::to_float(qr[d * p.q_stride[3]]), k_lds[lane * pitch + d], s);
+        if (DS > 0 && q_contig) {
+            // the row is one run of memory at an address every lane shares: wide scalar loads
+            const uint4* q16 = reinterpret_cast<const uint4*>(qr);
+#pragma unroll
+            for (int d = 0; d < DS; d += 16 / (int)sizeof(T)) {
+                const uint4 w = q16[d / (16 / (int)sizeof(T))];
+                const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                for (int e = 0; e < 16 / (int)sizeof(T); e++) {
+                    s = fmaf(piece_elem<T>(ws, e), kreg[d + e], s);
+                }
+            }
+        } else if (DS > 0) {
+#pragma unroll
+            for (int d = 0; d < DS; d++) s = fmaf(Elem<T>::to_float(qr[d * p.q_stride[3]]), kreg[d], s);
+        } else {
+            for (int64_t d = 0; d < D; d++) s = fmaf(Elem<T>::to_float(qr[d * p.q_stride[3]]), k_lds[lane * pitch + d], s);
+        }
         const bool vis = live && (n < Nc || nrel <= m);
         if (vis) {
             // the eager path holds P in the tensor dtype (softmax output) before weighting it;
@@ -299,26 +418,36 @@ __global__ void cast_scores_kernel(const float* colsum, T* scores, int64_t s0, i
     scores[b * s0 + h * s1 + n * s2] = Elem<T>::from_float(colsum[idx]);
 }
 
-template <typename T>
-int core_generic_t(const CoreProblem& p, hipStream_t stream) {
+template <typename T, int DS>
+int core_generic_d(const CoreProblem& p, hipStream_t stream) {
     const int64_t rows = p.B * p.H * p.Q;
     {
+        const size_t lds_f = (size_t)CKV_WAVE * (2 * p.D + 4) * sizeof(float);
+        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fwd_generic_kernel<T, DS>), (int)lds_f)) return rc;
         StageScope sc(CKV_STAGE_FWD, stream);
-        hipLaunchKernelGGL(fwd_generic_kernel<T>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((fwd_generic_kernel<T, DS>), dim3((unsigned)((rows + 3) / 4)), dim3(256), lds_f, stream, p);
     }
     CKV_HIP_TRY(hipGetLastError());
     if (p.colsum) {
         const int64_t chunks = (p.N + CKV_WAVE - 1) / CKV_WAVE;
         const size_t lds = (size_t)CKV_WAVE * (p.D + 1) * sizeof(float);
-        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(colsum_generic_kernel<T>), (int)lds)) return rc;
+        if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(colsum_generic_kernel<T, DS>), (int)lds)) return rc;
         {
             StageScope sc(CKV_STAGE_SCORES, stream);
-            hipLaunchKernelGGL(colsum_generic_kernel<T>, dim3((unsigned)(p.B * p.H * chunks)), dim3(CKV_WAVE), lds,
+            hipLaunchKernelGGL((colsum_generic_kernel<T, DS>), dim3((unsigned)(p.B * p.H * chunks)), dim3(CKV_WAVE), lds,
                                stream, p);
         }
         CKV_HIP_TRY(hipGetLastError());
     }
     return CKV_OK;
+}
+
+// the two head sizes models use get kernels with the size built in; every other size the general ones
+template <typename T>
+int core_generic_t(const CoreProblem& p, hipStream_t stream) {
+    if (p.D == 128) return core_generic_d<T, 128>(p, stream);
+    if (p.D == 64) return core_generic_d<T, 64>(p, stream);
+    return core_generic_d<T, 0>(p, stream);
 }
 
 }  // namespace
