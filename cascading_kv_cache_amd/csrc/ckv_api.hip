@@ -12,7 +12,8 @@ struct Span {
     int stage;
     hipEvent_t t0, t1;
 };
-int g_prof_level = 0;  // 0 off, 1 every stage, 2 attention main kernels only
+int g_prof_level = 0;  // 0 off, 1 every stage, 2 attention main kernels only, 3 update kernels only, 4 = 2 sampled
+int64_t g_sample_count[CKV_STAGE_COUNT] = {};
 std::vector<Span> g_spans;
 hipEvent_t g_open[CKV_STAGE_COUNT];
 std::mutex g_prof_mutex;  // guards g_spans and g_open: calls on several host threads may time stages at once
@@ -56,10 +57,11 @@ int ensure_dynamic_lds(const void* func, int bytes) {
     return CKV_OK;
 }
 
-// level 2: the attention main kernels; level 3: the kernels of the cache update.  Both time single kernels by
-// events attached to their dispatch.
+// level 2: the attention main kernels; level 3: the kernels of the cache update; level 4: the attention main
+// kernels, every fourth launch of each.  All time single kernels by events attached to their dispatch.
+constexpr int kSamplePeriod = 4;
 static bool dispatch_timed(int stage) {
-    return (g_prof_level == 2 && (stage == CKV_STAGE_FWD || stage == CKV_STAGE_DECODE)) ||
+    return ((g_prof_level == 2 || g_prof_level == 4) && (stage == CKV_STAGE_FWD || stage == CKV_STAGE_DECODE)) ||
            (g_prof_level == 3 && (stage == CKV_STAGE_PLAN || stage == CKV_STAGE_APPLY));
 }
 
@@ -70,6 +72,10 @@ bool prof_kernel_events_wanted(int stage) { return dispatch_timed(stage); }
 void prof_kernel_events(int stage, hipEvent_t* start, hipEvent_t* stop) {
     *start = *stop = nullptr;
     if (!prof_kernel_events_wanted(stage)) return;
+    if (g_prof_level == 4) {  // the first launch of a stage after the level was set, then every kSamplePeriod-th
+        std::lock_guard<std::mutex> lock(g_prof_mutex);
+        if (g_sample_count[stage]++ % kSamplePeriod != 0) return;
+    }
     hipEvent_t e0, e1;
     if (hipEventCreate(&e0) != hipSuccess) return;
     if (hipEventCreate(&e1) != hipSuccess) {
@@ -106,7 +112,11 @@ void prof_end(int stage, hipStream_t stream) {
 
 extern "C" int ckv_profile_enable(int on) {
     const int prev = ckv::g_prof_level;
-    ckv::g_prof_level = on < 0 || on > 3 ? 1 : on;
+    ckv::g_prof_level = on < 0 || on > 4 ? 1 : on;
+    {
+        std::lock_guard<std::mutex> lock(ckv::g_prof_mutex);
+        for (int i = 0; i < CKV_STAGE_COUNT; i++) ckv::g_sample_count[i] = 0;
+    }
     return prev;
 }
 

@@ -314,8 +314,10 @@ typedef enum ckv_stage {
 } ckv_stage;
 
 /* on: 0 = off, 1 = every stage bracketed by event records in the stream, 2 = only the attention main kernels
- * (CKV_STAGE_FWD, CKV_STAGE_DECODE), 3 = only the kernels of the cache update (CKV_STAGE_PLAN, CKV_STAGE_APPLY).
- * Levels 2 and 3 attach the events to the kernels' own dispatches: nothing is put between a kernel and its
+ * (CKV_STAGE_FWD, CKV_STAGE_DECODE), 3 = only the kernels of the cache update (CKV_STAGE_PLAN, CKV_STAGE_APPLY),
+ * 4 = as 2, but only the first and then every fourth launch of each of the two kernels is timed (a timed dispatch
+ * still costs a few microseconds around the kernel; `launches` counts the timed ones).
+ * Levels 2 to 4 attach the events to the kernels' own dispatches: nothing is put between a kernel and its
  * neighbours, and the figures are kernel durations, fit for timing inside a throughput measurement. */
 int ckv_profile_enable(int on);                       /* returns the previous setting */
 int ckv_profile_read(double* ms, int64_t* launches);  /* both arrays CKV_STAGE_COUNT long */

@@ -43,6 +43,16 @@ def test_main_kernels_only():
             assert n == 0 and ms == 0.0, name
 
 
+def test_main_kernels_sampled():
+    """Level 4: as level 2, but the first and then every fourth launch of each of the two kernels."""
+    st = _run(4, steps_prefill=5, steps_decode=9)
+    assert st["fwd"][1] == 2 and st["decode"][1] == 3   # launches 0 and 4 of 5; 0, 4 and 8 of 9
+    assert 0.0 < st["fwd"][0] < 100.0 and 0.0 < st["decode"][0] < 100.0
+    for name, (ms, n) in st.items():
+        if name not in ("fwd", "decode"):
+            assert n == 0 and ms == 0.0, name
+
+
 def test_every_stage():
     st = _run(1)
     assert st["fwd"][1] == 3 and st["scores"][1] == 3 and st["finish"][1] == 3
