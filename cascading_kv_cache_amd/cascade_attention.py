@@ -213,7 +213,8 @@ def cascade_attention(query_states, key_states, value_states, cache: CascadingKV
         a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
         _abi.check(lib.ckv_attn(C.byref(a), C.c_void_p(stream)), "ckv_attn")
         if update_cache:
-            cache.update_state(key_states, value_states, L, score_states=new_scores, _stream=stream)
+            cache.update_state(key_states, value_states, L, score_states=new_scores, _stream=stream,
+                               _device_counter=replayable)
     return out, new_scores
 
 
@@ -264,6 +265,7 @@ class DecodeStepGraph:
             self.q.copy_(q)
             self.k.copy_(k)
             self.v.copy_(v)
+        cache._flush_counter()  # the recorded update reads and advances the device counter itself
         if self._generation != cache._generation:  # first use, or the cache was reset / reallocated since
             self._generation = cache._generation
             self.graph, self._warm = None, False

@@ -17,6 +17,21 @@ from . import _abi
 _WORKSPACES = {}
 
 
+_COUNTER_TABLES = {}
+COUNTER_TABLE_ENTRIES = 1 << 21
+
+
+def _counter_table(device) -> Tensor:
+    """``0, 1, 2, ...`` as int64 on ``device`` (16 MiB, built once): element n is a device-resident n."""
+    device = torch.device(device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    t = _COUNTER_TABLES.get(key)
+    if t is None:
+        t = torch.arange(COUNTER_TABLE_ENTRIES, dtype=torch.long, device=device)
+        _COUNTER_TABLES[key] = t
+    return t
+
+
 def workspace(device: torch.device, nbytes: int, stream: int = 0) -> Tensor:
     """Scratch for one library call: one buffer per (device, stream), grown on demand.  Calls on one
     stream run in order, so they can share a buffer; calls on different streams of a device may
@@ -198,7 +213,8 @@ class CascadingKVCache:
         self._seen_tokens = 0
         self._generation += 1   # a step recorded into a graph before the reset no longer describes this cache
         self._seen_host = [0 for _ in range(self.layers)]
-        self.seen_tokens_by_layer.zero_()
+        self._seen_pending = [0 for _ in range(self.layers)]
+        self._seen_dev.zero_()
         for group in (self.stored_tokens, self.stored_sinks, self.start_indices, self.pos, self.sink_pos,
                       self.key_cache, self.value_cache, self.score_cache, self.sink_keys, self.sink_values,
                       self.og_pos):
@@ -219,6 +235,7 @@ class CascadingKVCache:
         self._update_memo, self._attn_memo = {}, {}  # argument blocks described once per input layout
         # host mirror of seen_tokens_by_layer: lets callers branch without a device sync
         self._seen_host = [0] * n_layers
+        self._seen_pending = [0] * n_layers   # tokens the device counter has not been told about yet
         self.beta = 0.9999999  # cascading_cache.py:1247
 
         def per_layer(fill, dtype, *tail):
@@ -228,7 +245,7 @@ class CascadingKVCache:
 
         slots = lambda l: self.max_seq_len[l]    # noqa: E731
         levels = lambda l: self.cascades[l]      # noqa: E731
-        self.seen_tokens_by_layer = torch.zeros(n_layers, dtype=torch.long, device=device)
+        self._seen_dev = torch.zeros(n_layers, dtype=torch.long, device=device)
         self.do_cache = [torch.ones(self.cascades[l], device=device, dtype=torch.bool) for l in range(n_layers)]
         self.do_cache_every_n = [
             torch.tensor(acceptance_periods(self.cascade_func, self.cascades[l]), device=device, dtype=torch.long)
@@ -247,6 +264,24 @@ class CascadingKVCache:
         self.sink_values = per_layer(0, self.dtype, sinks, self.dim)
         self.mask = per_layer(True, torch.bool, slots)
         self.sink_mask = per_layer(True, torch.bool, sinks)
+
+    @property
+    def seen_tokens_by_layer(self) -> Tensor:
+        """Tokens seen per layer, on the device (cascading_cache.py:1231); current whenever it is looked at."""
+        self._flush_counter()
+        return self._seen_dev
+
+    @seen_tokens_by_layer.setter
+    def seen_tokens_by_layer(self, value: Tensor):
+        self._seen_pending = [0] * self.layers
+        self._seen_dev = value
+
+    def _flush_counter(self):
+        """Tells the device counter about the updates that went by the constant table."""
+        for l, n in enumerate(self._seen_pending):
+            if n:
+                self._seen_dev[l] += n
+                self._seen_pending[l] = 0
 
     def sync_host_counter(self) -> List[int]:
         """Re-reads the host mirror of ``seen_tokens_by_layer`` from the device (one read-back).
@@ -295,7 +330,7 @@ class CascadingKVCache:
         handed out again.)"""
         ts = (self.key_cache[L], self.value_cache[L], self.score_cache[L], self.sink_keys[L], self.sink_values[L],
               self.mask[L], self.sink_mask[L], self.pos[L], self.og_pos[L], self.sink_pos[L], self.stored_tokens[L],
-              self.start_indices[L], self.stored_sinks[L], self.do_cache_every_n[L], self.seen_tokens_by_layer)
+              self.start_indices[L], self.stored_sinks[L], self.do_cache_every_n[L], self._seen_dev)
         return tuple(t.data_ptr() for t in ts) + (self.score_cache[L].stride(), self.score_cache[L].dtype)
 
     def update(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None):
@@ -318,8 +353,9 @@ class CascadingKVCache:
                 self.key_cache[L], self.value_cache[L], self.score_cache[L],
                 self.mask[L], self.pos[L], self.og_pos[L], self.do_cache_every_n[L],
                 self.stored_tokens[L], self.start_indices[L], self.stored_sinks[L],
-                self.num_sink_tokens, self.window_length[L], self.seen_tokens_by_layer[L], self.max_seq_len[L],
+                self.num_sink_tokens, self.window_length[L], self._seen_dev[L], self.max_seq_len[L],
                 self.eager_fill)
+            a._counter = a.real_token_idx   # the layer's element of the device counter
             a._need = _abi.lib().ckv_update_workspace_bytes(a.N, a.H, a.K, a.max_seq_len, a.cascades)
             if len(memo) > 64:
                 memo.clear()
@@ -329,14 +365,20 @@ class CascadingKVCache:
         return a
 
     def update_state(self, key_states: Tensor, value_states: Tensor, layer_idx: int, score_states: Tensor = None,
-                     _stream: Optional[int] = None):
+                     _stream: Optional[int] = None, _device_counter: bool = False):
         """``update`` without building the tuple of views it returns (the shifted position row of
         ``get_vals`` is a device operation of its own); for callers that read the state in place.
 
         The argument block of ``ckv_update`` is described once per layer and input layout and reused:
         between two calls of the same shape only the three input pointers change (single-token steps
         at batch 1 are bound by this host code, not by the device).  ``_stream``: raw stream handle when
-        the caller already holds the device context."""
+        the caller already holds the device context.
+
+        The update reads the number of tokens seen so far from device memory (``real_token_idx``).  The host knows
+        that number, so the call points the library at the element of a constant table ``0, 1, 2, ...`` that holds
+        it and leaves the device counter ``seen_tokens_by_layer`` to be brought up to date when somebody looks at
+        it: a step then carries no launch for the counter.  ``_device_counter``: read and advance the device counter
+        itself, as the reference does (cascading_cache.py:1343-1346): what a step recorded into a graph needs."""
         _require_device(key_states, "k")
         if score_states is None:
             score_states = torch.zeros(self.max_batch_size, self.heads, key_states.size(2),
@@ -345,6 +387,14 @@ class CascadingKVCache:
             self._seen_tokens += key_states.shape[-2]
 
         a = self._update_args(key_states, value_states, score_states, layer_idx)
+        n_new = key_states.shape[-2]
+        table = None if _device_counter else _counter_table(key_states.device)
+        if table is not None and self._seen_host[layer_idx] < table.numel():
+            a.real_token_idx = table.data_ptr() + 8 * self._seen_host[layer_idx]
+        else:
+            table = None
+            self._flush_counter()
+            a.real_token_idx = a._counter
         if _stream is None:
             with torch.cuda.device(key_states.device):
                 stream = torch.cuda.current_stream(key_states.device).cuda_stream
@@ -356,5 +406,8 @@ class CascadingKVCache:
             a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
             _abi.check(_abi.lib().ckv_update(C.byref(a), C.c_void_p(_stream)), "ckv_update")
         # after the kernel, as in the reference (cascading_cache.py:1343-1346)
-        self.seen_tokens_by_layer[layer_idx] += key_states.shape[-2]
-        self._seen_host[layer_idx] += key_states.shape[-2]
+        if table is None:
+            self._seen_dev[layer_idx] += n_new
+        else:
+            self._seen_pending[layer_idx] += n_new
+        self._seen_host[layer_idx] += n_new
