@@ -166,3 +166,42 @@ def test_reference_preconditions_and_errors():
         c.update(torch.zeros(1, 1, 2, 8, device="cuda:0", dtype=torch.float16),
                  torch.zeros(1, 1, 2, 8, device="cuda:0", dtype=torch.float16), 0,
                  torch.zeros(1, 1, 2, device="cuda:0", dtype=torch.float16))
+
+
+def test_token_counter_by_table_and_by_device_counter():
+    """An update reads the tokens seen so far from a constant table the host indexes, and the device counter
+    ``seen_tokens_by_layer`` is brought up to date when it is read; past the end of the table (made tiny here) the
+    update reads and advances the device counter itself.  Either way the original token indices (og_pos) and every
+    other state tensor equal the oracle's."""
+    from cascading_kv_cache_amd import cascading_cache as cc
+
+    dtype = torch.float32
+    gpu, cpu = make_pair(2, 2, 16, 2, 8, 2, dtype)
+    gen = torch.Generator().manual_seed(5)
+
+    def feed(q):
+        k = torch.randn(2, 2, q, 16, generator=gen)
+        v = torch.randn(2, 2, q, 16, generator=gen)
+        s = (torch.rand(2, 2, q, generator=gen) * 1e-6)
+        gpu.update_state(k.cuda(), v.cuda(), 0, s.cuda())
+        cpu.update(k, v, s)
+
+    for q in (3, 1, 5, 1, 1):          # nobody looks at the device counter in between
+        feed(q)
+    assert gpu._seen_pending == [11] and int(gpu._seen_dev[0]) == 0
+    assert int(gpu.seen_tokens_by_layer[0]) == 11 and gpu._seen_pending == [0]
+    assert_same_state(gpu, cpu, "by the table")
+
+    key = ("cuda", 0)
+    full = cc._COUNTER_TABLES[key]
+    try:
+        cc._COUNTER_TABLES[key] = full[:13]        # tokens 11 and 12 still come from the table, later ones do not
+        for q in (1, 1, 4, 1, 7):
+            feed(q)
+        assert gpu._seen_pending == [0] and int(gpu._seen_dev[0]) == 25
+        assert_same_state(gpu, cpu, "by the device counter")
+    finally:
+        cc._COUNTER_TABLES[key] = full
+    feed(2)
+    assert gpu._seen_pending == [2]
+    assert_same_state(gpu, cpu, "back on the table")
