@@ -274,6 +274,147 @@ __global__ void __launch_bounds__(256) fwd_generic_kernel(CoreProblem p) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// forward, several rows per wavefront: the same arithmetic as fwd_generic_kernel, row by row, for head sizes known
+// at compile time and chunks whose length is a multiple of the 4 x R rows of a workgroup (so that a workgroup never
+// straddles two heads).  A staged chunk of 64 keys then serves 4 x R rows, and a K or V element read from LDS
+// serves R of them: the one-row kernel is bound by what its workgroups re-read through the L2.
+// ---------------------------------------------------------------------------------------------
+template <typename T, int DS, int R>
+__global__ void __launch_bounds__(256) fwd_generic_rows_kernel(CoreProblem p) {
+    extern __shared__ __attribute__((aligned(16))) float kv_tile[];  // K [64][DS + 4], V [64][DS]
+    __shared__ __attribute__((aligned(16))) float q_lds[4 * R][DS];
+    __shared__ __attribute__((aligned(16))) float pe_lds[4][R][CKV_WAVE];
+    const int wave = threadIdx.x / CKV_WAVE, lane = threadIdx.x % CKV_WAVE;
+    const int64_t row0 = (int64_t)blockIdx.x * (4 * R);   // all rows exist and share (b, h): Q % (4 R) == 0
+    const int64_t m0 = row0 % p.Q;
+    const int64_t h = (row0 / p.Q) % p.H;
+    const int64_t b = row0 / (p.Q * p.H);
+    const int64_t G = p.H / p.KVH, kvh = h / G;
+    const int64_t N = p.N, Nc = N - p.Q;
+    constexpr int pitch = DS + 4;
+    {
+        const T* qrows = (const T*)p.q + b * p.q_stride[0] + h * p.q_stride[1];
+        for (int i = threadIdx.x; i < 4 * R * DS; i += 256) {
+            const int r = i / DS, d = i % DS;
+            q_lds[r][d] = Elem<T>::to_float(qrows[(m0 + r) * p.q_stride[2] + d * p.q_stride[3]]);
+        }
+    }
+    const T* kbase = (const T*)p.k + b * p.kv_stride[0] + kvh * p.kv_stride[1];
+    const T* vbase = (const T*)p.v + b * p.kv_stride[0] + kvh * p.kv_stride[1];
+    float* k_t = kv_tile;
+    float* v_t = kv_tile + CKV_WAVE * pitch;
+    const int64_t n_end_wg = Nc + m0 + 4 * R;  // what the last row of the workgroup sees
+    float m_run[R], l_run[R], o[R][DS / CKV_WAVE];
+#pragma unroll
+    for (int i = 0; i < R; i++) {
+        m_run[i] = -INFINITY;
+        l_run[i] = 0.f;
+#pragma unroll
+        for (int r = 0; r < DS / CKV_WAVE; r++) o[i][r] = 0.f;
+    }
+    for (int64_t base = 0; base < n_end_wg; base += CKV_WAVE) {
+        __syncthreads();  // the chunk before is no longer read (the first time: the queries are in place)
+        for (int i = threadIdx.x; i < CKV_WAVE * DS; i += 256) {
+            const int r = i / DS, d = i % DS;
+            const int64_t nn = base + r;
+            float kx = 0.f, vx = 0.f;
+            if (nn < n_end_wg) {
+                kx = Elem<T>::to_float(kbase[nn * p.kv_stride[2] + d * p.kv_stride[3]]);
+                vx = Elem<T>::to_float(vbase[nn * p.kv_stride[2] + d * p.kv_stride[3]]);
+            }
+            k_t[r * pitch + d] = kx;
+            v_t[r * DS + d] = vx;
+        }
+        __syncthreads();
+        const int64_t n = base + lane;
+        const bool key_ok = !(n < Nc && p.kmasked && p.kmasked[n < Nc ? n : 0] != 0);
+        // logits of this lane's key for the R rows: one pass over the key row, R chains
+        float acc[R];
+#pragma unroll
+        for (int i = 0; i < R; i++) acc[i] = 0.f;
+        const float* kr = k_t + lane * pitch;
+#pragma unroll 8
+        for (int d = 0; d < DS; d += 4) {
+            const float4 k4 = *reinterpret_cast<const float4*>(kr + d);
+#pragma unroll
+            for (int i = 0; i < R; i++) {
+                const float4 q4 = *reinterpret_cast<const float4*>(&q_lds[wave * R + i][d]);
+                acc[i] = fmaf(q4.x, k4.x, acc[i]);
+                acc[i] = fmaf(q4.y, k4.y, acc[i]);
+                acc[i] = fmaf(q4.z, k4.z, acc[i]);
+                acc[i] = fmaf(q4.w, k4.w, acc[i]);
+            }
+        }
+        int cnt[R];
+        bool upd[R];
+#pragma unroll
+        for (int i = 0; i < R; i++) {
+            const int64_t n_end = Nc + m0 + wave * R + i + 1;
+            cnt[i] = 0;
+            upd[i] = false;
+            if (base >= n_end) continue;
+            const bool valid = n < n_end && key_ok;
+            const float s = valid ? acc[i] * p.scale : -INFINITY;
+            float cmax = s;
+            for (int off = 32; off > 0; off >>= 1) cmax = fmaxf(cmax, __shfl_xor(cmax, off));
+            if (cmax == -INFINITY) continue;  // nothing visible in this chunk
+            const float m_new = fmaxf(m_run[i], cmax);
+            const float pe = valid ? expf(s - m_new) : 0.f;
+            float csum = pe;
+            for (int off = 32; off > 0; off >>= 1) csum += __shfl_xor(csum, off);
+            const float alpha = m_run[i] == -INFINITY ? 0.f : expf(m_run[i] - m_new);
+            l_run[i] = l_run[i] * alpha + csum;
+            m_run[i] = m_new;
+#pragma unroll
+            for (int r = 0; r < DS / CKV_WAVE; r++) o[i][r] *= alpha;
+            cnt[i] = n_end - base < CKV_WAVE ? (int)(n_end - base) : CKV_WAVE;
+            upd[i] = true;
+            pe_lds[wave][i][lane] = pe;
+        }
+        int cnt_max = 0;
+#pragma unroll
+        for (int i = 0; i < R; i++) cnt_max = cnt[i] > cnt_max ? cnt[i] : cnt_max;
+        // P.V: a V element read once serves the R rows; per row the keys are added in ascending order, a key with
+        // probability 0 (hidden, or past the row's diagonal) is not touched
+        for (int j4 = 0; j4 < cnt_max; j4 += 4) {
+            float pj[R][4];
+#pragma unroll
+            for (int i = 0; i < R; i++) {
+                float4 p4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (upd[i]) p4 = *reinterpret_cast<const float4*>(&pe_lds[wave][i][j4]);
+                pj[i][0] = p4.x;
+                pj[i][1] = p4.y;
+                pj[i][2] = p4.z;
+                pj[i][3] = p4.w;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int j = j4 + e;
+                const float* vr = v_t + j * DS;
+                float vv[DS / CKV_WAVE];
+#pragma unroll
+                for (int r = 0; r < DS / CKV_WAVE; r++) vv[r] = vr[lane + r * CKV_WAVE];
+#pragma unroll
+                for (int i = 0; i < R; i++) {
+                    if (j >= cnt[i] || pj[i][e] == 0.f) continue;
+#pragma unroll
+                    for (int r = 0; r < DS / CKV_WAVE; r++) o[i][r] = fmaf(pj[i][e], vv[r], o[i][r]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < R; i++) {
+        const int64_t m = m0 + wave * R + i;
+        const float inv = 1.f / l_run[i];
+        T* orow = (T*)p.out + b * p.out_stride[0] + h * p.out_stride[1] + m * p.out_stride[2];
+#pragma unroll
+        for (int r = 0; r < DS / CKV_WAVE; r++) orow[(lane + r * CKV_WAVE) * p.out_stride[3]] = Elem<T>::from_float(o[i][r] * inv);
+        if (lane == 0 && p.lse) p.lse[row0 + wave * R + i] = m_run[i] + logf(l_run[i]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // score sums: one wavefront per (b, h, 64 keys); lanes = keys, loop over the query rows.  DS > 0: the head size,
 // known at compile time: the lane's key row then lives in registers and a logit is one chain of DS fused
 // multiply-adds against query elements every lane reads from the same address.
@@ -423,10 +564,23 @@ int core_generic_d(const CoreProblem& p, hipStream_t stream) {
     const int64_t rows = p.B * p.H * p.Q;
     {
         const size_t lds_f = (size_t)CKV_WAVE * (2 * p.D + 4) * sizeof(float);
+        constexpr int kRowsPerWave = 4;
+        if constexpr (DS > 0) {
+            if (p.Q % (4 * kRowsPerWave) == 0) {
+                const void* fn = reinterpret_cast<const void*>(fwd_generic_rows_kernel<T, DS, kRowsPerWave>);
+                if (int rc = ensure_dynamic_lds(fn, (int)lds_f)) return rc;
+                StageScope sc(CKV_STAGE_FWD, stream);
+                hipLaunchKernelGGL((fwd_generic_rows_kernel<T, DS, kRowsPerWave>), dim3((unsigned)(rows / (4 * kRowsPerWave))),
+                                   dim3(256), lds_f, stream, p);
+                CKV_HIP_TRY(hipGetLastError());
+                goto scores;
+            }
+        }
         if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(fwd_generic_kernel<T, DS>), (int)lds_f)) return rc;
         StageScope sc(CKV_STAGE_FWD, stream);
         hipLaunchKernelGGL((fwd_generic_kernel<T, DS>), dim3((unsigned)((rows + 3) / 4)), dim3(256), lds_f, stream, p);
     }
+scores:
     CKV_HIP_TRY(hipGetLastError());
     if (p.colsum) {
         const int64_t chunks = (p.N + CKV_WAVE - 1) / CKV_WAVE;
