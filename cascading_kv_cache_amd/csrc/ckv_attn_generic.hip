@@ -416,12 +416,13 @@ __global__ void __launch_bounds__(256) fwd_generic_rows_kernel(CoreProblem p) {
 
 // ---------------------------------------------------------------------------------------------
 // score sums: one wavefront per (b, h, 64 keys); lanes = keys, loop over the query rows.  DS > 0: the head size,
-// known at compile time: the lane's key row then lives in registers and a logit is one chain of DS fused
-// multiply-adds against query elements every lane reads from the same address.
+// known at compile time: the query rows then pass through LDS and four of them share each read of the key row.
 // ---------------------------------------------------------------------------------------------
+constexpr int kColQTile = 32;  // query rows per LDS tile of the score kernel (a multiple of 4)
+
 template <typename T, int DS>
 __global__ void __launch_bounds__(CKV_WAVE) colsum_generic_kernel(CoreProblem p) {
-    extern __shared__ float k_lds[];  // [64][D + 1]
+    extern __shared__ __attribute__((aligned(16))) float k_lds[];  // K [64][D + 1]; with DS > 0: K [64][DS + 4], Q [kColQTile][DS]
     const int lane = threadIdx.x;
     const int64_t D = DS > 0 ? DS : p.D, N = p.N, Q = p.Q, Nc = N - Q;
     const int64_t chunks = (N + CKV_WAVE - 1) / CKV_WAVE;
@@ -431,18 +432,13 @@ __global__ void __launch_bounds__(CKV_WAVE) colsum_generic_kernel(CoreProblem p)
     const int64_t G = p.H / p.KVH, kvh = h / G;
     const int64_t n = c * CKV_WAVE + lane;
     const T* kbase = (const T*)p.k + b * p.kv_stride[0] + kvh * p.kv_stride[1];
-    const int64_t pitch = D + 1;
+    const int64_t pitch = DS > 0 ? D + 4 : D + 1;  // rows of 16-byte pieces when the head size is built in
     for (int64_t i = lane; i < CKV_WAVE * D; i += CKV_WAVE) {
         const int64_t r = i / D, d = i % D;
         const int64_t nn = c * CKV_WAVE + r;
         k_lds[r * pitch + d] = nn < N ? Elem<T>::to_float(kbase[nn * p.kv_stride[2] + d * p.kv_stride[3]]) : 0.f;
     }
     __syncthreads();
-    float kreg[DS > 0 ? DS : 1];
-    if (DS > 0) {
-#pragma unroll
-        for (int d = 0; d < DS; d++) kreg[d] = k_lds[lane * pitch + d];
-    }
     bool live = n < N;
     if (live && n < Nc && p.kmasked) live = p.kmasked[n] == 0;
     const int64_t nrel = n - Nc;  // >= 0 for chunk keys
@@ -451,32 +447,9 @@ __global__ void __launch_bounds__(CKV_WAVE) colsum_generic_kernel(CoreProblem p)
     if (m0 < 0) m0 = 0;
     const T* qbase = (const T*)p.q + b * p.q_stride[0] + h * p.q_stride[1];
     const float* lse = p.lse + (b * p.H + h) * Q;
-    // rows of 16-byte pieces: unit stride along the head dim, every row 16-byte aligned
-    const bool q_contig = p.q_stride[3] == 1 && (reinterpret_cast<uintptr_t>(p.q) & 15) == 0 &&
-                          (p.q_stride[0] * sizeof(T)) % 16 == 0 && (p.q_stride[1] * sizeof(T)) % 16 == 0 &&
-                          (p.q_stride[2] * sizeof(T)) % 16 == 0;
     float acc = 0.f;
-    for (int64_t m = m0; m < Q; m++) {
-        const T* qr = qbase + m * p.q_stride[2];
-        float s = 0.f;
-        if (DS > 0 && q_contig) {
-            // the row is one run of memory at an address every lane shares: wide scalar loads
-            const uint4* q16 = reinterpret_cast<const uint4*>(qr);
-#pragma unroll
-            for (int d = 0; d < DS; d += 16 / (int)sizeof(T)) {
-                const uint4 w = q16[d / (16 / (int)sizeof(T))];
-                const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-                for (int e = 0; e < 16 / (int)sizeof(T); e++) {
-                    s = fmaf(piece_elem<T>(ws, e), kreg[d + e], s);
-                }
-            }
-        } else if (DS > 0) {
-#pragma unroll
-            for (int d = 0; d < DS; d++) s = fmaf(Elem<T>::to_float(qr[d * p.q_stride[3]]), kreg[d], s);
-        } else {
-            for (int64_t d = 0; d < D; d++) s = fmaf(Elem<T>::to_float(qr[d * p.q_stride[3]]), k_lds[lane * pitch + d], s);
-        }
+    // what one visible (row, key) pair adds, rows in ascending order
+    auto add_row = [&](int64_t m, float s) {
         const bool vis = live && (n < Nc || nrel <= m);
         if (vis) {
             // the eager path holds P in the tensor dtype (softmax output) before weighting it;
@@ -487,6 +460,48 @@ __global__ void __launch_bounds__(CKV_WAVE) colsum_generic_kernel(CoreProblem p)
             } else {
                 acc = fmaf(p.w_ema[m], pt, acc);
             }
+        }
+    };
+    if constexpr (DS > 0) {
+        // Query rows pass through LDS in tiles of kColQTile; the logits of four rows are worked out together (four
+        // independent chains over the head dims, each in ascending order; a piece of the lane's key row read from
+        // LDS serves all four), then the rows are added in order.
+        float* q_t = k_lds + CKV_WAVE * (DS + 4);   // [kColQTile][DS]
+        const float* krow = k_lds + lane * (DS + 4);
+        for (int64_t mt = m0; mt < Q; mt += kColQTile) {
+            __syncthreads();  // the tile before is no longer read
+#pragma unroll 8
+            for (int i = lane; i < kColQTile * DS; i += CKV_WAVE) {
+                const int r = i / DS, d = i % DS;
+                q_t[i] = mt + r < Q ? Elem<T>::to_float(qbase[(mt + r) * p.q_stride[2] + d * p.q_stride[3]]) : 0.f;
+            }
+            __syncthreads();
+            const int rows_here = Q - mt < kColQTile ? (int)(Q - mt) : kColQTile;
+            for (int mi = 0; mi < rows_here; mi += 4) {
+                float s4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+                for (int d = 0; d < DS; d += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(krow + d);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const float4 q4 = *reinterpret_cast<const float4*>(q_t + (mi + i) * DS + d);
+                        s4[i] = fmaf(q4.x, k4.x, s4[i]);
+                        s4[i] = fmaf(q4.y, k4.y, s4[i]);
+                        s4[i] = fmaf(q4.z, k4.z, s4[i]);
+                        s4[i] = fmaf(q4.w, k4.w, s4[i]);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (mi + i < rows_here) add_row(mt + mi + i, s4[i]);
+            }
+        }
+    } else {
+        for (int64_t m = m0; m < Q; m++) {
+            const T* qr = qbase + m * p.q_stride[2];
+            float s = 0.f;
+            for (int64_t d = 0; d < D; d++) s = fmaf(Elem<T>::to_float(qr[d * p.q_stride[3]]), k_lds[lane * pitch + d], s);
+            add_row(m, s);
         }
     }
     if (n < N) p.colsum[(b * p.H + h) * N + n] = acc;
@@ -584,7 +599,9 @@ scores:
     CKV_HIP_TRY(hipGetLastError());
     if (p.colsum) {
         const int64_t chunks = (p.N + CKV_WAVE - 1) / CKV_WAVE;
-        const size_t lds = (size_t)CKV_WAVE * (p.D + 1) * sizeof(float);
+        // K tile (padded to a multiple of 16 bytes so that the query tile behind it is aligned), then the query tile
+        const size_t lds = DS > 0 ? ((size_t)CKV_WAVE * (DS + 4) + (size_t)kColQTile * DS) * sizeof(float)
+                                  : (size_t)CKV_WAVE * (p.D + 1) * sizeof(float);
         if (int rc = ensure_dynamic_lds(reinterpret_cast<const void*>(colsum_generic_kernel<T, DS>), (int)lds)) return rc;
         {
             StageScope sc(CKV_STAGE_SCORES, stream);
